@@ -1,0 +1,200 @@
+/*
+ * souffle_hip.h -- C ABI of libsouffle_hip.so: the MI355X (gfx950) implementation of
+ * the fused-encoder hot path of summerspringwei/souffle-models.
+ *
+ * Conventions
+ *   - every entry point returns 0 on success or a negative souffle_status; the text
+ *     of the last failure on the calling thread is at souffle_last_error();
+ *   - no entry point aborts, prints, synchronises the device or allocates device
+ *     memory: all buffers (inputs, outputs, workspace) are caller-owned device
+ *     pointers, 16-byte aligned, and the work is queued on the given HIP stream
+ *     (souffle_stream_t is a hipStream_t; NULL = the default stream);
+ *   - a workspace must be zeroed once with souffle_workspace_init() before its
+ *     first use (it holds grid-barrier state); it may then be reused by any number
+ *     of calls, one at a time.  Calls that share a workspace must not overlap;
+ *   - weights are fp16 matrices stored [K][N] with N contiguous, Y = X.W
+ *     (reference: cpp/bert/kernels/gemm_three_stages.h:95-131,
+ *      cpp/bert/test_souffle_bert_layer.py:139-143); activations are fp16 row-major.
+ *
+ * Each declaration cites the reference interface it replaces.
+ */
+#ifndef SOUFFLE_HIP_H
+#define SOUFFLE_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *souffle_stream_t;
+
+enum souffle_status {
+  SOUFFLE_OK = 0,
+  SOUFFLE_ERR_NULL = -1,        /* a required pointer is NULL */
+  SOUFFLE_ERR_SHAPE = -2,       /* unsupported shape / configuration */
+  SOUFFLE_ERR_ALIGN = -3,       /* a pointer is not 16-byte aligned */
+  SOUFFLE_ERR_WORKSPACE = -4,   /* workspace missing or too small */
+  SOUFFLE_ERR_DEVICE = -5,      /* no usable gfx950 device / query failed */
+  SOUFFLE_ERR_LAUNCH = -6,      /* the HIP launch was rejected (text has the HIP error) */
+  SOUFFLE_ERR_UNSUPPORTED = -7
+};
+
+/* Replaces checkCuda's print+assert (cpp/souffle_utils/cuda_utils.h:10-19). */
+const char *souffle_last_error(void);
+const char *souffle_version(void);
+
+/* Replaces check_compatability (cpp/souffle_utils/cuda_utils.h:86-98): the device
+ * facts the launch geometry and the roofline are derived from. */
+typedef struct {
+  int num_cus, lds_bytes_per_cu, clock_khz, mem_clock_khz, mem_bus_bits, l2_bytes;
+  int cooperative_launch, wavefront_size;
+  char arch[64];
+} souffle_devinfo;
+int souffle_device_info(souffle_devinfo *out);
+
+/* Zero the control block at the head of a workspace (stream-ordered, no allocation).
+ * The reference instead zero-allocates its scratch on every call
+ * (cpp/bert/bert_binding.cu:32-78). */
+int souffle_workspace_init(void *workspace, size_t workspace_bytes, souffle_stream_t stream);
+
+/* ------------------------------------------------------------------ BERT ---- */
+enum { SOUFFLE_ACT_GELU_TANH = 0, SOUFFLE_ACT_RELU = 1 };
+
+typedef struct {
+  int batch, seq_len;          /* runtime; batch*seq_len must be a multiple of 128, seq_len of 64, seq_len <= 512 */
+  int hidden, heads, ffn;      /* 768, 12, 3072 (the reference's compile-time family, cpp/bert/kernels/bert.h:8-16) */
+  int act;                     /* SOUFFLE_ACT_*; reference fused path uses ReLU, its unfused path tanh-GELU */
+  float scale;                 /* multiplies q.k (0.125 = 1/sqrt(64)) */
+  float ln_eps;
+  int num_layers;              /* used by the encoder entry points */
+  int reserved;
+} souffle_bert_cfg;
+
+/* fp16 device pointers; every bias and LN vector may be NULL (0 / gamma 1 / beta 0).
+ * Roles as in cpp/bert/bert_binding.cu:25-29 (weights) and cpp/bert/bert_base_impl.cu:151-189 (biases, LN). */
+typedef struct {
+  const void *w_qkv;  /* [3][768][768] */
+  const void *b_qkv;  /* [3][768]      */
+  const void *w_o;    /* [768][768]    */
+  const void *b_o;    /* [768]         */
+  const void *ln1_g, *ln1_b;
+  const void *w_fc1;  /* [768][3072]   */
+  const void *b_fc1;  /* [3072]        */
+  const void *w_fc2;  /* [3072][768]   */
+  const void *b_fc2;  /* [768]         */
+  const void *ln2_g, *ln2_b;
+} souffle_bert_layer_w;
+
+/* Optional fp16 device outputs for the per-stage tensors the reference binding returns
+ * (cpp/bert/bert_binding.cu:534); any member (or the struct pointer) may be NULL. */
+typedef struct {
+  void *qkv;    /* [3][B][12][S][64]  output_qkv              */
+  void *probs;  /* [B][12][S][S]      query_key_output        */
+  void *ctx;    /* [B*S][768]         attn_value_output       */
+  void *ln1;    /* [B*S][768]         attn_fc_output (post-LN)*/
+  void *fc1;    /* [B*S][3072]        feed_forward_fc1_output */
+} souffle_bert_dump;
+
+size_t souffle_bert_workspace_bytes(const souffle_bert_cfg *cfg);
+
+/* One encoder layer as ONE persistent cooperative launch.
+ * Replaces souffle_bert_layer<1,12,384,64,3072>(..., opt_level=3|4)
+ * (cpp/bert/bert_binding.cu:23-535, fused path :395-528).
+ * x,y: [B*S][768] fp16; mask: additive fp16 [B][S][S] or NULL. */
+int souffle_bert_layer_fused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *w,
+                             const void *x, const void *mask, void *y,
+                             const souffle_bert_dump *dump,
+                             void *workspace, size_t workspace_bytes, souffle_stream_t stream);
+/* The same layer as separate per-op launches: the unfused HIP baseline.
+ * Replaces opt_level 1|2 of the same binding (cpp/bert/bert_binding.cu:119-393)
+ * and the per-op chain of Bert::Solve (cpp/bert/bert_base_impl.cu:590-678). */
+int souffle_bert_layer_unfused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *w,
+                               const void *x, const void *mask, void *y,
+                               const souffle_bert_dump *dump,
+                               void *workspace, size_t workspace_bytes, souffle_stream_t stream);
+/* cfg->num_layers layers with distinct weights in one cooperative launch /
+ * as per-op launches.  Replaces souffle_bert_base() (cpp/bert/bert_base_impl.cu:277-308,590-678). */
+int souffle_bert_encoder_fused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
+                               const void *x, const void *mask, void *y,
+                               void *workspace, size_t workspace_bytes, souffle_stream_t stream);
+int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
+                                 const void *x, const void *mask, void *y,
+                                 void *workspace, size_t workspace_bytes, souffle_stream_t stream);
+
+/* ------------------------------------------------------------------ LSTM ---- */
+enum { SOUFFLE_GATES_IFGO = 0, SOUFFLE_GATES_IGFO = 1 };
+typedef struct {
+  int layers, hidden, timesteps, batch;  /* 10, 256, <=4096, 1 */
+  int gate_order;                        /* slot meaning of the four gate matrices */
+  float forget_bias;                     /* reference kernel: 1.0 (cpp/lstm/lstm_reuse_shared_memory.cu:314) */
+} souffle_lstm_cfg;
+size_t souffle_lstm_workspace_bytes(const souffle_lstm_cfg *cfg);
+/* Replaces fused_lstm<1,10,256,100> (cpp/lstm/lstm_binding.cu:30-78).
+ * w_ih, w_hh: fp16 [layers*4][hidden out][hidden in]; bias: fp32 [layers][4][hidden] or NULL;
+ * x: fp32 [T][hidden]; y: fp32 [T][hidden] (top-layer h per step). */
+int souffle_lstm_fused(const souffle_lstm_cfg *cfg, const void *w_ih, const void *w_hh,
+                       const float *bias, const float *x, float *y,
+                       void *workspace, size_t workspace_bytes, souffle_stream_t stream);
+
+/* ------------------------------------------------------------------ Swin ---- */
+typedef struct {
+  int height, width, channels, heads, window, shift, mlp_ratio;  /* 56,56,128,4,7,3,4 */
+  int use_shift_mask;
+  float ln_eps;
+} souffle_swin_cfg;
+typedef struct {   /* fp16 device pointers, biases / LN vectors nullable */
+  const void *ln1_g, *ln1_b;
+  const void *w_qkv, *b_qkv;    /* [C][3C], [3C]  columns (q|k|v) x head x hd */
+  const void *rel_table;        /* [(2w-1)^2][heads] or NULL */
+  const void *w_proj, *b_proj;  /* [C][C], [C] */
+  const void *ln2_g, *ln2_b;
+  const void *w_fc1, *b_fc1;    /* [C][rC] */
+  const void *w_fc2, *b_fc2;    /* [rC][C] */
+} souffle_swin_block_w;
+size_t souffle_swin_workspace_bytes(const souffle_swin_cfg *cfg);
+/* Regular + shifted window block in one cooperative launch.  The op list is
+ * python/models/swin_transformer/swin_transformer_main.py:11-61 (Part-1..8), which the
+ * reference only runs as separate TVM kernels (:196-330).  x,y: fp16 [H*W][C]. */
+int souffle_swin_block_pair_fused(const souffle_swin_cfg *cfg, const souffle_swin_block_w w[2],
+                                  const void *x, void *y,
+                                  void *workspace, size_t workspace_bytes, souffle_stream_t stream);
+/* Host-side index maps (bit-exact contract).  Replaces the te index expressions of
+ * python/models/swin_transformer/swin_self_attention.py:66-82,101-120,179-204,226-265.
+ * gather_idx[w*N+n] = token; scatter_idx[token] = w*N+n; relpos_idx[p*N+q] = table row;
+ * region_id[w*N+n] = shifted-window region label.  Any output may be NULL. */
+int souffle_swin_index_maps(int height, int width, int window, int shift,
+                            int32_t *gather_idx, int32_t *scatter_idx,
+                            int32_t *relpos_idx, int32_t *region_id);
+/* Y1 = X.W1 ; Y2 = Y1.W2, no bias / activation.
+ * Replaces swin_fused_feed_mlp<1,256,512,2048> (cpp/swin_transformer/swin_transformer_binding.cu:154-209). */
+int souffle_swin_ffn_fused(const void *x, const void *w1, const void *w2, void *y1, void *y2,
+                           int M, int K, int F, void *workspace, size_t workspace_bytes,
+                           souffle_stream_t stream);
+/* Y = X.W.  Replaces swin_ffn (cpp/swin_transformer/swin_transformer_binding.cu:62-100) and
+ * swin_trans_fc2 (cpp/swin_transformer/swin_trans_fc2_binding.cu:19-61). */
+int souffle_gemm_f16(const void *x, const void *w, void *y, int M, int N, int K,
+                     souffle_stream_t stream);
+
+/* ----------------------------------------------------- EfficientNet SE ---- */
+enum { SOUFFLE_SE_MUL = 0, SOUFFLE_SE_ADD = 1 };
+size_t souffle_se_workspace_bytes(int C, int HW, int R);
+/* Replaces torch_dispatch_efficientnet_se_module_v2_short_cut_fused
+ * (cpp/efficientnet/efficientnet_se_module_binding.cu:164-227).
+ * x,y: fp32 [C][H*W] (NCHW, batch 1); w_reduce fp32 [R][C]; w_expand fp32 [C][R];
+ * biases nullable; pooled: fp32 [C] out (nullable). */
+int souffle_se_module_fused(const float *x, const float *w_reduce, const float *b_reduce,
+                            const float *w_expand, const float *b_expand,
+                            float *y, float *pooled, int C, int HW, int R, int combine,
+                            void *workspace, size_t workspace_bytes, souffle_stream_t stream);
+
+/* ------------------------------------------------------------- timing ---- */
+/* Replaces benchmarkCudaFunc (cpp/souffle_utils/cuda_utils.h:102-136): after `warmup`
+ * launches, min over `rounds` of the mean of `repeat` event-timed launches, in us.
+ * `fn(arg)` must queue exactly one unit of work on `stream`. */
+int souffle_bench_us(int (*fn)(void *), void *arg, souffle_stream_t stream,
+                     int warmup, int rounds, int repeat, double *min_of_means_us,
+                     double *median_us);
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,157 @@
+// Entry points that are not tied to one model family: error text, device facts,
+// workspace initialisation, the event-timing helper and the plain GEMM.
+#include <algorithm>
+#include <cstring>
+#include <mutex>
+#include <type_traits>
+#include <vector>
+#include "gemm_tile.hpp"
+#include "host_util.hpp"
+
+namespace souffle {
+
+char *error_buffer() {
+  static thread_local char buf[512] = "";
+  return buf;
+}
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int device_facts(DeviceFacts *out) {
+  static std::mutex mu;
+  static DeviceFacts cached[16] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return fail(SOUFFLE_ERR_DEVICE, "no HIP device is available"); }
+  if (dev < 0 || dev >= 16) return fail(SOUFFLE_ERR_DEVICE, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lk(mu);
+  if (!cached[dev].ok) {
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, dev) != hipSuccess) { (void)hipGetLastError(); return fail(SOUFFLE_ERR_DEVICE, "hipGetDeviceProperties failed"); }
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
+      return fail(SOUFFLE_ERR_DEVICE, "built for gfx950 only, device is %s", p.gcnArchName);
+    cached[dev].num_cus = p.multiProcessorCount;
+    cached[dev].lds_per_cu = (int)p.maxSharedMemoryPerMultiProcessor;
+    cached[dev].cooperative = p.cooperativeLaunch;
+    strncpy(cached[dev].arch, p.gcnArchName, 63);
+    cached[dev].ok = 1;
+  }
+  *out = cached[dev];
+  return SOUFFLE_OK;
+}
+
+__global__ void k_zero_words(unsigned *p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+// Plain Y = X.W (fp16 in/out, fp32 accumulate): one tile per workgroup.
+template <class Tile>
+__global__ void __launch_bounds__(256) k_gemm(const half_t *X, const half_t *W, half_t *Y, int M, int N, int K) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int tiles_n = N / Tile::kBN, items = (M / Tile::kBM) * tiles_n;
+  for (int item = blockIdx.x; item < items; item += gridDim.x) {
+    const int tm = item / tiles_n, n0 = (item % tiles_n) * Tile::kBN;
+    auto aload = [&](int m, int k) { return *reinterpret_cast<const u4 *>(X + (size_t)m * K + k); };
+    auto epi = [&](int m, int n, f4 v) { *reinterpret_cast<u2 *>(Y + (size_t)m * N + n) = pack_h4(v); };
+    Tile::run(reinterpret_cast<half_t *>(lds_raw), W, N, tm * Tile::kBM, n0, 0, K / Tile::kBK, aload, epi);
+  }
+}
+
+template <class Tile>
+int launch_gemm(const half_t *x, const half_t *w, half_t *y, int M, int N, int K, int num_cus, hipStream_t st) {
+  static bool attr_done = false;
+  if (!attr_done) {
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm<Tile>, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES));
+    attr_done = true;
+  }
+  const int items = (M / Tile::kBM) * (N / Tile::kBN);
+  hipLaunchKernelGGL(k_gemm<Tile>, dim3(std::min(items, num_cus * 4)), dim3(256), Tile::LDS_BYTES, st, x, w, y, M, N, K);
+  SOUFFLE_HIP_TRY(hipGetLastError());
+  return SOUFFLE_OK;
+}
+
+}  // namespace souffle
+
+using namespace souffle;
+
+extern "C" const char *souffle_last_error(void) { return error_buffer(); }
+extern "C" const char *souffle_version(void) { return "souffle_hip 0.1 (gfx950)"; }
+
+extern "C" int souffle_device_info(souffle_devinfo *out) {
+  if (!out) return fail(SOUFFLE_ERR_NULL, "out is NULL");
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return fail(SOUFFLE_ERR_DEVICE, "no HIP device is available"); }
+  hipDeviceProp_t p;
+  if (hipGetDeviceProperties(&p, dev) != hipSuccess) { (void)hipGetLastError(); return fail(SOUFFLE_ERR_DEVICE, "hipGetDeviceProperties failed"); }
+  memset(out, 0, sizeof(*out));
+  out->num_cus = p.multiProcessorCount;
+  out->lds_bytes_per_cu = (int)p.maxSharedMemoryPerMultiProcessor;
+  out->clock_khz = p.clockRate;
+  out->mem_clock_khz = p.memoryClockRate;
+  out->mem_bus_bits = p.memoryBusWidth;
+  out->l2_bytes = p.l2CacheSize;
+  out->cooperative_launch = p.cooperativeLaunch;
+  out->wavefront_size = p.warpSize;
+  strncpy(out->arch, p.gcnArchName, sizeof(out->arch) - 1);
+  return SOUFFLE_OK;
+}
+
+extern "C" int souffle_workspace_init(void *ws, size_t bytes, souffle_stream_t stream) {
+  if (!ws) return fail(SOUFFLE_ERR_WORKSPACE, "workspace is NULL");
+  if (!aligned16(ws)) return fail(SOUFFLE_ERR_ALIGN, "workspace must be 16-byte aligned");
+  if (bytes < (size_t)kCtlWords * 4) return fail(SOUFFLE_ERR_WORKSPACE, "workspace smaller than its %d-byte control block", kCtlWords * 4);
+  // A fill kernel rather than a memset node, so that callers may capture this call.
+  hipLaunchKernelGGL(k_zero_words, dim3((kCtlWords + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<unsigned *>(ws), kCtlWords);
+  SOUFFLE_HIP_TRY(hipGetLastError());
+  return SOUFFLE_OK;
+}
+
+extern "C" int souffle_gemm_f16(const void *x, const void *w, void *y, int M, int N, int K, souffle_stream_t stream) {
+  if (!x || !w || !y) return fail(SOUFFLE_ERR_NULL, "x, w and y must not be NULL");
+  if (!aligned16(x) || !aligned16(w) || !aligned16(y)) return fail(SOUFFLE_ERR_ALIGN, "x, w and y must be 16-byte aligned");
+  if (M <= 0 || N <= 0 || K <= 0 || M % 64 || N % 64 || K % 64)
+    return fail(SOUFFLE_ERR_SHAPE, "M, N and K must be positive multiples of 64 (got %d,%d,%d)", M, N, K);
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool large = M % 128 == 0 && N % 128 == 0 && (long long)(M / 128) * (N / 128) >= df.num_cus;
+  if (large) return launch_gemm<GemmTile<128, 128, 64, 2, 2>>((const half_t *)x, (const half_t *)w, (half_t *)y, M, N, K, df.num_cus, st);
+  return launch_gemm<GemmTile<64, 64, 64, 2, 2>>((const half_t *)x, (const half_t *)w, (half_t *)y, M, N, K, df.num_cus, st);
+}
+
+// Timing rule of the reference's benchmarkCudaFunc (cpp/souffle_utils/cuda_utils.h:102-136):
+// warm up, then the minimum over rounds of the mean of `repeat` event-timed launches.
+extern "C" int souffle_bench_us(int (*fn)(void *), void *arg, souffle_stream_t stream, int warmup, int rounds,
+                                int repeat, double *min_of_means_us, double *median_us) {
+  if (!fn) return fail(SOUFFLE_ERR_NULL, "fn is NULL");
+  if (rounds <= 0 || repeat <= 0 || warmup < 0) return fail(SOUFFLE_ERR_SHAPE, "rounds and repeat must be positive");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipEvent_t e0, e1;
+  SOUFFLE_HIP_TRY(hipEventCreate(&e0));
+  SOUFFLE_HIP_TRY(hipEventCreate(&e1));
+  int rc = SOUFFLE_OK;
+  for (int i = 0; i < warmup && rc == SOUFFLE_OK; ++i) rc = fn(arg);
+  std::vector<double> means;
+  for (int r = 0; r < rounds && rc == SOUFFLE_OK; ++r) {
+    if (hipEventRecord(e0, st) != hipSuccess) { rc = fail(SOUFFLE_ERR_LAUNCH, "hipEventRecord failed"); break; }
+    for (int i = 0; i < repeat && rc == SOUFFLE_OK; ++i) rc = fn(arg);
+    if (rc != SOUFFLE_OK) break;
+    if (hipEventRecord(e1, st) != hipSuccess || hipEventSynchronize(e1) != hipSuccess) { rc = fail(SOUFFLE_ERR_LAUNCH, "event record/sync failed: %s", hipGetErrorString(hipGetLastError())); break; }
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess) { rc = fail(SOUFFLE_ERR_LAUNCH, "hipEventElapsedTime failed"); break; }
+    means.push_back((double)ms * 1000.0 / repeat);
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc != SOUFFLE_OK) return rc;
+  std::sort(means.begin(), means.end());
+  if (min_of_means_us) *min_of_means_us = means.front();
+  if (median_us) *median_us = means[means.size() / 2];
+  return SOUFFLE_OK;
+}

@@ -1,0 +1,506 @@
+// BERT-base encoder layer(s) on gfx950: a persistent cooperative megakernel (all stages
+// of all layers in one launch, grid barriers between stages) and the same stages as
+// separate launches (the unfused per-op baseline).
+//
+// Stage list per layer (reference counterparts in brackets):
+//   1 QKV GEMM + bias + head split        [cpp/bert/kernels/fused_sqq_bert.cu:2333-2765]
+//   2 scores, scale, mask, softmax, P.V   [fused_sqq_bert.cu:2772-3329]  (P never leaves the CU)
+//   3 out-projection, split-K partials    [fused_sqq_bert.cu:3334-3687]
+//   4 reduce + bias + residual + LN1      [fused_sqq_bert.cu:3690-3782]
+//   5 FC1 + bias + activation             [cpp/bert/kernels/fused_sqq_feedforward.cu:38-362]
+//   6 FC2, split-K partials               [fused_sqq_feedforward.cu:368-835]
+//   7 reduce + bias + residual + LN2      [fused_sqq_feedforward.cu:368-835]
+// Softmax is max-subtracted fp32 and LayerNorm is two-pass fp32 in registers, with a
+// fixed summation order (no float atomics), so results are run-to-run identical.
+#include <type_traits>
+#include "gemm_tile.hpp"
+#include "host_util.hpp"
+
+namespace souffle {
+namespace bert {
+
+constexpr int H = 768, NH = 12, HD = 64, F = 3072;
+constexpr int kMaxLayers = 24;
+constexpr int kMaxSplitK = 8;
+
+struct LayerW {
+  const half_t *w_qkv, *b_qkv, *w_o, *b_o, *ln1_g, *ln1_b, *w_fc1, *b_fc1, *w_fc2, *b_fc2, *ln2_g, *ln2_b;
+};
+
+struct Args {
+  int B, S, M, act, num_layers, splitk_o, splitk_f;
+  float scale, eps;
+  const half_t *x, *mask;
+  half_t *y;
+  half_t *qkv, *ctx, *y1, *h, *xa, *xb, *probs;
+  float *part;
+  unsigned *ctl;
+  LayerW layers[kMaxLayers];
+};
+
+// ------------------------------------------------------------------ stages ----
+template <bool COH, class Tile>
+__device__ __forceinline__ void stage_qkv(half_t *lds, const Args &a, const LayerW &w, const half_t *xin,
+                                          int first, int stride) {
+  constexpr int BM = Tile::kBM, BN = Tile::kBN, BK = Tile::kBK;
+  const int tiles_n = 3 * H / BN, items = (a.M / BM) * tiles_n;
+  for (int item = first; item < items; item += stride) {
+    const int tm = item / tiles_n, n0 = (item % tiles_n) * BN, j = n0 / H, nn0 = n0 % H;
+    auto aload = [&](int m, int k) { return ld16<COH>(xin, (m * H + k) * 2); };
+    auto epi = [&](int m, int n, f4 v) {
+      if (w.b_qkv) {
+        const h4 bb = *reinterpret_cast<const h4 *>(w.b_qkv + j * H + n);
+        v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+      }
+      const int b = m / a.S, s = m % a.S, hh = n / HD, d = n % HD;
+      st8<COH>(a.qkv, ((((j * a.B + b) * NH + hh) * a.S + s) * HD + d) * 2, pack_h4(v));
+    };
+    Tile::run(lds, w.w_qkv + (size_t)j * H * H, H, tm * BM, nn0, 0, H / BK, aload, epi);
+  }
+}
+
+// Y = act(X.W + b), fp16 out (FC1).
+template <bool COH, class Tile>
+__device__ __forceinline__ void stage_fc1(half_t *lds, const Args &a, const LayerW &w, int first, int stride) {
+  constexpr int BM = Tile::kBM, BN = Tile::kBN, BK = Tile::kBK;
+  const int tiles_n = F / BN, items = (a.M / BM) * tiles_n;
+  for (int item = first; item < items; item += stride) {
+    const int tm = item / tiles_n, n0 = (item % tiles_n) * BN;
+    auto aload = [&](int m, int k) { return ld16<COH>(a.y1, (m * H + k) * 2); };
+    auto epi = [&](int m, int n, f4 v) {
+      if (w.b_fc1) {
+        const h4 bb = *reinterpret_cast<const h4 *>(w.b_fc1 + n);
+        v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(v[i], 0.f) : gelu_tanh(v[i]);
+      st8<COH>(a.h, (m * F + n) * 2, pack_h4(v));
+    };
+    Tile::run(lds, w.w_fc1, F, tm * BM, n0, 0, H / BK, aload, epi);
+  }
+}
+
+// fp32 split-K partials of X[M][K].W[K][H]: part[ks][m][n].
+template <bool COH, class Tile>
+__device__ __forceinline__ void stage_partial(half_t *lds, const Args &a, const half_t *X, int K,
+                                              const half_t *W, int splitk, int first, int stride) {
+  constexpr int BM = Tile::kBM, BN = Tile::kBN, BK = Tile::kBK;
+  const int tiles_n = H / BN, items = (a.M / BM) * tiles_n * splitk, kper = K / splitk;
+  for (int item = first; item < items; item += stride) {
+    const int ks = item % splitk, t = item / splitk, tm = t / tiles_n, n0 = (t % tiles_n) * BN;
+    auto aload = [&](int m, int k) { return ld16<COH>(X, (m * K + k) * 2); };
+    auto epi = [&](int m, int n, f4 v) {
+      st16<COH>(a.part, ((ks * a.M + m) * H + n) * 4, __builtin_bit_cast(u4, v));
+    };
+    Tile::run(lds, W, H, tm * BM, n0, ks * kper, kper / BK, aload, epi);
+  }
+}
+
+// out[m] = LN(sum_ks part[ks][m] + bias + resid[m]) * g + b; one wave per row.
+template <bool COH>
+__device__ __forceinline__ void stage_ln(const Args &a, int splitk, const half_t *bias, const half_t *resid,
+                                         const half_t *gam, const half_t *bet, half_t *out,
+                                         int first_row, int row_stride) {
+  const int lane = threadIdx.x & 63;
+  for (int m = first_row; m < a.M; m += row_stride) {
+    f4 v[3];
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      const int n = c * 256 + lane * 4;
+      f4 s = __builtin_bit_cast(f4, ld16<COH>(a.part, (m * H + n) * 4));
+      for (int ks = 1; ks < splitk; ++ks) s += __builtin_bit_cast(f4, ld16<COH>(a.part, ((ks * a.M + m) * H + n) * 4));
+      const h4 r = as_h4(ld8<COH>(resid, (m * H + n) * 2));
+      s += f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+      if (bias) {
+        const h4 bb = *reinterpret_cast<const h4 *>(bias + n);
+        s += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+      }
+      v[c] = s;
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) sum += v[c][0] + v[c][1] + v[c][2] + v[c][3];
+    const float mean = wave_sum(sum) * (1.0f / H);
+    float sq = 0.f;
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { const float d = v[c][i] - mean; sq += d * d; }
+    const float rstd = rsqrtf(wave_sum(sq) * (1.0f / H) + a.eps);
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      const int n = c * 256 + lane * 4;
+      f4 o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = (v[c][i] - mean) * rstd;
+      if (gam) {
+        const h4 gg = *reinterpret_cast<const h4 *>(gam + n);
+        o *= f4{(float)gg[0], (float)gg[1], (float)gg[2], (float)gg[3]};
+      }
+      if (bet) {
+        const h4 bb = *reinterpret_cast<const h4 *>(bet + n);
+        o += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+      }
+      st8<COH>(out, (m * H + n) * 2, pack_h4(o));
+    }
+  }
+}
+
+// One (batch, head, 64-query block) per workgroup pass; each wave owns 16 queries.
+// Scores are computed transposed (keys x queries) so that the softmax reduction over
+// keys is in-lane plus two cross-lane steps, and the probabilities are already in the
+// B-operand layout of the 16x16x16 MFMA used for P.V.  V is staged row-major in LDS
+// and read through the transposing LDS load.
+constexpr int kVLD = HD + 8;
+template <bool COH, int NKT>
+__device__ __forceinline__ void attn_item(half_t *lds, const Args &a, int item) {
+  constexpr int S = NKT * 16;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+  const int qblocks = S / 64;
+  const int qb = item % qblocks, bh = item / qblocks, b = bh / NH, hh = bh % NH;
+  const int head_off = ((b * NH + hh) * S) * HD;                 // halves, within one of q/k/v
+  const int plane = a.B * NH * S * HD;
+  const half_t *Q = a.qkv, *K = a.qkv + plane, *V = a.qkv + 2 * (size_t)plane;
+
+  __syncthreads();   // LDS reuse
+  for (int id = tid; id < S * HD / 8; id += 256) {
+    const int r = id / (HD / 8), c = (id % (HD / 8)) * 8;
+    *reinterpret_cast<u4 *>(lds + r * kVLD + c) = ld16<COH>(V, (head_off + r * HD + c) * 2);
+  }
+  const int q0 = qb * 64 + wave * 16;
+  h8 qop[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) qop[ks] = as_h8(ld16<COH>(Q, (head_off + (q0 + l16) * HD + ks * 32 + g * 8) * 2));
+
+  f4 sc[NKT];
+#pragma unroll
+  for (int t = 0; t < NKT; ++t) {
+    const h8 k0 = as_h8(ld16<COH>(K, (head_off + (t * 16 + l16) * HD + g * 8) * 2));
+    const h8 k1 = as_h8(ld16<COH>(K, (head_off + (t * 16 + l16) * HD + 32 + g * 8) * 2));
+    f4 c = mfma_16x16x32(k0, qop[0], f4{0.f, 0.f, 0.f, 0.f});
+    sc[t] = mfma_16x16x32(k1, qop[1], c);
+  }
+  // sc[t][v] = score(key = 16t + 4g + v, query = q0 + l16)
+  const int q = q0 + l16;
+  float mx = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < NKT; ++t) {
+    f4 s = sc[t] * a.scale;
+    if (a.mask) {
+      const h4 mk = *reinterpret_cast<const h4 *>(a.mask + ((size_t)b * S + q) * S + t * 16 + g * 4);
+      s += f4{(float)mk[0], (float)mk[1], (float)mk[2], (float)mk[3]};
+    }
+    sc[t] = s;
+    mx = fmaxf(mx, fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+  }
+  mx = fmaxf(mx, wave_xor(mx, 16));
+  mx = fmaxf(mx, wave_xor(mx, 32));
+  float sum = 0.f;
+#pragma unroll
+  for (int t = 0; t < NKT; ++t) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { sc[t][i] = __expf(sc[t][i] - mx); sum += sc[t][i]; }
+  }
+  sum += wave_xor(sum, 16);
+  sum += wave_xor(sum, 32);
+  const float inv = 1.0f / sum;
+  h4 p[NKT];
+#pragma unroll
+  for (int t = 0; t < NKT; ++t) {
+    const f4 pr = sc[t] * inv;
+    p[t] = h4{(half_t)pr[0], (half_t)pr[1], (half_t)pr[2], (half_t)pr[3]};
+    if (a.probs)
+      st8<false>(a.probs, (int)((((size_t)(b * NH + hh) * S + q) * S + t * 16 + g * 4) * 2), as_u2(p[t]));
+  }
+  __syncthreads();   // V tile is in LDS
+  f4 o[HD / 16];
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt) o[dt] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int t = 0; t < NKT; ++t) {
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) {
+      const h4 vop = lds_read_tr16(lds + (t * 16 + g * 4 + (l16 >> 2)) * kVLD + dt * 16 + (l16 & 3) * 4);
+      o[dt] = mfma_16x16x16(vop, p[t], o[dt]);
+    }
+  }
+  // o[dt][v] = ctx(query q, d = 16dt + 4g + v)
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt)
+    st8<COH>(a.ctx, ((b * S + q) * H + hh * HD + dt * 16 + g * 4) * 2, pack_h4(o[dt]));
+}
+
+template <bool COH>
+__device__ __forceinline__ void stage_attn(half_t *lds, const Args &a, int first, int stride) {
+  const int items = a.B * NH * (a.S / 64);
+  for (int item = first; item < items; item += stride) {
+    switch (a.S) {
+      case 64: attn_item<COH, 4>(lds, a, item); break;
+      case 128: attn_item<COH, 8>(lds, a, item); break;
+      case 256: attn_item<COH, 16>(lds, a, item); break;
+      case 384: attn_item<COH, 24>(lds, a, item); break;
+      default: attn_item<COH, 32>(lds, a, item); break;   // 512 (validated on the host)
+    }
+  }
+}
+
+using TileSmall = GemmTile<64, 64, 64, 2, 2>;
+using TileLarge = GemmTile<128, 128, 64, 2, 2>;
+constexpr int kAttnLdsBytes = 512 * kVLD * 2;
+constexpr int lds_bytes(bool large) {
+  const int t = large ? TileLarge::LDS_BYTES : TileSmall::LDS_BYTES;
+  return t > kAttnLdsBytes ? t : kAttnLdsBytes;
+}
+
+// ------------------------------------------------------------ megakernel ----
+template <bool LARGE>
+__global__ void __launch_bounds__(256) k_encoder_mega(Args a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  half_t *lds = reinterpret_cast<half_t *>(lds_raw);
+  using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
+  GridBarrier bar;
+  grid_barrier_begin(bar, a.ctl);
+  const int first = blockIdx.x, stride = gridDim.x;
+  const int wave = threadIdx.x >> 6;
+  const half_t *xin = a.x;
+  for (int l = 0; l < a.num_layers; ++l) {
+    const LayerW &w = a.layers[l];
+    half_t *yout = (l == a.num_layers - 1) ? a.y : ((l & 1) ? a.xb : a.xa);
+    stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
+    grid_sync(bar);
+    stage_attn<true>(lds, a, first, stride);
+    grid_sync(bar);
+    stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
+    grid_sync(bar);
+    stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
+    grid_sync(bar);
+    stage_fc1<true, Tile>(lds, a, w, first, stride);
+    grid_sync(bar);
+    stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
+    grid_sync(bar);
+    stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
+    if (l + 1 < a.num_layers) grid_sync(bar);
+    xin = yout;
+  }
+  grid_barrier_end(bar);
+}
+
+// ------------------------------------------------------ per-op kernels ----
+template <bool LARGE>
+__global__ void __launch_bounds__(256) k_qkv(Args a, int l, const half_t *xin) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
+  stage_qkv<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], xin, blockIdx.x, gridDim.x);
+}
+__global__ void __launch_bounds__(256) k_attn(Args a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  stage_attn<false>(reinterpret_cast<half_t *>(lds_raw), a, blockIdx.x, gridDim.x);
+}
+template <bool LARGE>
+__global__ void __launch_bounds__(256) k_partial(Args a, const half_t *X, int K, const half_t *W, int splitk) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
+  stage_partial<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, X, K, W, splitk, blockIdx.x, gridDim.x);
+}
+__global__ void __launch_bounds__(256) k_ln(Args a, int splitk, const half_t *bias, const half_t *resid,
+                                            const half_t *gam, const half_t *bet, half_t *out) {
+  stage_ln<false>(a, splitk, bias, resid, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
+}
+template <bool LARGE>
+__global__ void __launch_bounds__(256) k_fc1(Args a, int l) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
+  stage_fc1<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], blockIdx.x, gridDim.x);
+}
+
+// ------------------------------------------------------------------- host ----
+struct Plan {
+  bool large;
+  int splitk_o, splitk_f;
+  size_t off_ctl, off_qkv, off_ctx, off_y1, off_h, off_xa, off_xb, off_part, total;
+};
+
+static int validate(const souffle_bert_cfg *c) {
+  if (!c) return fail(SOUFFLE_ERR_NULL, "cfg is NULL");
+  if (c->hidden != H || c->heads != NH || c->ffn != F)
+    return fail(SOUFFLE_ERR_SHAPE, "only hidden=768 heads=12 ffn=3072 is built (got %d/%d/%d)", c->hidden, c->heads, c->ffn);
+  if (c->batch <= 0 || c->seq_len <= 0) return fail(SOUFFLE_ERR_SHAPE, "batch and seq_len must be positive");
+  const int s = c->seq_len;
+  if (!(s == 64 || s == 128 || s == 256 || s == 384 || s == 512))
+    return fail(SOUFFLE_ERR_SHAPE, "seq_len must be one of 64,128,256,384,512 (got %d)", s);
+  const long long m = (long long)c->batch * s;
+  if (m >= 1024 && m % 128 != 0) return fail(SOUFFLE_ERR_SHAPE, "batch*seq_len >= 1024 must be a multiple of 128 (got %lld)", m);
+  if (m > 65536) return fail(SOUFFLE_ERR_SHAPE, "batch*seq_len must be <= 65536 (got %lld)", m);
+  if (c->act != SOUFFLE_ACT_GELU_TANH && c->act != SOUFFLE_ACT_RELU) return fail(SOUFFLE_ERR_SHAPE, "unknown activation %d", c->act);
+  if (!(c->ln_eps >= 0.f)) return fail(SOUFFLE_ERR_SHAPE, "ln_eps must be >= 0");
+  return SOUFFLE_OK;
+}
+
+static Plan make_plan(const souffle_bert_cfg *c) {
+  Plan p;
+  const size_t M = (size_t)c->batch * c->seq_len;
+  p.large = M >= 1024;
+  p.splitk_o = p.large ? 1 : 4;
+  p.splitk_f = p.large ? 1 : 8;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off += round_up(bytes, 256); return o; };
+  p.off_ctl = take(kCtlWords * 4);
+  p.off_qkv = take(3 * M * H * 2);
+  p.off_ctx = take(M * H * 2);
+  p.off_y1 = take(M * H * 2);
+  p.off_h = take(M * F * 2);
+  p.off_xa = take(M * H * 2);
+  p.off_xb = take(M * H * 2);
+  p.off_part = take((size_t)(p.splitk_f > p.splitk_o ? p.splitk_f : p.splitk_o) * M * H * 4);
+  p.total = off;
+  return p;
+}
+
+static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_layer_w *layers, int nl,
+                     const void *x, const void *mask, void *y, const souffle_bert_dump *dump,
+                     void *ws, size_t ws_bytes, const Plan &p) {
+  if (!layers || !x || !y) return fail(SOUFFLE_ERR_NULL, "layers, x and y must not be NULL");
+  if (!ws) return fail(SOUFFLE_ERR_WORKSPACE, "workspace is NULL (need %zu bytes)", p.total);
+  if (ws_bytes < p.total) return fail(SOUFFLE_ERR_WORKSPACE, "workspace too small: %zu < %zu bytes", ws_bytes, p.total);
+  if (nl < 1 || nl > kMaxLayers) return fail(SOUFFLE_ERR_SHAPE, "num_layers must be in 1..%d (got %d)", kMaxLayers, nl);
+  if (!aligned16(x) || !aligned16(y) || !aligned16(ws) || (mask && !aligned16(mask)))
+    return fail(SOUFFLE_ERR_ALIGN, "x, y, mask and workspace must be 16-byte aligned");
+  char *base = static_cast<char *>(ws);
+  a.B = c->batch; a.S = c->seq_len; a.M = c->batch * c->seq_len; a.act = c->act; a.num_layers = nl;
+  a.splitk_o = p.splitk_o; a.splitk_f = p.splitk_f; a.scale = c->scale; a.eps = c->ln_eps;
+  a.x = static_cast<const half_t *>(x); a.mask = static_cast<const half_t *>(mask); a.y = static_cast<half_t *>(y);
+  a.ctl = reinterpret_cast<unsigned *>(base + p.off_ctl);
+  a.qkv = reinterpret_cast<half_t *>(base + p.off_qkv);
+  a.ctx = reinterpret_cast<half_t *>(base + p.off_ctx);
+  a.y1 = reinterpret_cast<half_t *>(base + p.off_y1);
+  a.h = reinterpret_cast<half_t *>(base + p.off_h);
+  a.xa = reinterpret_cast<half_t *>(base + p.off_xa);
+  a.xb = reinterpret_cast<half_t *>(base + p.off_xb);
+  a.part = reinterpret_cast<float *>(base + p.off_part);
+  a.probs = nullptr;
+  if (dump) {   // the per-stage tensors are produced in the reference's own layouts: write them in place
+    if (dump->qkv) a.qkv = static_cast<half_t *>(dump->qkv);
+    if (dump->ctx) a.ctx = static_cast<half_t *>(dump->ctx);
+    if (dump->ln1) a.y1 = static_cast<half_t *>(dump->ln1);
+    if (dump->fc1) a.h = static_cast<half_t *>(dump->fc1);
+    a.probs = static_cast<half_t *>(dump->probs);
+    if (!aligned16(a.qkv) || !aligned16(a.ctx) || !aligned16(a.y1) || !aligned16(a.h) || !aligned16(a.probs))
+      return fail(SOUFFLE_ERR_ALIGN, "dump pointers must be 16-byte aligned");
+  }
+  for (int l = 0; l < nl; ++l) {
+    const souffle_bert_layer_w &s = layers[l];
+    if (!s.w_qkv || !s.w_o || !s.w_fc1 || !s.w_fc2) return fail(SOUFFLE_ERR_NULL, "layer %d: a weight matrix is NULL", l);
+    const void *ptrs[12] = {s.w_qkv, s.b_qkv, s.w_o, s.b_o, s.ln1_g, s.ln1_b, s.w_fc1, s.b_fc1, s.w_fc2, s.b_fc2, s.ln2_g, s.ln2_b};
+    for (const void *q : ptrs)
+      if (!aligned16(q)) return fail(SOUFFLE_ERR_ALIGN, "layer %d: a weight/bias pointer is not 16-byte aligned", l);
+    LayerW &d = a.layers[l];
+    d.w_qkv = (const half_t *)s.w_qkv; d.b_qkv = (const half_t *)s.b_qkv; d.w_o = (const half_t *)s.w_o; d.b_o = (const half_t *)s.b_o;
+    d.ln1_g = (const half_t *)s.ln1_g; d.ln1_b = (const half_t *)s.ln1_b; d.w_fc1 = (const half_t *)s.w_fc1; d.b_fc1 = (const half_t *)s.b_fc1;
+    d.w_fc2 = (const half_t *)s.w_fc2; d.b_fc2 = (const half_t *)s.b_fc2; d.ln2_g = (const half_t *)s.ln2_g; d.ln2_b = (const half_t *)s.ln2_b;
+  }
+  return SOUFFLE_OK;
+}
+
+template <bool LARGE>
+static int launch_mega(Args &a, int grid, hipStream_t st) {
+  const int lds = lds_bytes(LARGE);
+  static bool attr_done = false;
+  if (!attr_done) {
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_encoder_mega<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    attr_done = true;
+  }
+  void *args[] = {&a};
+  SOUFFLE_HIP_TRY(hipLaunchCooperativeKernel((const void *)k_encoder_mega<LARGE>, dim3(grid), dim3(256), args, lds, st));
+  return SOUFFLE_OK;
+}
+
+static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *layers, int nl, const void *x,
+                     const void *mask, void *y, const souffle_bert_dump *dump, void *ws, size_t ws_bytes,
+                     souffle_stream_t stream) {
+  if (int rc = validate(c)) return rc;
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  if (!df.cooperative) return fail(SOUFFLE_ERR_DEVICE, "device does not support cooperative launch");
+  const Plan p = make_plan(c);
+  static thread_local Args a;
+  if (int rc = fill_args(a, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return p.large ? launch_mega<true>(a, df.num_cus, st) : launch_mega<false>(a, df.num_cus, st);
+}
+
+template <bool LARGE>
+static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
+  using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
+  constexpr int BM = LARGE ? 128 : 64, BN = LARGE ? 128 : 64;
+  static bool attr_done = false;
+  if (!attr_done) {
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_qkv<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_partial<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_fc1<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_attn, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLdsBytes));
+    attr_done = true;
+  }
+  const int cap = num_cus * 4;
+  auto grid_for = [&](int items) { return items < cap ? items : cap; };
+  const int tm = a.M / BM;
+  const half_t *xin = a.x;
+  for (int l = 0; l < nl; ++l) {
+    const LayerW &w = a.layers[l];
+    half_t *yout = (l == nl - 1) ? a.y : ((l & 1) ? a.xb : a.xa);
+    hipLaunchKernelGGL(k_qkv<LARGE>, dim3(grid_for(tm * (3 * H / BN))), dim3(256), Tile::LDS_BYTES, st, a, l, xin);
+    hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), a.S * kVLD * 2, st, a);
+    hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for(tm * (H / BN) * a.splitk_o)), dim3(256), Tile::LDS_BYTES, st, a, a.ctx, H, w.w_o, a.splitk_o);
+    hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
+    hipLaunchKernelGGL(k_fc1<LARGE>, dim3(grid_for(tm * (F / BN))), dim3(256), Tile::LDS_BYTES, st, a, l);
+    hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for(tm * (H / BN) * a.splitk_f)), dim3(256), Tile::LDS_BYTES, st, a, a.h, F, w.w_fc2, a.splitk_f);
+    hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout);
+    xin = yout;
+  }
+  SOUFFLE_HIP_TRY(hipGetLastError());
+  return SOUFFLE_OK;
+}
+
+static int run_unfused(const souffle_bert_cfg *c, const souffle_bert_layer_w *layers, int nl, const void *x,
+                       const void *mask, void *y, const souffle_bert_dump *dump, void *ws, size_t ws_bytes,
+                       souffle_stream_t stream) {
+  if (int rc = validate(c)) return rc;
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  const Plan p = make_plan(c);
+  static thread_local Args a;
+  if (int rc = fill_args(a, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return p.large ? run_unfused_t<true>(a, nl, df.num_cus, st) : run_unfused_t<false>(a, nl, df.num_cus, st);
+}
+
+}  // namespace bert
+}  // namespace souffle
+
+using namespace souffle;
+
+extern "C" size_t souffle_bert_workspace_bytes(const souffle_bert_cfg *cfg) {
+  if (bert::validate(cfg)) return 0;
+  return bert::make_plan(cfg).total;
+}
+extern "C" int souffle_bert_layer_fused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *w, const void *x,
+                                        const void *mask, void *y, const souffle_bert_dump *dump, void *ws,
+                                        size_t ws_bytes, souffle_stream_t stream) {
+  return bert::run_fused(cfg, w, 1, x, mask, y, dump, ws, ws_bytes, stream);
+}
+extern "C" int souffle_bert_layer_unfused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *w, const void *x,
+                                          const void *mask, void *y, const souffle_bert_dump *dump, void *ws,
+                                          size_t ws_bytes, souffle_stream_t stream) {
+  return bert::run_unfused(cfg, w, 1, x, mask, y, dump, ws, ws_bytes, stream);
+}
+extern "C" int souffle_bert_encoder_fused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
+                                          const void *x, const void *mask, void *y, void *ws, size_t ws_bytes,
+                                          souffle_stream_t stream) {
+  if (!cfg) return fail(SOUFFLE_ERR_NULL, "cfg is NULL");
+  return bert::run_fused(cfg, layers, cfg->num_layers, x, mask, y, nullptr, ws, ws_bytes, stream);
+}
+extern "C" int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
+                                            const void *x, const void *mask, void *y, void *ws, size_t ws_bytes,
+                                            souffle_stream_t stream) {
+  if (!cfg) return fail(SOUFFLE_ERR_NULL, "cfg is NULL");
+  return bert::run_unfused(cfg, layers, cfg->num_layers, x, mask, y, nullptr, ws, ws_bytes, stream);
+}

@@ -1,0 +1,35 @@
+// Host-side helpers shared by the C-ABI translation units: thread-local error text,
+// argument checks, device facts.  Replaces checkCuda / check_compatability of the
+// reference (cpp/souffle_utils/cuda_utils.h:10-19,86-98): nothing here prints or aborts.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include "../../include/souffle_hip.h"
+
+namespace souffle {
+
+char *error_buffer();                       // thread-local, 512 bytes
+int fail(int code, const char *fmt, ...);   // formats into error_buffer(), returns code
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+struct DeviceFacts {
+  int ok;            // 0 until queried successfully
+  int num_cus, lds_per_cu, cooperative;
+  char arch[64];
+};
+// Cached per process for the current device; returns a negative status on failure.
+int device_facts(DeviceFacts *out);
+
+inline size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+#define SOUFFLE_HIP_TRY(expr)                                                            \
+  do {                                                                                   \
+    hipError_t e_ = (expr);                                                              \
+    if (e_ != hipSuccess)                                                                \
+      return ::souffle::fail(SOUFFLE_ERR_LAUNCH, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+}  // namespace souffle

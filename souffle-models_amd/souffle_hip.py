@@ -1,0 +1,171 @@
+"""ctypes view of libsouffle_hip.so (the C ABI declared in include/souffle_hip.h).
+
+The binding modules in this directory (bert_binding, lstm_binding,
+swin_transformer_binding, swin_trans_fc2, efficientnet_se_module_binding) are thin
+wrappers over this module; torch is used for device memory and streams only.
+There is no CPU or eager fallback: if the library is missing, loading fails.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libsouffle_hip.so")
+
+ACT_GELU_TANH, ACT_RELU = 0, 1
+GATES_IFGO, GATES_IGFO = 0, 1
+SE_MUL, SE_ADD = 0, 1
+
+
+class BertCfg(C.Structure):
+    _fields_ = [("batch", C.c_int), ("seq_len", C.c_int), ("hidden", C.c_int), ("heads", C.c_int),
+                ("ffn", C.c_int), ("act", C.c_int), ("scale", C.c_float), ("ln_eps", C.c_float),
+                ("num_layers", C.c_int), ("reserved", C.c_int)]
+
+
+BERT_W_FIELDS = ["w_qkv", "b_qkv", "w_o", "b_o", "ln1_g", "ln1_b", "w_fc1", "b_fc1", "w_fc2", "b_fc2",
+                 "ln2_g", "ln2_b"]
+
+
+class BertLayerW(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in BERT_W_FIELDS]
+
+
+class BertDump(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ["qkv", "probs", "ctx", "ln1", "fc1"]]
+
+
+class LstmCfg(C.Structure):
+    _fields_ = [("layers", C.c_int), ("hidden", C.c_int), ("timesteps", C.c_int), ("batch", C.c_int),
+                ("gate_order", C.c_int), ("forget_bias", C.c_float)]
+
+
+class SwinCfg(C.Structure):
+    _fields_ = [("height", C.c_int), ("width", C.c_int), ("channels", C.c_int), ("heads", C.c_int),
+                ("window", C.c_int), ("shift", C.c_int), ("mlp_ratio", C.c_int),
+                ("use_shift_mask", C.c_int), ("ln_eps", C.c_float)]
+
+
+SWIN_W_FIELDS = ["ln1_g", "ln1_b", "w_qkv", "b_qkv", "rel_table", "w_proj", "b_proj", "ln2_g", "ln2_b",
+                 "w_fc1", "b_fc1", "w_fc2", "b_fc2"]
+
+
+class SwinBlockW(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in SWIN_W_FIELDS]
+
+
+class DevInfo(C.Structure):
+    _fields_ = [("num_cus", C.c_int), ("lds_bytes_per_cu", C.c_int), ("clock_khz", C.c_int),
+                ("mem_clock_khz", C.c_int), ("mem_bus_bits", C.c_int), ("l2_bytes", C.c_int),
+                ("cooperative_launch", C.c_int), ("wavefront_size", C.c_int), ("arch", C.c_char * 64)]
+
+
+BENCH_FN = C.CFUNCTYPE(C.c_int, C.c_void_p)
+
+# name -> (restype, argtypes); every symbol include/souffle_hip.h declares
+SIGNATURES = {
+    "souffle_last_error": (C.c_char_p, []),
+    "souffle_version": (C.c_char_p, []),
+    "souffle_device_info": (C.c_int, [C.POINTER(DevInfo)]),
+    "souffle_workspace_init": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
+    "souffle_bert_workspace_bytes": (C.c_size_t, [C.POINTER(BertCfg)]),
+    "souffle_bert_layer_fused": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
+                                           C.c_void_p, C.POINTER(BertDump), C.c_void_p, C.c_size_t, C.c_void_p]),
+    "souffle_bert_layer_unfused": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
+                                             C.c_void_p, C.POINTER(BertDump), C.c_void_p, C.c_size_t, C.c_void_p]),
+    "souffle_bert_encoder_fused": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
+                                             C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "souffle_bert_encoder_unfused": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
+                                               C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "souffle_lstm_workspace_bytes": (C.c_size_t, [C.POINTER(LstmCfg)]),
+    "souffle_lstm_fused": (C.c_int, [C.POINTER(LstmCfg), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                     C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "souffle_swin_workspace_bytes": (C.c_size_t, [C.POINTER(SwinCfg)]),
+    "souffle_swin_block_pair_fused": (C.c_int, [C.POINTER(SwinCfg), C.POINTER(SwinBlockW), C.c_void_p, C.c_void_p,
+                                                C.c_void_p, C.c_size_t, C.c_void_p]),
+    "souffle_swin_index_maps": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                          C.c_void_p, C.c_void_p]),
+    "souffle_swin_ffn_fused": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                         C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "souffle_gemm_f16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+    "souffle_se_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
+    "souffle_se_module_fused": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                          C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t,
+                                          C.c_void_p]),
+    "souffle_bench_us": (C.c_int, [BENCH_FN, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                   C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+}
+
+_lib = None
+
+
+class SouffleError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__("souffle_hip error %d: %s" % (code, text))
+        self.code = code
+
+
+def lib():
+    """Load the library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libsouffle_hip.so is missing at %s: build it with build.py "
+                               "(there is no fallback path)" % LIB_PATH)
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def last_error():
+    return lib().souffle_last_error().decode()
+
+
+def check(rc):
+    if rc != 0:
+        raise SouffleError(rc, last_error())
+
+
+def ptr(t):
+    """Device pointer of a torch tensor (or None)."""
+    return None if t is None else t.data_ptr()
+
+
+def current_stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+class Workspace:
+    """A zero-initialised device workspace, cached by the binding modules."""
+
+    def __init__(self, nbytes, device="cuda:0"):
+        import torch
+        self.buf = torch.zeros(max(int(nbytes), 16384) // 4 + 4, dtype=torch.int32, device=device)
+        self.nbytes = self.buf.numel() * 4
+        check(lib().souffle_workspace_init(self.buf.data_ptr(), self.nbytes, current_stream()))
+
+    @property
+    def ptr(self):
+        return self.buf.data_ptr()
+
+
+def device_info():
+    info = DevInfo()
+    check(lib().souffle_device_info(C.byref(info)))
+    return {n: (getattr(info, n).decode() if n == "arch" else getattr(info, n)) for n, _ in DevInfo._fields_}
+
+
+def bench_us(launch, warmup=20, rounds=10, repeat=100, stream=None):
+    """min-of-means and median (us) of `launch()` under the reference's timing rule
+    (cpp/souffle_utils/cuda_utils.h:102-136), timed with HIP events on `stream`."""
+    def _fn(_):
+        launch()
+        return 0
+    cb = BENCH_FN(_fn)
+    mn, med = C.c_double(), C.c_double()
+    check(lib().souffle_bench_us(cb, None, current_stream() if stream is None else stream, warmup, rounds,
+                                 repeat, C.byref(mn), C.byref(med)))
+    return mn.value, med.value

@@ -1,0 +1,127 @@
+"""GPU parity of the BERT encoder layer / encoder (through the C ABI via bert_binding)
+against the CPU oracle on identical fp16-rounded seeded inputs.
+Tolerance: max-abs <= 2e-2 and mean-abs <= 2e-3 on every tensor the reference returns."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import synth
+from gpu_util import announce, assert_close, dev, dev_weights
+
+pytestmark = pytest.mark.gpu
+NAMES = ["output_qkv", "query_key_output", "attn_value_output", "attn_fc_output", "feed_forward_fc1_output",
+         "feed_forward_fc2_output"]
+
+
+def run_layer(w, x, B, S, opt_level, **kw):
+    import bert_binding
+    dw = dev_weights(w)
+    extra = {k: dw[k] for k in dw if k not in ("qkv_weight", "attn_fc_weight", "fc1_weight", "fc2_weight")}
+    outs = bert_binding.souffle_bert_layer(dev(x).view(B, S, 768), dw["qkv_weight"], dw["attn_fc_weight"],
+                                           dw["fc1_weight"], dw["fc2_weight"], opt_level, **extra, **kw)
+    torch.cuda.synchronize()
+    return outs
+
+
+@pytest.mark.parametrize("opt_level", [4, 1])
+@pytest.mark.parametrize("B,S", [(1, 128), (1, 384), (1, 64), (2, 256)])
+def test_layer_config0_all_stages(B, S, opt_level):
+    """Benchmark config 0 (zero biases, gamma 1, beta 0, tanh-GELU, scale 1/8, eps 1e-12, no mask)."""
+    announce("bert layer cfg0 B=%d S=%d opt=%d" % (B, S, opt_level))
+    w, x = synth.bert_layer_weights(0, 0), synth.bert_input(0, B, S)
+    ref = oracle.bert_layer(x, w, B, S, dump=True)
+    got = run_layer(w, x, B, S, opt_level)
+    for n, g, r in zip(NAMES, got, ref):
+        assert_close(n, g, r)
+
+
+@pytest.mark.parametrize("opt_level", [3, 2])
+def test_layer_bias_affine_mask(opt_level):
+    announce("bert layer bias+affine+mask opt=%d" % opt_level)
+    B, S = 2, 128
+    w, x = synth.bert_layer_weights(0, 1, with_bias=True), synth.bert_input(7, B, S)
+    keep = synth.uniform01(synth.seed_of(0, 99), B * S * S).reshape(B, S, S) < 0.85
+    keep[:, :, 0] = True
+    mask = np.where(keep, 0.0, -10000.0).astype(np.float16)
+    ref = oracle.bert_layer(x, w, B, S, mask=mask, dump=True)
+    got = run_layer(w, x, B, S, opt_level, mask=dev(mask))
+    for n, g, r in zip(NAMES, got, ref):
+        assert_close(n, g, r)
+
+
+def test_layer_reference_compat_mode():
+    """What the reference's fused CUDA path computes: ReLU, scale 1/sqrt(768), eps 1e-5."""
+    announce("bert layer reference-compat")
+    B, S = 1, 384
+    w, x = synth.bert_layer_weights(0, 2), synth.bert_input(0, B, S)
+    ref = oracle.bert_layer(x, w, B, S, act="relu", scale=768 ** -0.5, ln_eps=1e-5, dump=True)
+    got = run_layer(w, x, B, S, 4, reference_compat=True)
+    for n, g, r in zip(NAMES, got, ref):
+        assert_close(n, g, r)
+
+
+def test_layer_mfma_bound_shape():
+    """B=32, S=128 (M=4096): the large-tile path."""
+    announce("bert layer B=32 S=128")
+    B, S = 32, 128
+    w, x = synth.bert_layer_weights(2, 0), synth.bert_input(2, B, S)
+    ref = oracle.bert_layer(x, w, B, S, dump=True)
+    for opt in (4, 1):
+        got = run_layer(w, x, B, S, opt)
+        for n, g, r in zip(NAMES, got, ref):
+            assert_close("%s(opt %d)" % (n, opt), g, r)
+
+
+def test_fast_path_equals_dump_path_and_is_deterministic():
+    announce("bert layer dump=False determinism")
+    B, S = 1, 128
+    w, x = synth.bert_layer_weights(0, 0), synth.bert_input(0, B, S)
+    full = run_layer(w, x, B, S, 4)[-1]
+    a = run_layer(w, x, B, S, 4, dump=False)
+    b = run_layer(w, x, B, S, 4, dump=False)
+    c = run_layer(w, x, B, S, 1, dump=False)
+    assert torch.equal(a, b) and torch.equal(a, full)
+    assert torch.equal(a, c), "fused and per-op paths run the same arithmetic"
+
+
+@pytest.mark.parametrize("B,S,layers", [(1, 128, 12), (1, 384, 3), (32, 128, 2)])
+def test_encoder_matches_oracle(B, S, layers):
+    announce("bert encoder B=%d S=%d L=%d" % (B, S, layers))
+    import bert_binding
+    ws = [synth.bert_layer_weights(2, l) for l in range(layers)]
+    x = synth.bert_input(2, B, S)
+    ref = oracle.bert_encoder(x, ws, B, S)
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    y_f = enc(dev(x), fused=True)
+    y_u = enc(dev(x), fused=False)
+    torch.cuda.synchronize()
+    # errors of successive layers do not compound past the tolerance because each layer ends in a LayerNorm
+    assert_close("encoder fused", y_f, ref)
+    assert_close("encoder unfused", y_u, ref)
+    assert torch.equal(y_f, y_u)
+
+
+def test_layernorm_invariants_at_full_size():
+    """Size-independent property: with gamma 1 / beta 0 every output row has mean 0, variance 1."""
+    announce("bert LN invariants B=32")
+    B, S = 32, 128
+    w, x = synth.bert_layer_weights(2, 1), synth.bert_input(3, B, S)
+    y = run_layer(w, x, B, S, 4, dump=False).float()
+    assert y.mean(dim=1).abs().max().item() < 2e-3
+    assert (y.var(dim=1, unbiased=False) - 1).abs().max().item() < 5e-3
+
+
+def test_argument_errors_are_reported_not_fatal():
+    announce("bert argument errors")
+    import bert_binding
+    import souffle_hip as sh
+    w = dev_weights(synth.bert_layer_weights(0, 0))
+    x = torch.zeros(1, 100, 768, dtype=torch.float16, device="cuda:0")
+    with pytest.raises(sh.SouffleError) as e:
+        bert_binding.souffle_bert_layer(x, w["qkv_weight"], w["attn_fc_weight"], w["fc1_weight"], w["fc2_weight"], 4)
+    assert e.value.code == -2 and "seq_len" in str(e.value)
+    with pytest.raises(ValueError):
+        bert_binding.souffle_bert_layer(x, w["qkv_weight"], w["attn_fc_weight"], w["fc1_weight"], w["fc2_weight"], 9)
+    with pytest.raises(TypeError):
+        bert_binding.souffle_bert_layer(x.float(), w["qkv_weight"], w["attn_fc_weight"], w["fc1_weight"], w["fc2_weight"], 4)
