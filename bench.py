@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-encoder hot path on one MI355X.
+
+Default workload (the metric of BASELINE.json): the BERT-base 12-layer encoder at B=1,
+S=128, fp16, one persistent cooperative launch per forward pass.  A step is one forward
+pass over one synthetic input; the timed passes rotate through several distinct weight
+sets (> 512 MB in total) so that the weight stream comes from HBM, not from the 256 MB
+Infinity Cache.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload encoder|layer|encoder_b32|lstm|swin]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "souffle-models_amd"))
+
+HBM_PEAK_GBS = 8000.0            # MI355X published HBM3E bandwidth
+MFMA_F16_PEAK_TFLOPS = 2500.0    # MI355X published dense fp16 MFMA peak
+
+# algorithmic HBM bytes / flops of one encoder layer (weights once + biases + LN vectors + x in + y out)
+def layer_bytes(M):
+    return 7077888 * 2 + 13824 + 6144 + 2 * M * 768 * 2
+
+
+def layer_flops(B, S):
+    return 2.0 * B * S * 7077888 + 4.0 * B * S * S * 768
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--workload", default="encoder")
+    p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU-baseline sample")
+    p.add_argument("--no-cpu", action="store_true")
+    p.add_argument("--weight-sets", type=int, default=4)
+    return p.parse_args()
+
+
+def cpu_baseline_encoder(layers_np, x_np, B, S, budget_s):
+    """The CPU oracle (a port: the reference has no CPU path) timed on the host cores."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle
+    threads = os.cpu_count() or 1
+    try:
+        threads = len(os.sched_getaffinity(0))
+    except Exception:
+        pass
+    threads = min(threads, 16)
+    os.environ.setdefault("OMP_NUM_THREADS", str(threads))
+    oracle.bert_encoder(x_np, layers_np[:1], B, S, threads=threads)       # warm up
+    n, t0 = 0, time.perf_counter()
+    ref = None
+    while True:
+        ref = oracle.bert_encoder(x_np, layers_np, B, S, threads=threads)
+        n += 1
+        if time.perf_counter() - t0 > budget_s or n >= 50:
+            break
+    dt = (time.perf_counter() - t0) / n
+    return ref, {"value": dt * 1e6, "unit": "us", "cores": threads, "kind": "port",
+                 "sample": "%d passes of the %d-layer encoder B=%d S=%d through oracle/bert_oracle.c (OpenMP fp32)" % (n, len(layers_np), B, S)}
+
+
+def time_steps(launch, steps, warmup):
+    """W untimed steps, then exactly K timed steps bracketed by synchronize on both sides;
+    HIP events on the launch stream give the average launch duration."""
+    import torch
+    for i in range(warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        launch(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = e0.elapsed_time(e1) / steps
+    return wall_ms, ev_ms
+
+
+def bench_encoder(args, B, S, L, name):
+    import numpy as np
+    import torch
+    import bert_binding
+    import souffle_hip as sh
+    import synth
+
+    dev = torch.device("cuda:0")
+    to_dev = lambda w: {k: torch.from_numpy(v).to(dev) for k, v in w.items()}
+    layers_np = [synth.bert_layer_weights(2, l) for l in range(L)]
+    x_np = synth.bert_input(2, B, S)
+    x = torch.from_numpy(x_np).to(dev)
+    M = B * S
+    # distinct weight sets for the cold-cache rotation (set 0 is the checked one; the others
+    # are shuffled copies: same sizes and value distribution, different addresses)
+    sets = [[to_dev(w) for w in layers_np]]
+    for s in range(1, max(1, args.weight_sets)):
+        sets.append([{k: v.clone() for k, v in sets[0][(l + s) % L].items()} for l in range(L)])
+    encs = [bert_binding.Encoder(ls, B, S) for ls in sets]
+    out = torch.empty((M, 768), dtype=torch.float16, device=dev)
+
+    # parity gate
+    cpu = None
+    y = encs[0](x, out=out).float().cpu().numpy()
+    if not args.no_cpu:
+        ref, cpu = cpu_baseline_encoder(layers_np, x_np, B, S, args.cpu_seconds)
+        d = np.abs(y - ref)
+        if not (np.isfinite(y).all() and d.max() <= 2e-2 and d.mean() <= 2e-3):
+            print("PARITY FAILURE: max-abs %.4g mean-abs %.4g" % (d.max(), d.mean()), file=sys.stderr)
+            sys.exit(1)
+        parity = {"max_abs": float(d.max()), "mean_abs": float(d.mean())}
+    else:
+        parity = None
+
+    cold_wall, cold_ev = time_steps(lambda i: encs[i % len(encs)](x, out=out), args.steps, args.warmup)
+    warm_wall, warm_ev = time_steps(lambda i: encs[0](x, out=out), args.steps, args.warmup)
+    unf_wall, unf_ev = time_steps(lambda i: encs[i % len(encs)](x, out=out, fused=False), max(10, args.steps // 4), 5)
+    # the reference's own timing rule (min over rounds of the mean of repeated event-timed launches)
+    mn, med = sh.bench_us(lambda: encs[0](x, out=out), warmup=10, rounds=5, repeat=max(10, args.steps // 5))
+
+    bytes_alg = L * layer_bytes(M)
+    flops = L * layer_flops(B, S)
+    mfma_bound = flops / (MFMA_F16_PEAK_TFLOPS * 1e12) > bytes_alg / (HBM_PEAK_GBS * 1e9)
+    if mfma_bound:
+        ach = flops / (cold_ev * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": ach, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": ach / MFMA_F16_PEAK_TFLOPS, "traffic": None}
+    else:
+        ach = bytes_alg / (cold_ev * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS,
+                "traffic": None}
+    roof["kernel"] = "k_encoder_mega (one cooperative launch = %d layers)" % L
+    roof["algorithmic_bytes_per_launch"] = bytes_alg
+    roof["algorithmic_flops_per_launch"] = flops
+    roof["avg_launch_us"] = cold_ev * 1e3
+    res = {
+        "metric": "bert_base_encoder_latency_us", "value": cold_wall * 1e3, "unit": "us", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": cold_wall, "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": name, "batch": B, "seq_len": S, "layers": L, "hidden": 768, "heads": 12, "ffn": 3072,
+                   "weights": "random N(0,0.02) fp16, %d rotating sets" % len(encs)},
+        "roofline": roof,
+        "extra": {"per_layer_us_cold": cold_ev * 1e3 / L, "warm_cache_us": warm_ev * 1e3, "per_layer_us_warm": warm_ev * 1e3 / L,
+                  "unfused_per_op_us": unf_ev * 1e3, "fused_speedup_vs_unfused": unf_ev / cold_ev,
+                  "min_of_means_us_warm": mn, "median_us_warm": med, "parity": parity,
+                  "launches_fused": 1, "launches_unfused": 7 * L},
+    }
+    if cpu:
+        res["cpu_baseline"] = cpu
+        res["extra"]["gpu_speedup_vs_cpu"] = cpu["value"] / (cold_ev * 1e3)
+    return res
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("no GPU available", file=sys.stderr)
+        sys.exit(3)
+    if args.workload == "encoder":
+        res = bench_encoder(args, 1, 128, 12, "BERT-base 12-layer encoder, B=1, S=128, fp16 (BASELINE configs[2], first shape)")
+    elif args.workload == "layer":
+        res = bench_encoder(args, 1, 128, 1, "single BERT-base encoder layer, B=1, S=128, fp16 (BASELINE configs[0])")
+    elif args.workload == "encoder_s384":
+        res = bench_encoder(args, 1, 384, 12, "BERT-base 12-layer encoder, B=1, S=384, fp16")
+    elif args.workload == "encoder_b32":
+        args.weight_sets = 1
+        res = bench_encoder(args, 32, 128, 12, "BERT-base 12-layer encoder, B=32, S=128, fp16 (MFMA-bound shape)")
+    else:
+        import bench_extra
+        res = bench_extra.run(args)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

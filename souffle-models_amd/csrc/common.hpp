@@ -63,6 +63,17 @@ __device__ __forceinline__ u2 ld8(const void *base, int byte_off) {
   if constexpr (COH) return __builtin_amdgcn_raw_buffer_load_b64(make_rsrc(base), byte_off, 0, kAuxSc1);
   else return *reinterpret_cast<const u2 *>(reinterpret_cast<const char *>(base) + byte_off);
 }
+// 8-byte relaxed agent-scope atomics: a (value, tag) pair that is published and polled
+// as one unit.  Being atomic operations, polling loads are re-issued on every spin.
+__device__ __forceinline__ u2 ld8_atomic(const void *p) {
+  const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long *>(p), __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+  return u2{(unsigned)v, (unsigned)(v >> 32)};
+}
+__device__ __forceinline__ void st8_atomic(void *p, u2 v) {
+  __hip_atomic_store(reinterpret_cast<unsigned long long *>(p), (unsigned long long)v[0] | ((unsigned long long)v[1] << 32),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 template <bool COH>
 __device__ __forceinline__ unsigned ld4(const void *base, int byte_off) {
   if constexpr (COH) return __builtin_amdgcn_raw_buffer_load_b32(make_rsrc(base), byte_off, 0, kAuxSc1);

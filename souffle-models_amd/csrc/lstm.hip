@@ -73,7 +73,7 @@ __global__ void __launch_bounds__(256) k_lstm(Args a) {
       u2 p;
       int spin = 0;
       do {
-        p = ld8<true>(below, (t * HID + tid) * 8);
+        p = ld8_atomic(below + (size_t)t * HID + tid);
       } while (p[1] != (unsigned)(t + 1) && ++spin < kMaxSpin);
       failed |= spin >= kMaxSpin;
       v0 = __uint_as_float(p[0]);
@@ -82,7 +82,7 @@ __global__ void __launch_bounds__(256) k_lstm(Args a) {
       u2 p;
       int spin = 0;
       do {
-        p = ld8<true>(own, ((t - 1) * HID + tid) * 8);
+        p = ld8_atomic(own + (size_t)(t - 1) * HID + tid);
       } while (p[1] != (unsigned)t && ++spin < kMaxSpin);
       failed |= spin >= kMaxSpin;
       v1 = __uint_as_float(p[0]);
@@ -112,7 +112,7 @@ __global__ void __launch_bounds__(256) k_lstm(Args a) {
       // (cpp/lstm/lstm_reuse_shared_memory.cu:309-318)
       cstate = cstate * sigmoidf_(pf + a.forget_bias) + sigmoidf_(pi) * tanhf_(pg);
       const float h = tanhf_(cstate) * sigmoidf_(po);
-      st8<true>(own, (t * HID + unit) * 8, u2{__float_as_uint(h), (unsigned)(t + 1)});
+      st8_atomic(own + (size_t)t * HID + unit, u2{__float_as_uint(h), (unsigned)(t + 1)});
       if (l == a.layers - 1) a.y[(size_t)t * HID + unit] = h;
     }
   }
@@ -122,7 +122,7 @@ __global__ void __launch_bounds__(256) k_lstm(Args a) {
   grid_sync(bar);
   for (int i = tid; i < a.timesteps * UNITS_PER_WG; i += 256) {
     const int t = i / UNITS_PER_WG, u = g * UNITS_PER_WG + i % UNITS_PER_WG;
-    st8<true>(own, (t * HID + u) * 8, u2{0u, 0u});
+    st8_atomic(own + (size_t)t * HID + u, u2{0u, 0u});
   }
   grid_barrier_end(bar);
 }
