@@ -1,5 +1,145 @@
-// placeholder until the SE kernel lands
+// EfficientNet squeeze-excite module as one persistent cooperative kernel on gfx950.
+//
+// Replaces torch_dispatch_efficientnet_se_module_v2_short_cut_fused
+// (cpp/efficientnet/efficientnet_se_module_binding.cu:164-227) and its kernel
+// efficientnet_se_module_v2_short_cut_fused (cpp/efficientnet/kernels/se_module_global_fused.cu:318-444),
+// which uses three grid barriers and fixed per-shape launch tables.  Here a WAVE owns a
+// (channel, chunk) slice of the input, keeps it in registers from the pooling pass to the
+// final combine (x is read from HBM exactly once and y written once), and one grid
+// barrier separates the partial sums from the two tiny fully-connected layers, which every
+// workgroup evaluates for its own channels.  Any C, H*W, R within the limits below.
+#include "common.hpp"
 #include "host_util.hpp"
+
+namespace souffle {
+namespace se {
+
+constexpr int EPT = 8;        // elements per lane per unit
+constexpr int UPW = 2;        // units per wave
+constexpr int MAX_C = 2048, MAX_R = 64;
+
+struct Args {
+  int C, HW, R, chunks, combine;
+  const float *x, *w_reduce, *b_reduce, *w_expand, *b_expand;
+  float *y, *pooled, *part;
+  unsigned *ctl;
+};
+
+__global__ void __launch_bounds__(256) k_se(Args a) {
+  __shared__ float p_s[MAX_C];
+  __shared__ float r_s[MAX_R];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int gw = blockIdx.x * 4 + wave, nw = gridDim.x * 4;
+  const int units = a.C * a.chunks, slice = (a.HW + a.chunks - 1) / a.chunks;
+  GridBarrier bar;
+  grid_barrier_begin(bar, a.ctl);
+
+  float v[UPW][EPT];
+#pragma unroll
+  for (int k = 0; k < UPW; ++k) {
+    const int u = gw + k * nw;
+    float s = 0.f;
+    if (u < units) {
+      const int c = u / a.chunks, ch = u % a.chunks;
+      const int lo = ch * slice, hi = min(a.HW, lo + slice);
+      const float *src = a.x + (size_t)c * a.HW;
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) {
+        const int e = lo + lane + 64 * i;
+        v[k][i] = e < hi ? src[e] : 0.f;
+        s += v[k][i];
+      }
+      s = wave_sum(s);
+      if (lane == 0) st4<true>(a.part, u * 4, __float_as_uint(s));
+    }
+  }
+  grid_sync(bar);
+
+  // pooled mean of every channel (all workgroups need all of it for the reduce layer)
+  for (int c = tid; c < a.C; c += 256) {
+    float s = 0.f;
+    for (int ch = 0; ch < a.chunks; ++ch) s += __uint_as_float(ld4<true>(a.part, (c * a.chunks + ch) * 4));
+    s *= 1.0f / a.HW;
+    p_s[c] = s;
+    if (blockIdx.x == 0 && a.pooled) a.pooled[c] = s;
+  }
+  __syncthreads();
+  // r = swish(W_r p + b_r)
+  for (int j = wave; j < a.R; j += 4) {
+    float s = 0.f;
+    for (int c = lane; c < a.C; c += 64) s += a.w_reduce[(size_t)j * a.C + c] * p_s[c];
+    s = wave_sum(s);
+    if (a.b_reduce) s += a.b_reduce[j];
+    if (lane == 0) r_s[j] = s / (1.0f + __expf(-s));
+  }
+  __syncthreads();
+  // e = sigmoid(W_e r + b_e) for this wave's channels, then combine with the held slice
+#pragma unroll
+  for (int k = 0; k < UPW; ++k) {
+    const int u = gw + k * nw;
+    if (u < units) {
+      const int c = u / a.chunks, ch = u % a.chunks;
+      float s = lane < a.R ? a.w_expand[(size_t)c * a.R + lane] * r_s[lane] : 0.f;
+      s = wave_sum(s);
+      if (a.b_expand) s += a.b_expand[c];
+      const float e = 1.0f / (1.0f + __expf(-s));
+      const int lo = ch * slice, hi = min(a.HW, lo + slice);
+      float *dst = a.y + (size_t)c * a.HW;
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) {
+        const int idx = lo + lane + 64 * i;
+        if (idx < hi) dst[idx] = a.combine == SOUFFLE_SE_ADD ? v[k][i] + e : v[k][i] * e;
+      }
+    }
+  }
+  grid_barrier_end(bar);
+}
+
+static int plan(int C, int HW, int R, int num_cus, int *chunks) {
+  if (C <= 0 || HW <= 0 || R <= 0) return fail(SOUFFLE_ERR_SHAPE, "C, HW and R must be positive");
+  if (C > MAX_C || R > MAX_R) return fail(SOUFFLE_ERR_SHAPE, "C <= %d and R <= %d required (got %d, %d)", MAX_C, MAX_R, C, R);
+  const int waves = num_cus * 4;
+  // smallest chunk count whose slices fit a wave's registers, then as many as the waves allow
+  int ch = (HW + 64 * EPT - 1) / (64 * EPT);
+  while ((long long)C * (ch + 1) <= waves && (HW + ch) / (ch + 1) >= 64) ++ch;
+  if ((long long)C * ch > (long long)waves * UPW)
+    return fail(SOUFFLE_ERR_SHAPE, "input of %d x %d elements exceeds the register-resident limit of %d", C, HW, waves * UPW * 64 * EPT);
+  *chunks = ch;
+  return SOUFFLE_OK;
+}
+
+}  // namespace se
+}  // namespace souffle
+
 using namespace souffle;
-extern "C" size_t souffle_se_workspace_bytes(int, int, int) { return 0; }
-extern "C" int souffle_se_module_fused(const float *, const float *, const float *, const float *, const float *, float *, float *, int, int, int, int, void *, size_t, souffle_stream_t) { return fail(SOUFFLE_ERR_UNSUPPORTED, "se module is not built yet"); }
+
+extern "C" size_t souffle_se_workspace_bytes(int C, int HW, int R) {
+  int chunks = 0;
+  if (se::plan(C, HW, R, 256, &chunks)) return 0;
+  // sized for any CU count: partial sums of at most 2048 (channel, chunk) units
+  return round_up(kCtlWords * 4, 256) + 4 * 4096;
+}
+
+extern "C" int souffle_se_module_fused(const float *x, const float *w_reduce, const float *b_reduce, const float *w_expand,
+                                       const float *b_expand, float *y, float *pooled, int C, int HW, int R, int combine,
+                                       void *ws, size_t ws_bytes, souffle_stream_t stream) {
+  if (!x || !w_reduce || !w_expand || !y) return fail(SOUFFLE_ERR_NULL, "x, w_reduce, w_expand and y must not be NULL");
+  if (combine != SOUFFLE_SE_MUL && combine != SOUFFLE_SE_ADD) return fail(SOUFFLE_ERR_SHAPE, "unknown combine op %d", combine);
+  if (C <= 0 || HW <= 0 || R <= 0 || C > se::MAX_C || R > se::MAX_R)
+    return fail(SOUFFLE_ERR_SHAPE, "need 0 < C <= %d, 0 < R <= %d, HW > 0 (got %d, %d, %d)", se::MAX_C, se::MAX_R, C, R, HW);
+  const size_t need = round_up(kCtlWords * 4, 256) + 4 * 4096;
+  if (!ws || ws_bytes < need) return fail(SOUFFLE_ERR_WORKSPACE, "workspace missing or too small: need %zu bytes", need);
+  if (!aligned16(ws)) return fail(SOUFFLE_ERR_ALIGN, "workspace must be 16-byte aligned");
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  if (!df.cooperative) return fail(SOUFFLE_ERR_DEVICE, "device does not support cooperative launch");
+  int chunks = 0;
+  if (int rc = se::plan(C, HW, R, df.num_cus, &chunks)) return rc;
+  if ((long long)C * chunks > 4096) return fail(SOUFFLE_ERR_SHAPE, "too many (channel, chunk) units");
+  se::Args a{C, HW, R, chunks, combine, x, w_reduce, b_reduce, w_expand, b_expand, y, pooled,
+             reinterpret_cast<float *>(static_cast<char *>(ws) + round_up(kCtlWords * 4, 256)), static_cast<unsigned *>(ws)};
+  void *args[] = {&a};
+  SOUFFLE_HIP_TRY(hipLaunchCooperativeKernel((const void *)se::k_se, dim3(df.num_cus), dim3(256), args, 0,
+                                             static_cast<hipStream_t>(stream)));
+  return SOUFFLE_OK;
+}

@@ -1,0 +1,118 @@
+"""swin_transformer_binding: drop-in for the reference's pybind module of the same name
+(cpp/swin_transformer/swin_transformer_binding.cu:276-289), reduced to a wrapper over the
+C ABI, plus the Swin block pair the reference only has as TVM operator definitions.
+
+Reference functions kept (same positional arguments and return values):
+    swin_fused_feed_mlp(src, fc1_weight, fc2_weight) -> [fc1_output, fc2_output]
+    bench_swin_fused_feed_mlp(src, fc1_weight, fc2_weight, num_warmup, repeat, num_bench) -> us
+    swin_ffn(src, weight, M, N, K) -> Tensor[M,N]
+    bench_swin_ffn(M, N, K, num_warmup, num_bench, repeat) -> us
+New: swin_block_pair(x, block0, block1, ...) and index_maps(height, width, window, shift).
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+import souffle_hip as sh
+
+_workspaces = {}
+
+
+def _ws(key, nbytes, device):
+    ws = _workspaces.get((key, device))
+    if ws is None or ws.nbytes < nbytes:
+        ws = _workspaces[(key, device)] = sh.Workspace(nbytes, device)
+    return ws
+
+
+def _check(name, t, shape=None):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError("%s must be a CUDA tensor" % name)           # reference: CHECK_CUDA
+    if t.dtype != torch.float16 or not t.is_contiguous():
+        raise TypeError("%s must be a contiguous float16 tensor" % name)
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError("%s must have shape %s, got %s" % (name, tuple(shape), tuple(t.shape)))
+
+
+def swin_fused_feed_mlp(src, fc1_weight, fc2_weight):
+    """Y1 = src.W1, Y2 = Y1.W2 in one cooperative launch (no bias, no activation), as
+    cpp/swin_transformer/swin_transformer_binding.cu:154-209 (there fixed to 256x512x2048)."""
+    _check("src", src)
+    M, K = src.shape[-2], src.shape[-1]
+    _check("fc1_weight", fc1_weight)
+    Fd = fc1_weight.shape[1]
+    _check("fc1_weight", fc1_weight, (K, Fd))
+    _check("fc2_weight", fc2_weight, (Fd, K))
+    ws = _ws("ffn", 16384 + 32 * M * K, src.device)
+    y1 = torch.empty((M, Fd), dtype=torch.float16, device=src.device)
+    y2 = torch.empty((M, K), dtype=torch.float16, device=src.device)
+    sh.check(sh.lib().souffle_swin_ffn_fused(src.data_ptr(), fc1_weight.data_ptr(), fc2_weight.data_ptr(),
+                                             y1.data_ptr(), y2.data_ptr(), M, K, Fd, ws.ptr, ws.nbytes,
+                                             sh.current_stream()))
+    return [y1, y2]
+
+
+def bench_swin_fused_feed_mlp(src, fc1_weight, fc2_weight, num_warmup, repeat, num_bench):
+    """Latency in us under the reference's rule (cpp/swin_transformer/swin_transformer_binding.cu:213-219)."""
+    mn, _ = sh.bench_us(lambda: swin_fused_feed_mlp(src, fc1_weight, fc2_weight), num_warmup, num_bench, repeat)
+    return mn
+
+
+def swin_ffn(src, weight, M, N, K):
+    """Y[M,N] = src[M,K].weight[K,N] (cpp/swin_transformer/swin_transformer_binding.cu:62-100)."""
+    _check("src", src)
+    _check("weight", weight, (K, N))
+    if src.numel() != M * K:
+        raise ValueError("src must have M*K elements")
+    y = torch.empty((M, N), dtype=torch.float16, device=src.device)
+    sh.check(sh.lib().souffle_gemm_f16(src.data_ptr(), weight.data_ptr(), y.data_ptr(), M, N, K, sh.current_stream()))
+    return y
+
+
+def bench_swin_ffn(M, N, K, num_warmup, num_bench, repeat):
+    src = torch.randn((M, K), device="cuda:0").half()
+    weight = (torch.randn((K, N), device="cuda:0") * 0.02).half()
+    mn, _ = sh.bench_us(lambda: swin_ffn(src, weight, M, N, K), num_warmup, num_bench, repeat)
+    return mn
+
+
+BLOCK_KEYS = sh.SWIN_W_FIELDS
+
+
+def _block_w(w):
+    for k in ("w_qkv", "w_proj", "w_fc1", "w_fc2"):
+        _check(k, w[k])
+    for k, v in w.items():
+        if k not in BLOCK_KEYS:
+            raise KeyError("unknown block weight %r" % k)
+        _check(k, v)
+    s = sh.SwinBlockW(*[sh.ptr(w.get(k)) for k in BLOCK_KEYS])
+    s._keep = w
+    return s
+
+
+def swin_block_pair(x, block0, block1, height=56, width=56, heads=4, window=7, shift=3, mlp_ratio=4,
+                    use_shift_mask=True, ln_eps=1e-5):
+    """Regular-window block followed by shifted-window block (Swin-Base stage 1 by default).
+    x: [H*W, C] fp16.  block0/block1: dicts with the keys of souffle_swin_block_w."""
+    _check("x", x, (height * width, x.shape[-1]))
+    cfg = sh.SwinCfg(height, width, x.shape[-1], heads, window, shift, mlp_ratio, int(use_shift_mask), float(ln_eps))
+    nbytes = sh.lib().souffle_swin_workspace_bytes(C.byref(cfg))
+    if nbytes == 0:
+        raise sh.SouffleError(-2, sh.last_error())
+    ws = _ws(("pair", height, width), nbytes, x.device)
+    arr = (sh.SwinBlockW * 2)(_block_w(block0), _block_w(block1))
+    y = torch.empty_like(x)
+    sh.check(sh.lib().souffle_swin_block_pair_fused(C.byref(cfg), arr, x.data_ptr(), y.data_ptr(), ws.ptr, ws.nbytes,
+                                                    sh.current_stream()))
+    return y
+
+
+def index_maps(height, width, window, shift):
+    """(gather_idx, scatter_idx, relpos_idx[N,N], region_id) as int32 numpy arrays (host computation)."""
+    T, N = height * width, window * window
+    g, s, r, reg = (np.empty(T, np.int32), np.empty(T, np.int32), np.empty(N * N, np.int32), np.empty(T, np.int32))
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    sh.check(sh.lib().souffle_swin_index_maps(height, width, window, shift, p(g), p(s), p(r), p(reg)))
+    return g, s, r.reshape(N, N), reg
