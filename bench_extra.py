@@ -1,7 +1,139 @@
-"""Secondary bench workloads (LSTM, Swin) selected with bench.py --workload."""
+"""Secondary bench workloads selected with bench.py --workload {lstm,swin,se,layer_stages}.
+Each prints the same JSON shape as the default workload."""
+import os
 import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def _cpu_time(fn, budget_s):
+    fn()
+    n, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        n += 1
+        if time.perf_counter() - t0 > budget_s or n >= 50:
+            break
+    return (time.perf_counter() - t0) / n * 1e6, n
+
+
+def _threads():
+    try:
+        return min(len(os.sched_getaffinity(0)), 16)
+    except Exception:
+        return min(os.cpu_count() or 1, 16)
+
+
+def _base(metric, value_us, args, workload, dtype, roof, extra):
+    return {"metric": metric, "value": value_us, "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": value_us / 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+            "dtype": dtype, "data": "synthetic", "config": {"workload": workload}, "roofline": roof, "extra": extra}
+
+
+def bench_lstm(args):
+    import numpy as np
+    import torch
+    import lstm_binding
+    import synth
+    from bench import time_steps
+    w_ih, w_hh, x = synth.lstm_tensors(1)
+    d = lambda a, t: torch.from_numpy(a).to("cuda:0", dtype=t).contiguous()
+    dx, dwi, dwh = d(x, torch.float32).view(1, 100, 256), d(w_ih, torch.float16), d(w_hh, torch.float16)
+    y = lstm_binding.fused_lstm(dx, dwi, dwh)[0].cpu().numpy()
+    res_cpu = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle
+        ref = oracle.lstm(x, w_ih, w_hh)
+        dd = np.abs(y - ref)
+        if not (dd.max() <= 2e-2 and dd.mean() <= 2e-3):
+            print("PARITY FAILURE (lstm): %g %g" % (dd.max(), dd.mean()), file=sys.stderr)
+            sys.exit(1)
+        us, n = _cpu_time(lambda: oracle.lstm(x, w_ih, w_hh), min(args.cpu_seconds, 8.0))
+        res_cpu = {"value": us, "unit": "us", "cores": 1, "kind": "port",
+                   "sample": "%d passes of the 10x256 T=100 stack through oracle/lstm_oracle.c (scalar fp32)" % n}
+    wall, ev = time_steps(lambda i: lstm_binding.fused_lstm(dx, dwi, dwh), args.steps, args.warmup)
+    bytes_alg = 5242880 * 2 + 2 * 51200 * 2
+    ach = bytes_alg / (ev * 1e-3) / 1e9
+    roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
+            "kernel": "k_lstm", "algorithmic_bytes_per_launch": bytes_alg, "avg_launch_us": ev * 1e3,
+            "note": "109 dependent wavefront steps bound the latency, not the one-time 10.5 MB weight stream"}
+    res = _base("lstm_stack_latency_us", wall * 1e3, args, "stacked LSTM 10x256, T=100, batch 1 (BASELINE configs[1])", "f16",
+                roof, {"us_per_wavefront_step": ev * 1e3 / 109})
+    if res_cpu:
+        res["cpu_baseline"] = res_cpu
+    return res
+
+
+def bench_swin(args):
+    import numpy as np
+    import torch
+    import swin_transformer_binding as sb
+    import synth
+    from bench import time_steps
+    ws = [synth.swin_block_weights(3, b) for b in range(2)]
+    x = synth.swin_input(3)
+    dw = [{k: torch.from_numpy(v).cuda() for k, v in w.items()} for w in ws]
+    dx = torch.from_numpy(x).cuda()
+    y = sb.swin_block_pair(dx, dw[0], dw[1]).float().cpu().numpy()
+    res_cpu = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle
+        ref = oracle.swin_block_pair(x, ws)
+        dd = np.abs(y - ref)
+        if not (dd.max() <= 2e-2 and dd.mean() <= 2e-3):
+            print("PARITY FAILURE (swin): %g %g" % (dd.max(), dd.mean()), file=sys.stderr)
+            sys.exit(1)
+        thr = _threads()
+        us, n = _cpu_time(lambda: oracle.swin_block_pair(x, ws, threads=thr), min(args.cpu_seconds, 8.0))
+        res_cpu = {"value": us, "unit": "us", "cores": thr, "kind": "port",
+                   "sample": "%d passes of the 56x56x128 block pair through oracle/swin_oracle.c (OpenMP fp32)" % n}
+    wall, ev = time_steps(lambda i: sb.swin_block_pair(dx, dw[0], dw[1]), args.steps, args.warmup)
+    flops = 2 * (2.0 * 3136 * 196608 + 4.0 * 64 * 4 * 49 * 49 * 32)
+    ach = flops / (ev * 1e-3) / 1e12
+    roof = {"bound": "mfma", "achieved": ach, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": ach / MFMA_F16_PEAK_TFLOPS,
+            "traffic": None, "kernel": "k_block_pair", "algorithmic_flops_per_launch": flops, "avg_launch_us": ev * 1e3}
+    res = _base("swin_block_pair_latency_us", wall * 1e3, args,
+                "Swin-Base stage-1 block pair 56x56, C=128, 4 heads, window 7, shift 3 (BASELINE configs[3])", "f16", roof, {})
+    if res_cpu:
+        res["cpu_baseline"] = res_cpu
+    return res
+
+
+def bench_se(args):
+    import torch
+    import efficientnet_se_module_binding as eb
+    from bench import time_steps
+    shapes = [(32, 112, 8), (96, 56, 4), (144, 56, 6), (144, 28, 6), (240, 28, 10), (240, 14, 10), (480, 14, 20),
+              (672, 14, 28), (672, 7, 28), (1152, 7, 48)]
+    a100 = [23.33, 14.14, 15.65, 12.48, 12.86, 12.03, 12.86, 13.86, 13.28, 15.36]   # reference xlsx, A100
+    rows = []
+    for (Cc, Hh, R), ref_us in zip(shapes, a100):
+        x = torch.rand((1, Cc, Hh, Hh), device="cuda:0")
+        wr, we = torch.randn((R, Cc), device="cuda:0") * 0.3, torch.randn((Cc, R), device="cuda:0") * 0.3
+        wall, ev = time_steps(lambda i: eb.torch_dispatch_efficientnet_se_module_v2_short_cut_fused(x, wr, we, 2, combine="add"),
+                              args.steps, args.warmup)
+        rows.append({"C": Cc, "H": Hh, "R": R, "us": ev * 1e3, "reference_a100_us": ref_us,
+                     "GBps": 2.0 * Cc * Hh * Hh * 4 / (ev * 1e-3) / 1e9})
+    tot = sum(r["us"] for r in rows)
+    byt = sum(2.0 * r["C"] * r["H"] ** 2 * 4 for r in rows)
+    ach = byt / (tot * 1e-6) / 1e9
+    roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
+            "kernel": "k_se", "avg_launch_us": tot / len(rows)}
+    return _base("se_module_latency_us_sum_of_10_shapes", tot, args, "EfficientNet-B0 SE module, the reference's 10 shapes, fp32", "f32",
+                 roof, {"per_shape": rows, "reference_a100_sum_us": sum(a100)})
 
 
 def run(args):
+    if args.workload == "lstm":
+        return bench_lstm(args)
+    if args.workload == "swin":
+        return bench_swin(args)
+    if args.workload == "se":
+        return bench_se(args)
     print("unknown workload %r" % args.workload, file=sys.stderr)
     sys.exit(2)

@@ -57,6 +57,13 @@ int souffle_device_info(souffle_devinfo *out);
  * (cpp/bert/bert_binding.cu:32-78). */
 int souffle_workspace_init(void *workspace, size_t workspace_bytes, souffle_stream_t stream);
 
+/* In-kernel stage timestamps.  Replaces the profile_clock tensors the reference's fused
+ * kernels fill with clock64() per (stage, block, warp) (cpp/bert/bert_binding.cu:67-76,111-114).
+ * While a buffer is set, every persistent kernel stamps the 100 MHz wall clock on entry to and
+ * exit from each of its grid barriers: uint64 buf[(2*i + {0,1}) * grid + block] for barrier i.
+ * Pass NULL to switch tracing off (the default). */
+int souffle_set_stage_trace(void *device_buf, size_t bytes);
+
 /* ------------------------------------------------------------------ BERT ---- */
 enum { SOUFFLE_ACT_GELU_TANH = 0, SOUFFLE_ACT_RELU = 1 };
 

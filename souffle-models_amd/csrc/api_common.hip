@@ -44,6 +44,13 @@ int device_facts(DeviceFacts *out) {
   return SOUFFLE_OK;
 }
 
+static void *g_trace_buf = nullptr;
+static size_t g_trace_bytes = 0;
+void stage_trace(unsigned long long **buf, int *max_barriers, int nblk) {
+  *buf = static_cast<unsigned long long *>(g_trace_buf);
+  *max_barriers = g_trace_buf ? (int)(g_trace_bytes / ((size_t)nblk * 16)) : 0;
+}
+
 __global__ void k_zero_words(unsigned *p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0u;
@@ -98,6 +105,13 @@ extern "C" int souffle_device_info(souffle_devinfo *out) {
   out->cooperative_launch = p.cooperativeLaunch;
   out->wavefront_size = p.warpSize;
   strncpy(out->arch, p.gcnArchName, sizeof(out->arch) - 1);
+  return SOUFFLE_OK;
+}
+
+extern "C" int souffle_set_stage_trace(void *device_buf, size_t bytes) {
+  if (device_buf && !aligned16(device_buf)) return fail(SOUFFLE_ERR_ALIGN, "trace buffer must be 16-byte aligned");
+  g_trace_buf = device_buf;
+  g_trace_bytes = device_buf ? bytes : 0;
   return SOUFFLE_OK;
 }
 

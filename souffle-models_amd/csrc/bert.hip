@@ -13,6 +13,7 @@
 // Softmax is max-subtracted fp32 and LayerNorm is two-pass fp32 in registers, with a
 // fixed summation order (no float atomics), so results are run-to-run identical.
 #include <type_traits>
+#include "gemm_oneshot.hpp"
 #include "gemm_tile.hpp"
 #include "host_util.hpp"
 
@@ -35,6 +36,8 @@ struct Args {
   half_t *qkv, *ctx, *y1, *h, *xa, *xb, *probs;
   float *part;
   unsigned *ctl;
+  unsigned long long *trace;
+  int trace_cap;
   LayerW layers[kMaxLayers];
 };
 
@@ -97,19 +100,30 @@ __device__ __forceinline__ void stage_partial(half_t *lds, const Args &a, const 
 }
 
 // out[m] = LN(sum_ks part[ks][m] + bias + resid[m]) * g + b; one wave per row.
-template <bool COH>
-__device__ __forceinline__ void stage_ln(const Args &a, int splitk, const half_t *bias, const half_t *resid,
+template <bool COH, int SPLITK>
+__device__ __forceinline__ void stage_ln_t(const Args &a, const half_t *bias, const half_t *resid,
                                          const half_t *gam, const half_t *bet, half_t *out,
                                          int first_row, int row_stride) {
   const int lane = threadIdx.x & 63;
   for (int m = first_row; m < a.M; m += row_stride) {
     f4 v[3];
+    u4 raw[3][SPLITK];
+    u2 rres[3];
+    // every load of the row is issued before the first use
 #pragma unroll
     for (int c = 0; c < 3; ++c) {
       const int n = c * 256 + lane * 4;
-      f4 s = __builtin_bit_cast(f4, ld16<COH>(a.part, (m * H + n) * 4));
-      for (int ks = 1; ks < splitk; ++ks) s += __builtin_bit_cast(f4, ld16<COH>(a.part, ((ks * a.M + m) * H + n) * 4));
-      const h4 r = as_h4(ld8<COH>(resid, (m * H + n) * 2));
+#pragma unroll
+      for (int ks = 0; ks < SPLITK; ++ks) raw[c][ks] = ld16<COH>(a.part, ((ks * a.M + m) * H + n) * 4);
+      rres[c] = ld8<COH>(resid, (m * H + n) * 2);
+    }
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      const int n = c * 256 + lane * 4;
+      f4 s = __builtin_bit_cast(f4, raw[c][0]);
+#pragma unroll
+      for (int ks = 1; ks < SPLITK; ++ks) s += __builtin_bit_cast(f4, raw[c][ks]);
+      const h4 r = as_h4(rres[c]);
       s += f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
       if (bias) {
         const h4 bb = *reinterpret_cast<const h4 *>(bias + n);
@@ -146,52 +160,165 @@ __device__ __forceinline__ void stage_ln(const Args &a, int splitk, const half_t
   }
 }
 
+// ---- skinny (small M) variants: one-shot operand loads, see gemm_oneshot.hpp ----
+using OsFull = GemmOneShot<32, 768>;    // QKV, FC1: whole K in one shot
+using OsOut = GemmOneShot<32, 256>;     // out-projection: 3 K slices as fp32 partials
+using OsFc2 = GemmOneShot<64, 384>;     // FC2: 8 K slices as fp32 partials
+constexpr int kSplitOutSmall = H / OsOut::kKS, kSplitFc2Small = F / OsFc2::kKS;
+
+// Workgroups are dealt to the eight XCDs round-robin (block b runs on XCD b % 8, each XCD
+// has its own L2).  The m-tiles that share one weight slice are therefore given to
+// workgroups of ONE XCD in the same pass, so that the slice crosses the HBM -> L2 link once
+// and the other readers hit (or merge in) that L2.
+// Calls body(m_tile, weight_slice) for this workgroup's items.
+template <class Body>
+__device__ __forceinline__ void for_items_xcd(int m_tiles, int w_slices, Body body) {
+  if ((gridDim.x & 7) == 0) {
+    const int xcd = blockIdx.x & 7, nloc = gridDim.x >> 3, groups = (w_slices + 7) >> 3;
+    for (int j = blockIdx.x >> 3; j < groups * m_tiles; j += nloc) {
+      const int ws = (j / m_tiles) * 8 + xcd;
+      if (ws < w_slices) body(j % m_tiles, ws);
+    }
+  } else {
+    for (int it = blockIdx.x; it < m_tiles * w_slices; it += gridDim.x) body(it % m_tiles, it / m_tiles);
+  }
+}
+
+template <bool COH>
+__device__ __forceinline__ void stage_qkv_os(unsigned char *lds, const Args &a, const LayerW &w, const half_t *xin,
+                                             int first, int stride) {
+  using G = OsFull;
+  for_items_xcd(a.M / G::kBM, 3 * H / 64, [&](int mt, int nt) {
+    const int m0 = mt * G::kBM, n0 = nt * 64, j = n0 / H, nn0 = n0 % H;
+    __syncthreads();
+    G::issue_w(lds + G::X_BYTES, w.w_qkv + (size_t)j * H * H, H, nn0, 0);
+    G::template issue_x<COH>(lds, xin, H, m0, 0);
+    G::wait_loads();
+    G::compute(lds, lds + G::X_BYTES, [&](int mm, int nn, f4 v) {
+      const int m = m0 + mm, n = nn0 + nn;
+      if (w.b_qkv) {
+        const h4 bb = *reinterpret_cast<const h4 *>(w.b_qkv + j * H + n);
+        v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+      }
+      const int b = m / a.S, s = m % a.S, hh = n / HD, d = n % HD;
+      st8<COH>(a.qkv, ((((j * a.B + b) * NH + hh) * a.S + s) * HD + d) * 2, pack_h4(v));
+    });
+  });
+}
+
+template <bool COH>
+__device__ __forceinline__ void stage_fc1_os(unsigned char *lds, const Args &a, const LayerW &w, int first, int stride) {
+  using G = OsFull;
+  for_items_xcd(a.M / G::kBM, F / 64, [&](int mt, int nt) {
+    const int m0 = mt * G::kBM, n0 = nt * 64;
+    __syncthreads();
+    G::issue_w(lds + G::X_BYTES, w.w_fc1, F, n0, 0);
+    G::template issue_x<COH>(lds, a.y1, H, m0, 0);
+    G::wait_loads();
+    G::compute(lds, lds + G::X_BYTES, [&](int mm, int nn, f4 v) {
+      const int m = m0 + mm, n = n0 + nn;
+      if (w.b_fc1) {
+        const h4 bb = *reinterpret_cast<const h4 *>(w.b_fc1 + n);
+        v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(v[i], 0.f) : gelu_tanh(v[i]);
+      st8<COH>(a.h, (m * F + n) * 2, pack_h4(v));
+    });
+  });
+}
+
+template <bool COH, class G>
+__device__ __forceinline__ void stage_partial_os(unsigned char *lds, const Args &a, const half_t *X, int K,
+                                                 const half_t *W, int first, int stride) {
+  const int splitk = K / G::kKS;
+  for_items_xcd(a.M / G::kBM, (H / 64) * splitk, [&](int mt, int ws) {
+    const int ks = ws % splitk, m0 = mt * G::kBM, n0 = (ws / splitk) * 64;
+    __syncthreads();
+    G::issue_w(lds + G::X_BYTES, W, H, n0, ks * G::kKS);
+    G::template issue_x<COH>(lds, X, K, m0, ks * G::kKS);
+    G::wait_loads();
+    G::compute(lds, lds + G::X_BYTES, [&](int mm, int nn, f4 v) {
+      st16<COH>(a.part, ((ks * a.M + m0 + mm) * H + n0 + nn) * 4, __builtin_bit_cast(u4, v));
+    });
+  });
+}
+
+template <bool COH>
+__device__ __forceinline__ void stage_ln(const Args &a, int splitk, const half_t *bias, const half_t *resid,
+                                         const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
+  if (splitk == 1) stage_ln_t<COH, 1>(a, bias, resid, gam, bet, out, first_row, row_stride);
+  else if (splitk == kSplitOutSmall) stage_ln_t<COH, kSplitOutSmall>(a, bias, resid, gam, bet, out, first_row, row_stride);
+  else stage_ln_t<COH, kSplitFc2Small>(a, bias, resid, gam, bet, out, first_row, row_stride);
+}
+
 // One (batch, head, 64-query block) per workgroup pass; each wave owns 16 queries.
 // Scores are computed transposed (keys x queries) so that the softmax reduction over
 // keys is in-lane plus two cross-lane steps, and the probabilities are already in the
 // B-operand layout of the 16x16x16 MFMA used for P.V.  V is staged row-major in LDS
 // and read through the transposing LDS load.
-constexpr int kVLD = HD + 8;
+// Direct global->LDS load of a [rows][64] fp16 tile (128-byte rows = 8 slots of 16 bytes),
+// swizzled for its reader: MODE 0 for b128 operand reads of 16 consecutive rows
+// (slot ^= (row >> 1) & 7), MODE 1 for the transposing read of 4 consecutive rows (slot ^= row & 2).
+template <bool COH, int MODE>
+__device__ __forceinline__ void issue_rows64(unsigned char *lds, const half_t *src, int rows) {
+  typedef __attribute__((address_space(1))) const void *gptr_t;
+  typedef __attribute__((address_space(3))) void *lptr_t;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int inst = wave; inst < rows / 8; inst += 4) {
+    const int sl = inst * 64 + lane, r = sl >> 3, c = (sl & 7) ^ (MODE == 0 ? ((r >> 1) & 7) : (r & 2));
+    __builtin_amdgcn_global_load_lds((gptr_t)(src + (size_t)r * HD + c * 8), (lptr_t)(lds + inst * 1024), 16, 0, COH ? kAuxSc1 : 0);
+  }
+}
+
 template <bool COH, int NKT>
-__device__ __forceinline__ void attn_item(half_t *lds, const Args &a, int item) {
+__device__ __forceinline__ void attn_item(half_t *lds_h, const Args &a, int item) {
   constexpr int S = NKT * 16;
+  unsigned char *lds = reinterpret_cast<unsigned char *>(lds_h);
+  unsigned char *ks_ = lds, *vs_ = lds + S * 128, *qs_ = lds + 2 * S * 128;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
   const int qblocks = S / 64;
   const int qb = item % qblocks, bh = item / qblocks, b = bh / NH, hh = bh % NH;
   const int head_off = ((b * NH + hh) * S) * HD;                 // halves, within one of q/k/v
-  const int plane = a.B * NH * S * HD;
-  const half_t *Q = a.qkv, *K = a.qkv + plane, *V = a.qkv + 2 * (size_t)plane;
+  const size_t plane = (size_t)a.B * NH * S * HD;
+  const half_t *Q = a.qkv + head_off + (size_t)qb * 64 * HD, *K = a.qkv + plane + head_off, *V = a.qkv + 2 * plane + head_off;
 
   __syncthreads();   // LDS reuse
-  for (int id = tid; id < S * HD / 8; id += 256) {
-    const int r = id / (HD / 8), c = (id % (HD / 8)) * 8;
-    *reinterpret_cast<u4 *>(lds + r * kVLD + c) = ld16<COH>(V, (head_off + r * HD + c) * 2);
-  }
-  const int q0 = qb * 64 + wave * 16;
-  h8 qop[2];
-#pragma unroll
-  for (int ks = 0; ks < 2; ++ks) qop[ks] = as_h8(ld16<COH>(Q, (head_off + (q0 + l16) * HD + ks * 32 + g * 8) * 2));
+  issue_rows64<COH, 0>(ks_, K, S);
+  issue_rows64<COH, 1>(vs_, V, S);
+  issue_rows64<COH, 0>(qs_, Q, 64);
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
 
+  const half_t *kh = reinterpret_cast<const half_t *>(ks_), *vh = reinterpret_cast<const half_t *>(vs_),
+               *qh = reinterpret_cast<const half_t *>(qs_);
+  const int q0 = qb * 64 + wave * 16, q = q0 + l16;
+  h8 qop[2];
+  {
+    const int r = wave * 16 + l16;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) qop[ks] = *reinterpret_cast<const h8 *>(qh + (r * 8 + ((ks * 4 + g) ^ ((r >> 1) & 7))) * 8);
+  }
   f4 sc[NKT];
 #pragma unroll
   for (int t = 0; t < NKT; ++t) {
-    const h8 k0 = as_h8(ld16<COH>(K, (head_off + (t * 16 + l16) * HD + g * 8) * 2));
-    const h8 k1 = as_h8(ld16<COH>(K, (head_off + (t * 16 + l16) * HD + 32 + g * 8) * 2));
+    const int r = t * 16 + l16, sw = (r >> 1) & 7;
+    const h8 k0 = *reinterpret_cast<const h8 *>(kh + (r * 8 + (g ^ sw)) * 8);
+    const h8 k1 = *reinterpret_cast<const h8 *>(kh + (r * 8 + ((4 + g) ^ sw)) * 8);
     f4 c = mfma_16x16x32(k0, qop[0], f4{0.f, 0.f, 0.f, 0.f});
     sc[t] = mfma_16x16x32(k1, qop[1], c);
   }
   // sc[t][v] = score(key = 16t + 4g + v, query = q0 + l16)
-  const int q = q0 + l16;
   float mx = -INFINITY;
 #pragma unroll
   for (int t = 0; t < NKT; ++t) {
-    f4 s = sc[t] * a.scale;
+    f4 sv = sc[t] * a.scale;
     if (a.mask) {
       const h4 mk = *reinterpret_cast<const h4 *>(a.mask + ((size_t)b * S + q) * S + t * 16 + g * 4);
-      s += f4{(float)mk[0], (float)mk[1], (float)mk[2], (float)mk[3]};
+      sv += f4{(float)mk[0], (float)mk[1], (float)mk[2], (float)mk[3]};
     }
-    sc[t] = s;
-    mx = fmaxf(mx, fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+    sc[t] = sv;
+    mx = fmaxf(mx, fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
   }
   mx = fmaxf(mx, wave_xor(mx, 16));
   mx = fmaxf(mx, wave_xor(mx, 32));
@@ -212,15 +339,16 @@ __device__ __forceinline__ void attn_item(half_t *lds, const Args &a, int item) 
     if (a.probs)
       st8<false>(a.probs, (int)((((size_t)(b * NH + hh) * S + q) * S + t * 16 + g * 4) * 2), as_u2(p[t]));
   }
-  __syncthreads();   // V tile is in LDS
   f4 o[HD / 16];
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) o[dt] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int t = 0; t < NKT; ++t) {
+    const int kr = t * 16 + g * 4 + (l16 >> 2);
 #pragma unroll
     for (int dt = 0; dt < HD / 16; ++dt) {
-      const h4 vop = lds_read_tr16(lds + (t * 16 + g * 4 + (l16 >> 2)) * kVLD + dt * 16 + (l16 & 3) * 4);
+      const int c = dt * 2 + ((l16 & 3) >> 1);
+      const h4 vop = lds_read_tr16(vh + (kr * 8 + (c ^ (kr & 2))) * 8 + (l16 & 1) * 4);
       o[dt] = mfma_16x16x16(vop, p[t], o[dt]);
     }
   }
@@ -246,9 +374,10 @@ __device__ __forceinline__ void stage_attn(half_t *lds, const Args &a, int first
 
 using TileSmall = GemmTile<64, 64, 64, 2, 2>;
 using TileLarge = GemmTile<128, 128, 64, 2, 2>;
-constexpr int kAttnLdsBytes = 512 * kVLD * 2;
+constexpr int kAttnLdsBytes = 2 * 512 * 128 + 64 * 128;
+constexpr int kSmallGemmLds = OsFull::LDS_BYTES > OsFc2::LDS_BYTES ? OsFull::LDS_BYTES : OsFc2::LDS_BYTES;
 constexpr int lds_bytes(bool large) {
-  const int t = large ? TileLarge::LDS_BYTES : TileSmall::LDS_BYTES;
+  const int t = large ? TileLarge::LDS_BYTES : kSmallGemmLds;
   return t > kAttnLdsBytes ? t : kAttnLdsBytes;
 }
 
@@ -260,23 +389,29 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args a) {
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
   GridBarrier bar;
   grid_barrier_begin(bar, a.ctl);
+  bar.trace = a.trace;
+  bar.trace_cap = a.trace_cap;
   const int first = blockIdx.x, stride = gridDim.x;
   const int wave = threadIdx.x >> 6;
   const half_t *xin = a.x;
   for (int l = 0; l < a.num_layers; ++l) {
     const LayerW &w = a.layers[l];
     half_t *yout = (l == a.num_layers - 1) ? a.y : ((l & 1) ? a.xb : a.xa);
-    stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
+    if constexpr (LARGE) stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
+    else stage_qkv_os<true>(lds_raw, a, w, xin, first, stride);
     grid_sync(bar);
     stage_attn<true>(lds, a, first, stride);
     grid_sync(bar);
-    stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
+    if constexpr (LARGE) stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
+    else stage_partial_os<true, OsOut>(lds_raw, a, a.ctx, H, w.w_o, first, stride);
     grid_sync(bar);
     stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
     grid_sync(bar);
-    stage_fc1<true, Tile>(lds, a, w, first, stride);
+    if constexpr (LARGE) stage_fc1<true, Tile>(lds, a, w, first, stride);
+    else stage_fc1_os<true>(lds_raw, a, w, first, stride);
     grid_sync(bar);
-    stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
+    if constexpr (LARGE) stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
+    else stage_partial_os<true, OsFc2>(lds_raw, a, a.h, F, w.w_fc2, first, stride);
     grid_sync(bar);
     stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
     if (l + 1 < a.num_layers) grid_sync(bar);
@@ -290,7 +425,8 @@ template <bool LARGE>
 __global__ void __launch_bounds__(256) k_qkv(Args a, int l, const half_t *xin) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
-  stage_qkv<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], xin, blockIdx.x, gridDim.x);
+  if constexpr (LARGE) stage_qkv<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], xin, blockIdx.x, gridDim.x);
+  else stage_qkv_os<false>(lds_raw, a, a.layers[l], xin, blockIdx.x, gridDim.x);
 }
 __global__ void __launch_bounds__(256) k_attn(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -300,7 +436,9 @@ template <bool LARGE>
 __global__ void __launch_bounds__(256) k_partial(Args a, const half_t *X, int K, const half_t *W, int splitk) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
-  stage_partial<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, X, K, W, splitk, blockIdx.x, gridDim.x);
+  if constexpr (LARGE) stage_partial<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, X, K, W, splitk, blockIdx.x, gridDim.x);
+  else if (K == H) stage_partial_os<false, OsOut>(lds_raw, a, X, K, W, blockIdx.x, gridDim.x);
+  else stage_partial_os<false, OsFc2>(lds_raw, a, X, K, W, blockIdx.x, gridDim.x);
 }
 __global__ void __launch_bounds__(256) k_ln(Args a, int splitk, const half_t *bias, const half_t *resid,
                                             const half_t *gam, const half_t *bet, half_t *out) {
@@ -310,7 +448,8 @@ template <bool LARGE>
 __global__ void __launch_bounds__(256) k_fc1(Args a, int l) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
-  stage_fc1<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], blockIdx.x, gridDim.x);
+  if constexpr (LARGE) stage_fc1<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], blockIdx.x, gridDim.x);
+  else stage_fc1_os<false>(lds_raw, a, a.layers[l], blockIdx.x, gridDim.x);
 }
 
 // ------------------------------------------------------------------- host ----
@@ -340,8 +479,8 @@ static Plan make_plan(const souffle_bert_cfg *c) {
   Plan p;
   const size_t M = (size_t)c->batch * c->seq_len;
   p.large = M >= 1024;
-  p.splitk_o = p.large ? 1 : 4;
-  p.splitk_f = p.large ? 1 : 8;
+  p.splitk_o = p.large ? 1 : kSplitOutSmall;
+  p.splitk_f = p.large ? 1 : kSplitFc2Small;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += round_up(bytes, 256); return o; };
   p.off_ctl = take(kCtlWords * 4);
@@ -378,6 +517,8 @@ static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_laye
   a.xb = reinterpret_cast<half_t *>(base + p.off_xb);
   a.part = reinterpret_cast<float *>(base + p.off_part);
   a.probs = nullptr;
+  a.trace = nullptr;
+  a.trace_cap = 0;
   if (dump) {   // the per-stage tensors are produced in the reference's own layouts: write them in place
     if (dump->qkv) a.qkv = static_cast<half_t *>(dump->qkv);
     if (dump->ctx) a.ctx = static_cast<half_t *>(dump->ctx);
@@ -424,35 +565,36 @@ static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *laye
   const Plan p = make_plan(c);
   static thread_local Args a;
   if (int rc = fill_args(a, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
+  stage_trace(&a.trace, &a.trace_cap, df.num_cus);
   hipStream_t st = static_cast<hipStream_t>(stream);
   return p.large ? launch_mega<true>(a, df.num_cus, st) : launch_mega<false>(a, df.num_cus, st);
 }
 
 template <bool LARGE>
 static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
-  using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
-  constexpr int BM = LARGE ? 128 : 64, BN = LARGE ? 128 : 64;
+  constexpr int GEMM_LDS = LARGE ? TileLarge::LDS_BYTES : kSmallGemmLds;
+  constexpr int BN = LARGE ? 128 : 64;
+  constexpr int BM_QKV = LARGE ? 128 : OsFull::kBM, BM_OUT = LARGE ? 128 : OsOut::kBM, BM_FC2 = LARGE ? 128 : OsFc2::kBM;
   static bool attr_done = false;
   if (!attr_done) {
-    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_qkv<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES));
-    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_partial<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES));
-    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_fc1<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_qkv<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_partial<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_fc1<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_attn, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLdsBytes));
     attr_done = true;
   }
   const int cap = num_cus * 4;
   auto grid_for = [&](int items) { return items < cap ? items : cap; };
-  const int tm = a.M / BM;
   const half_t *xin = a.x;
   for (int l = 0; l < nl; ++l) {
     const LayerW &w = a.layers[l];
     half_t *yout = (l == nl - 1) ? a.y : ((l & 1) ? a.xb : a.xa);
-    hipLaunchKernelGGL(k_qkv<LARGE>, dim3(grid_for(tm * (3 * H / BN))), dim3(256), Tile::LDS_BYTES, st, a, l, xin);
-    hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), a.S * kVLD * 2, st, a);
-    hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for(tm * (H / BN) * a.splitk_o)), dim3(256), Tile::LDS_BYTES, st, a, a.ctx, H, w.w_o, a.splitk_o);
+    hipLaunchKernelGGL(k_qkv<LARGE>, dim3(grid_for((a.M / BM_QKV) * (3 * H / BN))), dim3(256), GEMM_LDS, st, a, l, xin);
+    hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), 2 * a.S * 128 + 64 * 128, st, a);
+    hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for((a.M / BM_OUT) * (H / BN) * a.splitk_o)), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, a.splitk_o);
     hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
-    hipLaunchKernelGGL(k_fc1<LARGE>, dim3(grid_for(tm * (F / BN))), dim3(256), Tile::LDS_BYTES, st, a, l);
-    hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for(tm * (H / BN) * a.splitk_f)), dim3(256), Tile::LDS_BYTES, st, a, a.h, F, w.w_fc2, a.splitk_f);
+    hipLaunchKernelGGL(k_fc1<LARGE>, dim3(grid_for((a.M / BM_QKV) * (F / BN))), dim3(256), GEMM_LDS, st, a, l);
+    hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for((a.M / BM_FC2) * (H / BN) * a.splitk_f)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, a.splitk_f);
     hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout);
     xin = yout;
   }

@@ -145,12 +145,19 @@ struct GridBarrier {
   unsigned gen;    // meaningful in thread 0 only
   unsigned nblk;
   int down;        // 0: counts run up on the next barrier, 1: down
+  // optional stage trace: thread 0 stamps the 100 MHz wall clock on entry to and exit from
+  // every barrier: trace[(2*i + {0,1}) * nblk + block] for the i-th barrier of the launch
+  unsigned long long *trace;
+  int trace_idx, trace_cap;
 };
 
 __device__ __forceinline__ void grid_barrier_begin(GridBarrier &b, unsigned *ctl) {
   b.ctl = ctl;
   b.nblk = gridDim.x;
   b.down = 0;
+  b.trace = nullptr;
+  b.trace_idx = 0;
+  b.trace_cap = 0;
   // Read before this workgroup's first arrival: the generation cannot advance until
   // every workgroup has arrived, so all workgroups read the same value.
   b.gen = __hip_atomic_load(ctl + 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -170,6 +177,8 @@ __device__ __forceinline__ bool grid_arrive(GridBarrier &b) {
 }
 
 __device__ __forceinline__ void grid_sync(GridBarrier &b) {
+  const bool tr = b.trace && b.trace_idx < b.trace_cap && threadIdx.x == 0;
+  if (tr) b.trace[(size_t)(2 * b.trace_idx) * b.nblk + blockIdx.x] = wall_clock64();
   __builtin_amdgcn_s_waitcnt(0);   // this wave's write-through stores are acknowledged
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -182,6 +191,8 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b) {
     }
   }
   b.down ^= 1;
+  if (tr) b.trace[(size_t)(2 * b.trace_idx + 1) * b.nblk + blockIdx.x] = wall_clock64();
+  b.trace_idx++;
   __syncthreads();
 }
 

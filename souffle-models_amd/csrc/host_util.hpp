@@ -23,6 +23,9 @@ struct DeviceFacts {
 // Cached per process for the current device; returns a negative status on failure.
 int device_facts(DeviceFacts *out);
 
+// Process-wide stage-trace buffer set by souffle_set_stage_trace (NULL = tracing off).
+void stage_trace(unsigned long long **buf, int *max_barriers, int nblk);
+
 inline size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 #define SOUFFLE_HIP_TRY(expr)                                                            \

@@ -66,6 +66,7 @@ SIGNATURES = {
     "souffle_last_error": (C.c_char_p, []),
     "souffle_version": (C.c_char_p, []),
     "souffle_device_info": (C.c_int, [C.POINTER(DevInfo)]),
+    "souffle_set_stage_trace": (C.c_int, [C.c_void_p, C.c_size_t]),
     "souffle_workspace_init": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "souffle_bert_workspace_bytes": (C.c_size_t, [C.POINTER(BertCfg)]),
     "souffle_bert_layer_fused": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
@@ -150,6 +151,14 @@ class Workspace:
     @property
     def ptr(self):
         return self.buf.data_ptr()
+
+
+def set_stage_trace(tensor):
+    """Point the in-kernel stage trace at an int64 CUDA tensor (None = off)."""
+    if tensor is None:
+        check(lib().souffle_set_stage_trace(None, 0))
+    else:
+        check(lib().souffle_set_stage_trace(tensor.data_ptr(), tensor.numel() * tensor.element_size()))
 
 
 def device_info():
