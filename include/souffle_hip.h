@@ -60,8 +60,9 @@ int souffle_workspace_init(void *workspace, size_t workspace_bytes, souffle_stre
 /* In-kernel stage timestamps.  Replaces the profile_clock tensors the reference's fused
  * kernels fill with clock64() per (stage, block, warp) (cpp/bert/bert_binding.cu:67-76,111-114).
  * While a buffer is set, every persistent kernel stamps the 100 MHz wall clock on entry to and
- * exit from each of its grid barriers: uint64 buf[(2*i + {0,1}) * grid + block] for barrier i.
- * Pass NULL to switch tracing off (the default). */
+ * exit from each of its grid barriers: uint64 buf[(2*i + {0,1}) * grid + block] for barrier i,
+ * i < cap = bytes / (grid * 80); up to 8 marks inside the stage before barrier i follow at
+ * buf[(2*cap + 8*i + id) * grid + block].  Pass NULL to switch tracing off (the default). */
 int souffle_set_stage_trace(void *device_buf, size_t bytes);
 
 /* ------------------------------------------------------------------ BERT ---- */

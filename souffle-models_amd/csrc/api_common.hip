@@ -48,7 +48,7 @@ static void *g_trace_buf = nullptr;
 static size_t g_trace_bytes = 0;
 void stage_trace(unsigned long long **buf, int *max_barriers, int nblk) {
   *buf = static_cast<unsigned long long *>(g_trace_buf);
-  *max_barriers = g_trace_buf ? (int)(g_trace_bytes / ((size_t)nblk * 16)) : 0;
+  *max_barriers = g_trace_buf ? (int)(g_trace_bytes / ((size_t)nblk * 80)) : 0;   // 2 stamps + 8 marks per barrier
 }
 
 __global__ void k_zero_words(unsigned *p, int n) {

@@ -33,7 +33,7 @@ struct Args {
   float scale, eps;
   const half_t *x, *mask;
   half_t *y;
-  half_t *qkv, *ctx, *y1, *h, *xa, *xb, *probs;
+  half_t *qkv, *ctx, *z1, *y1, *h, *xa, *xb, *probs;
   float *part;
   unsigned *ctl;
   unsigned long long *trace;
@@ -160,96 +160,194 @@ __device__ __forceinline__ void stage_ln_t(const Args &a, const half_t *bias, co
   }
 }
 
-// ---- skinny (small M) variants: one-shot operand loads, see gemm_oneshot.hpp ----
-using OsFull = GemmOneShot<32, 768>;    // QKV, FC1: whole K in one shot
-using OsOut = GemmOneShot<32, 256>;     // out-projection: 3 K slices as fp32 partials
+// ---- skinny (small M) path: one-shot operand loads, see gemm_oneshot.hpp ----
+using OsFull = GemmOneShot<32, 768>;    // QKV, out-projection, FC1: whole K in one shot
 using OsFc2 = GemmOneShot<64, 384>;     // FC2: 8 K slices as fp32 partials
-constexpr int kSplitOutSmall = H / OsOut::kKS, kSplitFc2Small = F / OsFc2::kKS;
+constexpr int kSplitFc2Small = F / OsFc2::kKS;
+constexpr int kXRegion = 49152;         // LDS: [0, 48 KB) X slice / attention tiles / reduction, [48 KB, 144 KB) W slice
+static_assert(OsFull::X_BYTES <= kXRegion && OsFc2::X_BYTES <= kXRegion, "X region");
+constexpr int kSmallGemmLds = kXRegion + (OsFull::W_BYTES > OsFc2::W_BYTES ? OsFull::W_BYTES : OsFc2::W_BYTES);
 
-// Workgroups are dealt to the eight XCDs round-robin (block b runs on XCD b % 8, each XCD
-// has its own L2).  The m-tiles that share one weight slice are therefore given to
-// workgroups of ONE XCD in the same pass, so that the slice crosses the HBM -> L2 link once
-// and the other readers hit (or merge in) that L2.
-// Calls body(m_tile, weight_slice) for this workgroup's items.
-template <class Body>
-__device__ __forceinline__ void for_items_xcd(int m_tiles, int w_slices, Body body) {
-  if ((gridDim.x & 7) == 0) {
-    const int xcd = blockIdx.x & 7, nloc = gridDim.x >> 3, groups = (w_slices + 7) >> 3;
-    for (int j = blockIdx.x >> 3; j < groups * m_tiles; j += nloc) {
-      const int ws = (j / m_tiles) * 8 + xcd;
-      if (ws < w_slices) body(j % m_tiles, ws);
-    }
-  } else {
-    for (int it = blockIdx.x; it < m_tiles * w_slices; it += gridDim.x) body(it % m_tiles, it / m_tiles);
+// One work item of a skinny GEMM stage: output tile origin, weight slice, activation slice.
+struct Item {
+  int m0, n0;           // output rows / columns of the tile (n0 relative to `W`'s own column space)
+  const half_t *W;      // weight matrix the slice comes from
+  int ldw, k0;          // its row pitch, first row of the K slice
+  int aux;              // stage specific (q/k/v index, K-slice index)
+};
+
+// Items are dealt m-tile fastest: the workgroups that share a weight slice are neighbours,
+// i.e. sit on different XCDs, so no L2 sees the same line requested twice at once.
+struct QkvItems {
+  const half_t *w_qkv; int M;
+  __device__ int count() const { return (M / OsFull::kBM) * (3 * H / 64); }
+  __device__ Item at(int it) const {
+    const int mt = M / OsFull::kBM, n0 = (it / mt) * 64, j = n0 / H;
+    return Item{(it % mt) * OsFull::kBM, n0 % H, w_qkv + (size_t)j * H * H, H, 0, j};
+  }
+};
+struct OutItems {
+  const half_t *w_o; int M;
+  __device__ int count() const { return (M / OsFull::kBM) * (H / 64); }
+  __device__ Item at(int it) const { const int mt = M / OsFull::kBM; return Item{(it % mt) * OsFull::kBM, (it / mt) * 64, w_o, H, 0, 0}; }
+};
+struct Fc1Items {
+  const half_t *w_fc1; int M;
+  __device__ int count() const { return (M / OsFull::kBM) * (F / 64); }
+  __device__ Item at(int it) const { const int mt = M / OsFull::kBM; return Item{(it % mt) * OsFull::kBM, (it / mt) * 64, w_fc1, F, 0, 0}; }
+};
+struct Fc2Items {
+  const half_t *w_fc2; int M;
+  __device__ int count() const { return (M / OsFc2::kBM) * (H / 64) * kSplitFc2Small; }
+  __device__ Item at(int it) const {
+    const int mt = M / OsFc2::kBM, ws = it / mt, ks = ws % kSplitFc2Small;
+    return Item{(it % mt) * OsFc2::kBM, (ws / kSplitFc2Small) * 64, w_fc2, H, ks * OsFc2::kKS, ks};
+  }
+};
+struct NoItems {
+  __device__ int count() const { return 0; }
+  __device__ Item at(int) const { return Item{0, 0, nullptr, 0, 0, 0}; }
+};
+
+// Queue the weight slice of this workgroup's first item of a stage (if it has one).
+template <class G, class Items>
+__device__ __forceinline__ bool preissue_w(unsigned char *lds, const Items &items) {
+  if ((int)blockIdx.x >= items.count()) return false;
+  const Item d = items.at(blockIdx.x);
+  G::issue_w(lds + kXRegion, d.W, d.ldw, d.n0, d.k0);
+  return true;
+}
+
+// Driver of a skinny GEMM stage.  `w_ready`: the weight slice of this workgroup's first item
+// was queued before the preceding grid barrier.  `pre(item)` runs after the operands have
+// landed (LayerNorm on load), `epi(item, m, n, v)` receives 4 consecutive columns of a row,
+// `next()` queues the first weight slice of the FOLLOWING stage as soon as the W region is free.
+template <class G, bool COH, class Items, class Pre, class Epi, class Next>
+__device__ __forceinline__ void gemm_stage(unsigned char *lds, const Items &items, const half_t *X, int ldx, bool w_ready,
+                                           Pre pre, Epi epi, Next next) {
+  const int n = items.count();
+  int it = blockIdx.x;
+  if (it >= n) { next(); return; }
+  for (; it < n; it += gridDim.x) {
+    const Item d = items.at(it);
+    __syncthreads();                       // LDS reuse
+    if (!w_ready) G::issue_w(lds + kXRegion, d.W, d.ldw, d.n0, d.k0);
+    G::template issue_x<COH>(lds, X, ldx, d.m0, d.k0);
+    G::wait_loads();
+    pre(d);
+    const bool last = it + (int)gridDim.x >= n;
+    G::compute(lds, lds + kXRegion, [&]() { if (last) next(); }, [&](int mm, int nn, f4 v) { epi(d, d.m0 + mm, d.n0 + nn, v); });
+    w_ready = false;
   }
 }
 
-template <bool COH>
-__device__ __forceinline__ void stage_qkv_os(unsigned char *lds, const Args &a, const LayerW &w, const half_t *xin,
-                                             int first, int stride) {
-  using G = OsFull;
-  for_items_xcd(a.M / G::kBM, 3 * H / 64, [&](int mt, int nt) {
-    const int m0 = mt * G::kBM, n0 = nt * 64, j = n0 / H, nn0 = n0 % H;
-    __syncthreads();
-    G::issue_w(lds + G::X_BYTES, w.w_qkv + (size_t)j * H * H, H, nn0, 0);
-    G::template issue_x<COH>(lds, xin, H, m0, 0);
-    G::wait_loads();
-    G::compute(lds, lds + G::X_BYTES, [&](int mm, int nn, f4 v) {
-      const int m = m0 + mm, n = nn0 + nn;
-      if (w.b_qkv) {
-        const h4 bb = *reinterpret_cast<const h4 *>(w.b_qkv + j * H + n);
-        v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
-      }
-      const int b = m / a.S, s = m % a.S, hh = n / HD, d = n % HD;
-      st8<COH>(a.qkv, ((((j * a.B + b) * NH + hh) * a.S + s) * HD + d) * 2, pack_h4(v));
-    });
-  });
+__device__ __forceinline__ f4 add_bias4(f4 v, const half_t *bias, int n) {
+  if (bias) {
+    const h4 bb = *reinterpret_cast<const h4 *>(bias + n);
+    v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+  }
+  return v;
 }
 
+// LayerNorm of the 32 complete rows of an OsFull X tile, in place in LDS.  Eight lanes
+// share a row; slot s of row r holds columns 8*(s ^ (r & 15)) .. +7.  Statistics and the
+// normalisation (one FMA per element) are fp32.  When `out` is given the normalised rows are also written to out[m0 + r][:].
 template <bool COH>
-__device__ __forceinline__ void stage_fc1_os(unsigned char *lds, const Args &a, const LayerW &w, int first, int stride) {
-  using G = OsFull;
-  for_items_xcd(a.M / G::kBM, F / 64, [&](int mt, int nt) {
-    const int m0 = mt * G::kBM, n0 = nt * 64;
-    __syncthreads();
-    G::issue_w(lds + G::X_BYTES, w.w_fc1, F, n0, 0);
-    G::template issue_x<COH>(lds, a.y1, H, m0, 0);
-    G::wait_loads();
-    G::compute(lds, lds + G::X_BYTES, [&](int mm, int nn, f4 v) {
-      const int m = m0 + mm, n = n0 + nn;
-      if (w.b_fc1) {
-        const h4 bb = *reinterpret_cast<const h4 *>(w.b_fc1 + n);
-        v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
-      }
+__device__ __forceinline__ void ln_rows_in_lds(unsigned char *lds_x, const half_t *gam, const half_t *bet, float eps,
+                                               half_t *out, int m0) {
+  constexpr int XGR = OsFull::XGR, PER = XGR / 8;
+  const int tid = threadIdx.x, r = tid >> 3, t8 = tid & 7;
+  h8 *row = reinterpret_cast<h8 *>(lds_x) + r * XGR;
+  float f[PER][8];
+  float sum = 0.f, sq = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(v[i], 0.f) : gelu_tanh(v[i]);
-      st8<COH>(a.h, (m * F + n) * 2, pack_h4(v));
-    });
-  });
-}
-
-template <bool COH, class G>
-__device__ __forceinline__ void stage_partial_os(unsigned char *lds, const Args &a, const half_t *X, int K,
-                                                 const half_t *W, int first, int stride) {
-  const int splitk = K / G::kKS;
-  for_items_xcd(a.M / G::kBM, (H / 64) * splitk, [&](int mt, int ws) {
-    const int ks = ws % splitk, m0 = mt * G::kBM, n0 = (ws / splitk) * 64;
-    __syncthreads();
-    G::issue_w(lds + G::X_BYTES, W, H, n0, ks * G::kKS);
-    G::template issue_x<COH>(lds, X, K, m0, ks * G::kKS);
-    G::wait_loads();
-    G::compute(lds, lds + G::X_BYTES, [&](int mm, int nn, f4 v) {
-      st16<COH>(a.part, ((ks * a.M + m0 + mm) * H + n0 + nn) * 4, __builtin_bit_cast(u4, v));
-    });
-  });
+  for (int i = 0; i < PER; ++i) {
+    const h8 x = row[t8 + 8 * i];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      f[i][e] = (float)x[e];
+      sum += f[i][e];
+      sq += f[i][e] * f[i][e];
+    }
+  }
+  sum += wave_xor(sum, 1); sum += wave_xor(sum, 2); sum += wave_xor(sum, 4);
+  sq += wave_xor(sq, 1); sq += wave_xor(sq, 2); sq += wave_xor(sq, 4);
+  // one-pass variance in fp32: the rows are residual sums with |mean| well below the
+  // standard deviation, so E[x^2] - mean^2 loses no significant digits
+  const float mean = sum * (1.0f / H);
+  const float var = fmaxf(sq * (1.0f / H) - mean * mean, 0.f);
+  const float rstd = rsqrtf(var + eps), shift = -mean * rstd;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int sl = t8 + 8 * i, k = (sl ^ (r & 15)) * 8;
+    h8 o;
+    if (gam || bet) {
+      h8 g8, b8;
+      if (gam) g8 = *reinterpret_cast<const h8 *>(gam + k);
+      if (bet) b8 = *reinterpret_cast<const h8 *>(bet + k);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float t = f[i][e] * rstd + shift;
+        if (gam) t *= (float)g8[e];
+        if (bet) t += (float)b8[e];
+        o[e] = (half_t)t;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (half_t)(f[i][e] * rstd + shift);
+    }
+    row[sl] = o;
+    if (out) st16<COH>(out, ((m0 + r) * H + k) * 2, as_u4(o));
+  }
+  __syncthreads();
 }
 
 template <bool COH>
 __device__ __forceinline__ void stage_ln(const Args &a, int splitk, const half_t *bias, const half_t *resid,
                                          const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
   if (splitk == 1) stage_ln_t<COH, 1>(a, bias, resid, gam, bet, out, first_row, row_stride);
-  else if (splitk == kSplitOutSmall) stage_ln_t<COH, kSplitOutSmall>(a, bias, resid, gam, bet, out, first_row, row_stride);
   else stage_ln_t<COH, kSplitFc2Small>(a, bias, resid, gam, bet, out, first_row, row_stride);
+}
+
+// The four skinny GEMM stages (shared by the megakernel and the per-op kernels).
+template <bool COH, class Next>
+__device__ __forceinline__ void small_qkv(unsigned char *lds, const Args &a, const LayerW &w, const half_t *xin, bool w_ready, Next next) {
+  gemm_stage<OsFull, COH>(lds, QkvItems{w.w_qkv, a.M}, xin, H, w_ready, [](const Item &) {},
+    [&](const Item &d, int m, int n, f4 v) {
+      v = add_bias4(v, w.b_qkv ? w.b_qkv + d.aux * H : nullptr, n);
+      const int b = m / a.S, s = m % a.S, hh = n / HD, dd = n % HD;
+      st8<COH>(a.qkv, ((((d.aux * a.B + b) * NH + hh) * a.S + s) * HD + dd) * 2, pack_h4(v));
+    }, next);
+}
+// z1 = ctx.Wo + b_o + x (pre-LayerNorm, fp16)
+template <bool COH, class Next>
+__device__ __forceinline__ void small_outproj(unsigned char *lds, const Args &a, const LayerW &w, const half_t *xin, bool w_ready, Next next) {
+  gemm_stage<OsFull, COH>(lds, OutItems{w.w_o, a.M}, a.ctx, H, w_ready, [](const Item &) {},
+    [&](const Item &, int m, int n, f4 v) {
+      v = add_bias4(v, w.b_o, n);
+      const h4 r = as_h4(ld8<COH>(xin, (m * H + n) * 2));
+      v += f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+      st8<COH>(a.z1, (m * H + n) * 2, pack_h4(v));
+    }, next);
+}
+// h = act(LN1(z1).W1 + b1): LayerNorm is applied to the X tile in LDS (every workgroup has
+// complete rows); the workgroups of the first n-tile also publish y1 = LN1(z1).
+template <bool COH, class Next>
+__device__ __forceinline__ void small_fc1(unsigned char *lds, const Args &a, const LayerW &w, bool w_ready, Next next) {
+  gemm_stage<OsFull, COH>(lds, Fc1Items{w.w_fc1, a.M}, a.z1, H, w_ready,
+    [&](const Item &d) { ln_rows_in_lds<COH>(lds, w.ln1_g, w.ln1_b, a.eps, d.n0 == 0 ? a.y1 : nullptr, d.m0); },
+    [&](const Item &, int m, int n, f4 v) {
+      v = add_bias4(v, w.b_fc1, n);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(v[i], 0.f) : gelu_tanh(v[i]);
+      st8<COH>(a.h, (m * F + n) * 2, pack_h4(v));
+    }, next);
+}
+// fp32 partials of h.W2 over 8 K slices
+template <bool COH, class Next>
+__device__ __forceinline__ void small_fc2(unsigned char *lds, const Args &a, const LayerW &w, bool w_ready, Next next) {
+  gemm_stage<OsFc2, COH>(lds, Fc2Items{w.w_fc2, a.M}, a.h, F, w_ready, [](const Item &) {},
+    [&](const Item &d, int m, int n, f4 v) { st16<COH>(a.part, ((d.aux * a.M + m) * H + n) * 4, __builtin_bit_cast(u4, v)); }, next);
 }
 
 // One (batch, head, 64-query block) per workgroup pass; each wave owns 16 queries.
@@ -375,7 +473,6 @@ __device__ __forceinline__ void stage_attn(half_t *lds, const Args &a, int first
 using TileSmall = GemmTile<64, 64, 64, 2, 2>;
 using TileLarge = GemmTile<128, 128, 64, 2, 2>;
 constexpr int kAttnLdsBytes = 2 * 512 * 128 + 64 * 128;
-constexpr int kSmallGemmLds = OsFull::LDS_BYTES > OsFc2::LDS_BYTES ? OsFull::LDS_BYTES : OsFc2::LDS_BYTES;
 constexpr int lds_bytes(bool large) {
   const int t = large ? TileLarge::LDS_BYTES : kSmallGemmLds;
   return t > kAttnLdsBytes ? t : kAttnLdsBytes;
@@ -394,26 +491,50 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args a) {
   const int first = blockIdx.x, stride = gridDim.x;
   const int wave = threadIdx.x >> 6;
   const half_t *xin = a.x;
+  bool qkv_ready = false;
   for (int l = 0; l < a.num_layers; ++l) {
-    const LayerW &w = a.layers[l];
+    const LayerW w = a.layers[l];
     half_t *yout = (l == a.num_layers - 1) ? a.y : ((l & 1) ? a.xb : a.xa);
-    if constexpr (LARGE) stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
-    else stage_qkv_os<true>(lds_raw, a, w, xin, first, stride);
-    grid_sync(bar);
-    stage_attn<true>(lds, a, first, stride);
-    grid_sync(bar);
-    if constexpr (LARGE) stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
-    else stage_partial_os<true, OsOut>(lds_raw, a, a.ctx, H, w.w_o, first, stride);
-    grid_sync(bar);
-    stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
-    grid_sync(bar);
-    if constexpr (LARGE) stage_fc1<true, Tile>(lds, a, w, first, stride);
-    else stage_fc1_os<true>(lds_raw, a, w, first, stride);
-    grid_sync(bar);
-    if constexpr (LARGE) stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
-    else stage_partial_os<true, OsFc2>(lds_raw, a, a.h, F, w.w_fc2, first, stride);
-    grid_sync(bar);
-    stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
+    if constexpr (LARGE) {
+      stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
+      grid_sync(bar);
+      stage_attn<true>(lds, a, first, stride);
+      grid_sync(bar);
+      stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
+      grid_sync(bar);
+      stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
+      grid_sync(bar);
+      stage_fc1<true, Tile>(lds, a, w, first, stride);
+      grid_sync(bar);
+      stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
+      grid_sync(bar);
+      stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
+    } else {
+      // Weight slices are queued one stage ahead: right after a stage's MFMA loop has
+      // released the W region, the slice of the next stage is requested, so it crosses HBM
+      // while the epilogue stores drain and the grid barrier is crossed.
+      const bool attn_fits = 2 * a.S * 128 + 64 * 128 <= kXRegion;   // attention tiles stay below the W region
+      const OutItems out_items{w.w_o, a.M};
+      const Fc1Items fc1_items{w.w_fc1, a.M};
+      const Fc2Items fc2_items{w.w_fc2, a.M};
+      bool out_ready = false;
+      small_qkv<true>(lds_raw, a, w, xin, qkv_ready, [&]() { if (attn_fits) out_ready = preissue_w<OsFull>(lds_raw, out_items); });
+      grid_sync(bar);
+      stage_attn<true>(lds, a, first, stride);
+      if (!attn_fits) { __syncthreads(); out_ready = preissue_w<OsFull>(lds_raw, out_items); }
+      grid_sync(bar);
+      bool fc1_ready = false, fc2_ready = false;
+      small_outproj<true>(lds_raw, a, w, xin, out_ready, [&]() { fc1_ready = preissue_w<OsFull>(lds_raw, fc1_items); });
+      grid_sync(bar);
+      small_fc1<true>(lds_raw, a, w, fc1_ready, [&]() { fc2_ready = preissue_w<OsFc2>(lds_raw, fc2_items); });
+      grid_sync(bar);
+      qkv_ready = false;
+      small_fc2<true>(lds_raw, a, w, fc2_ready, [&]() {
+        if (l + 1 < a.num_layers) qkv_ready = preissue_w<OsFull>(lds_raw, QkvItems{a.layers[l + 1].w_qkv, a.M});
+      });
+      grid_sync(bar);
+      stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
+    }
     if (l + 1 < a.num_layers) grid_sync(bar);
     xin = yout;
   }
@@ -426,7 +547,7 @@ __global__ void __launch_bounds__(256) k_qkv(Args a, int l, const half_t *xin) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
   if constexpr (LARGE) stage_qkv<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], xin, blockIdx.x, gridDim.x);
-  else stage_qkv_os<false>(lds_raw, a, a.layers[l], xin, blockIdx.x, gridDim.x);
+  else small_qkv<false>(lds_raw, a, a.layers[l], xin, false, []() {});
 }
 __global__ void __launch_bounds__(256) k_attn(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -437,8 +558,11 @@ __global__ void __launch_bounds__(256) k_partial(Args a, const half_t *X, int K,
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
   if constexpr (LARGE) stage_partial<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, X, K, W, splitk, blockIdx.x, gridDim.x);
-  else if (K == H) stage_partial_os<false, OsOut>(lds_raw, a, X, K, W, blockIdx.x, gridDim.x);
-  else stage_partial_os<false, OsFc2>(lds_raw, a, X, K, W, blockIdx.x, gridDim.x);
+  else {
+    LayerW w{};
+    w.w_fc2 = W;
+    small_fc2<false>(lds_raw, a, w, false, []() {});
+  }
 }
 __global__ void __launch_bounds__(256) k_ln(Args a, int splitk, const half_t *bias, const half_t *resid,
                                             const half_t *gam, const half_t *bet, half_t *out) {
@@ -449,14 +573,18 @@ __global__ void __launch_bounds__(256) k_fc1(Args a, int l) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
   if constexpr (LARGE) stage_fc1<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], blockIdx.x, gridDim.x);
-  else stage_fc1_os<false>(lds_raw, a, a.layers[l], blockIdx.x, gridDim.x);
+  else small_fc1<false>(lds_raw, a, a.layers[l], false, []() {});
+}
+__global__ void __launch_bounds__(256) k_outproj_small(Args a, int l, const half_t *xin) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  small_outproj<false>(lds_raw, a, a.layers[l], xin, false, []() {});
 }
 
 // ------------------------------------------------------------------- host ----
 struct Plan {
   bool large;
   int splitk_o, splitk_f;
-  size_t off_ctl, off_qkv, off_ctx, off_y1, off_h, off_xa, off_xb, off_part, total;
+  size_t off_ctl, off_qkv, off_ctx, off_z1, off_y1, off_h, off_xa, off_xb, off_part, total;
 };
 
 static int validate(const souffle_bert_cfg *c) {
@@ -479,13 +607,14 @@ static Plan make_plan(const souffle_bert_cfg *c) {
   Plan p;
   const size_t M = (size_t)c->batch * c->seq_len;
   p.large = M >= 1024;
-  p.splitk_o = p.large ? 1 : kSplitOutSmall;
+  p.splitk_o = 1;
   p.splitk_f = p.large ? 1 : kSplitFc2Small;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += round_up(bytes, 256); return o; };
   p.off_ctl = take(kCtlWords * 4);
   p.off_qkv = take(3 * M * H * 2);
   p.off_ctx = take(M * H * 2);
+  p.off_z1 = take(M * H * 2);
   p.off_y1 = take(M * H * 2);
   p.off_h = take(M * F * 2);
   p.off_xa = take(M * H * 2);
@@ -511,6 +640,7 @@ static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_laye
   a.ctl = reinterpret_cast<unsigned *>(base + p.off_ctl);
   a.qkv = reinterpret_cast<half_t *>(base + p.off_qkv);
   a.ctx = reinterpret_cast<half_t *>(base + p.off_ctx);
+  a.z1 = reinterpret_cast<half_t *>(base + p.off_z1);
   a.y1 = reinterpret_cast<half_t *>(base + p.off_y1);
   a.h = reinterpret_cast<half_t *>(base + p.off_h);
   a.xa = reinterpret_cast<half_t *>(base + p.off_xa);
@@ -574,13 +704,14 @@ template <bool LARGE>
 static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
   constexpr int GEMM_LDS = LARGE ? TileLarge::LDS_BYTES : kSmallGemmLds;
   constexpr int BN = LARGE ? 128 : 64;
-  constexpr int BM_QKV = LARGE ? 128 : OsFull::kBM, BM_OUT = LARGE ? 128 : OsOut::kBM, BM_FC2 = LARGE ? 128 : OsFc2::kBM;
+  constexpr int BM_QKV = LARGE ? 128 : OsFull::kBM, BM_OUT = LARGE ? 128 : OsFull::kBM, BM_FC2 = LARGE ? 128 : OsFc2::kBM;
   static bool attr_done = false;
   if (!attr_done) {
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_qkv<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_partial<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_fc1<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_attn, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLdsBytes));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_outproj_small, hipFuncAttributeMaxDynamicSharedMemorySize, kSmallGemmLds));
     attr_done = true;
   }
   const int cap = num_cus * 4;
@@ -591,8 +722,12 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     half_t *yout = (l == nl - 1) ? a.y : ((l & 1) ? a.xb : a.xa);
     hipLaunchKernelGGL(k_qkv<LARGE>, dim3(grid_for((a.M / BM_QKV) * (3 * H / BN))), dim3(256), GEMM_LDS, st, a, l, xin);
     hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), 2 * a.S * 128 + 64 * 128, st, a);
-    hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for((a.M / BM_OUT) * (H / BN) * a.splitk_o)), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, a.splitk_o);
-    hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
+    if (LARGE) {
+      hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, 1);
+      hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, 1, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
+    } else {   // small M: LN1 is applied by the FC1 kernel on its LDS-resident rows
+      hipLaunchKernelGGL(k_outproj_small, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, l, xin);
+    }
     hipLaunchKernelGGL(k_fc1<LARGE>, dim3(grid_for((a.M / BM_QKV) * (F / BN))), dim3(256), GEMM_LDS, st, a, l);
     hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for((a.M / BM_FC2) * (H / BN) * a.splitk_f)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, a.splitk_f);
     hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout);

@@ -127,53 +127,52 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 }
 
 // -------------------------------------------------------- grid barrier ----
-// Two-level arrival tree on relaxed agent-scope atomics plus a monotonic generation
-// word.  Control block (uint32 words, zeroed once before first use):
-//   [0]            root arrival count
-//   [32]           generation (monotonic; its start value is irrelevant)
-//   [64 + 32*g]    arrival count of group g, g < 64
-// Arrival counts run up on even barriers of a launch and down on odd ones, so no
-// count is ever reset (nothing to order against the release of the generation word).
-// grid_barrier_end() leaves every count at zero for the next launch.
+// One arrival counter per XCD (workgroup b runs on XCD b % 8 and adds 1 to counter b % 8
+// with a relaxed agent-scope atomic whose result is not awaited) and no release flag:
+// every workgroup polls all eight counters with one 8-lane load until each has reached its
+// target.  Counters only ever grow and are compared as signed differences, so a fast
+// workgroup arriving at the next barrier never disturbs a slow one that is still polling.
+// The critical path is one atomic on its way to memory plus one polling round trip.
+// Control block (uint32 words, zeroed once before first use):
+//   [32*x]        arrival counter of XCD x, x < 8 (one 128-byte line each)
+//   [256 + 32*x]  value counter x holds between launches; rewritten by grid_barrier_end()
+//                 (all workgroups read it before their first arrival, nobody writes it
+//                 before the last barrier of the launch has completed)
+//   [48]          sticky error flag for kernels with bounded spin loops
 // All data exchanged across a barrier must be written with st*<true> and read with
 // ld*<true>; the barrier itself carries no cache write-back or invalidate.
-constexpr int kBarGroup = 16;
-constexpr int kCtlWords = 64 + 32 * 64;
+constexpr int kCtlWords = 512;
+constexpr int kMaxBarrierSpin = 1 << 24;
 
 struct GridBarrier {
   unsigned *ctl;
-  unsigned gen;    // meaningful in thread 0 only
+  unsigned target;   // lane x < 8 of wave 0: value counter x reaches at the next barrier
+  unsigned gsz;      // lane x < 8 of wave 0: workgroups on XCD x
   unsigned nblk;
-  int down;        // 0: counts run up on the next barrier, 1: down
+  int count;         // barriers passed in this launch
   // optional stage trace: thread 0 stamps the 100 MHz wall clock on entry to and exit from
-  // every barrier: trace[(2*i + {0,1}) * nblk + block] for the i-th barrier of the launch
+  // every barrier: trace[(2*i + {0,1}) * nblk + block] for the i-th barrier of the launch,
+  // plus up to 8 free-form marks inside the stage that precedes barrier i:
+  // trace[(2*cap + 8*i + id) * nblk + block]
   unsigned long long *trace;
   int trace_idx, trace_cap;
 };
 
+__device__ __forceinline__ void trace_mark(const GridBarrier &b, int id) {
+  if (b.trace && b.trace_idx < b.trace_cap && threadIdx.x == 0)
+    b.trace[(size_t)(2 * b.trace_cap + 8 * b.trace_idx + id) * b.nblk + blockIdx.x] = wall_clock64();
+}
+
 __device__ __forceinline__ void grid_barrier_begin(GridBarrier &b, unsigned *ctl) {
   b.ctl = ctl;
   b.nblk = gridDim.x;
-  b.down = 0;
+  b.count = 0;
   b.trace = nullptr;
   b.trace_idx = 0;
   b.trace_cap = 0;
-  // Read before this workgroup's first arrival: the generation cannot advance until
-  // every workgroup has arrived, so all workgroups read the same value.
-  b.gen = __hip_atomic_load(ctl + 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Thread 0 only.  Returns true when this arrival completed the whole grid.
-__device__ __forceinline__ bool grid_arrive(GridBarrier &b) {
-  const unsigned grp = blockIdx.x / kBarGroup;
-  const unsigned ngrp = (b.nblk + kBarGroup - 1) / kBarGroup;
-  const unsigned gsz = min((unsigned)kBarGroup, b.nblk - grp * kBarGroup);
-  unsigned *gc = b.ctl + 64 + 32 * grp;
-  const unsigned inc = b.down ? 0xffffffffu : 1u;
-  const unsigned prev = __hip_atomic_fetch_add(gc, inc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (prev != (b.down ? 1u : gsz - 1)) return false;
-  const unsigned prev2 = __hip_atomic_fetch_add(b.ctl, inc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  return prev2 == (b.down ? 1u : ngrp - 1);
+  const unsigned x = threadIdx.x & 7;
+  b.gsz = (b.nblk + 7 - x) >> 3;
+  b.target = __hip_atomic_load(ctl + 256 + 32 * x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ void grid_sync(GridBarrier &b) {
@@ -181,16 +180,19 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b) {
   if (tr) b.trace[(size_t)(2 * b.trace_idx) * b.nblk + blockIdx.x] = wall_clock64();
   __builtin_amdgcn_s_waitcnt(0);   // this wave's write-through stores are acknowledged
   __syncthreads();
-  if (threadIdx.x == 0) {
-    b.gen++;
-    if (grid_arrive(b)) {
-      __hip_atomic_store(b.ctl + 32, b.gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    } else {
-      while ((int)(__hip_atomic_load(b.ctl + 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - b.gen) < 0)
-        __builtin_amdgcn_s_sleep(1);
+  b.target += b.gsz;
+  if (threadIdx.x < 64) {
+    if (threadIdx.x == 0)
+      (void)__hip_atomic_fetch_add(b.ctl + 32 * (blockIdx.x & 7), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int spin = 0; spin < kMaxBarrierSpin; ++spin) {
+      bool ok = true;
+      if (threadIdx.x < 8)
+        ok = (int)(__hip_atomic_load(b.ctl + 32 * threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - b.target) >= 0;
+      if (__all(ok)) break;
+      __builtin_amdgcn_s_sleep(1);
     }
   }
-  b.down ^= 1;
+  b.count++;
   if (tr) b.trace[(size_t)(2 * b.trace_idx + 1) * b.nblk + blockIdx.x] = wall_clock64();
   b.trace_idx++;
   __syncthreads();
@@ -198,10 +200,8 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b) {
 
 // Call once by every workgroup before the kernel returns.
 __device__ __forceinline__ void grid_barrier_end(GridBarrier &b) {
-  if (b.down) {            // odd number of barriers so far: run the counts back to zero
-    __syncthreads();
-    if (threadIdx.x == 0) (void)grid_arrive(b);
-  }
+  if (b.count > 0 && blockIdx.x < 8 && threadIdx.x == blockIdx.x)
+    __hip_atomic_store(b.ctl + 256 + 32 * blockIdx.x, b.target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace souffle

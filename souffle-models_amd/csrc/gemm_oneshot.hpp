@@ -1,18 +1,23 @@
 // "One-shot" fp16 MFMA GEMM item for skinny problems (few rows, weight-stream bound).
 //
 // A workgroup of 256 threads computes a BM x 64 tile of Y = X.W over a K slice of KS.
-// Both operand slices fit in LDS, so ALL of their loads are issued at once with the
-// direct global->LDS instruction (no register staging, ~100 KB in flight per CU): the item
-// costs one memory latency instead of one per K step.  This matters because at M = 128
-// every stage of the encoder is latency bound.
+// Both operand slices fit in LDS, so ALL of their loads are queued at once with the direct
+// global->LDS instruction (no register staging, ~100 KB in flight per CU): an item costs
+// one memory latency instead of one per K step, and the weight slice of the NEXT stage can
+// be queued before a grid barrier and land while the barrier is crossed.
 //
 // LDS layouts are unpadded (the direct load writes 64 consecutive 16-byte slots per wave
 // instruction) and XOR-swizzled at slot granularity instead:
-//   X slice [BM][KS]: slot(r, j) = r*KS/8 + (j ^ (r & 15))   16 rows of one k-granule -> 16 banks groups
+//   X slice [BM][KS]: slot(r, j) = r*KS/8 + (j ^ (r & 15))   16 rows of one k-granule -> 16 bank groups
 //   W slice [KS][64]: slot(k, c) = k*8    + (c ^ (k & 2))    4 rows of a transposing read -> 4 bank groups
 // W stays row-major [K][N] as the reference stores it; the k-vector operand comes from the
 // transposing LDS read.  The MFMA takes W as operand A and X as operand B so that a lane
 // holds 4 consecutive output columns of one row.
+//
+// The four waves split the tile as WAVES_M row blocks of 32 x WAVES_K slices of K; every
+// wave owns all 64 columns (8 independent accumulators, fully unrolled K loop), the K
+// slices are summed through a padded fp32 buffer in LDS, and the epilogue then runs with 8
+// or 16 consecutive columns of one row per thread.
 #pragma once
 #include "common.hpp"
 
@@ -21,14 +26,18 @@ namespace souffle {
 template <int BM, int KS>
 struct GemmOneShot {
   static_assert(KS % 128 == 0, "the X swizzle needs whole groups of 16 slots per row");
-  static_assert(BM == 32 || BM == 64 || BM == 128, "tile rows");
+  static_assert(BM == 32 || BM == 64, "tile rows");
   static constexpr int kBM = BM, kBN = 64, kKS = KS;
   static constexpr int XGR = KS / 8;                               // 16-byte slots per X row
   static constexpr int X_BYTES = BM * KS * 2, W_BYTES = KS * 64 * 2;
-  static constexpr int LDS_BYTES = X_BYTES + W_BYTES;
   static constexpr int X_INSTR = X_BYTES / 1024, W_INSTR = W_BYTES / 1024;   // wave-wide loads
-  static constexpr int WAVES_M = BM == 32 ? 1 : 2, WAVES_N = 4 / WAVES_M;
-  static constexpr int WTM = BM / WAVES_M, WTN = 64 / WAVES_N, TM = WTM / 16, TN = WTN / 16;
+  static constexpr int WAVES_M = BM / 32, WAVES_K = 4 / WAVES_M;
+  static constexpr int KSTEPS = KS / 32 / WAVES_K;                 // MFMA k-steps per wave
+  static_assert((KS / 32) % WAVES_K == 0, "K slice must split evenly over the waves");
+  static constexpr int RED_LD = 68;                                // floats per row of the reduction buffer
+  static constexpr int RED_BYTES = WAVES_K * BM * RED_LD * 4;
+  static_assert(RED_BYTES <= X_BYTES, "the reduction buffer reuses the X region");
+  static constexpr int CPT = BM * 64 / 256;                        // output columns per thread in the epilogue
 
   typedef __attribute__((address_space(1))) const void *gptr_t;
   typedef __attribute__((address_space(3))) void *lptr_t;
@@ -59,42 +68,60 @@ struct GemmOneShot {
     __syncthreads();
   }
 
-  // epi(m, n, v): v[i] = sum over the slice of X[m][k] W[k][n+i]; m, n relative to the tile origin.
-  template <class Epi>
-  __device__ static __forceinline__ void compute(const unsigned char *lds_x, const unsigned char *lds_w, Epi epi) {
+  // MFMA over this wave's share of the slice; then every wave is done reading X and W
+  // (so the caller may queue new loads into the W region), the partial tiles are summed
+  // through the X region, and epi(m, n, v) is called with v[i] = Y[m][n+i], i = 0..3,
+  // m and n relative to the tile origin, CPT/4 times per thread.
+  template <class AfterMfma, class Epi>
+  __device__ static __forceinline__ void compute(unsigned char *lds_x, const unsigned char *lds_w, AfterMfma after_mfma, Epi epi) {
     const half_t *xs = reinterpret_cast<const half_t *>(lds_x), *ws = reinterpret_cast<const half_t *>(lds_w);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l16 = lane & 15, g = lane >> 4;
-    const int wm0 = (wave / WAVES_N) * WTM, wn0 = (wave % WAVES_N) * WTN;
-    f4 acc[TM][TN];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+    const int wm = wave / WAVES_K, wk = wave % WAVES_K;
+    f4 acc[2][4];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-    for (int ks = 0; ks < KS / 32; ++ks) {
-      h8 xop[TM], wop[TN];
+      for (int j = 0; j < 4; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int r = wm0 + i * 16 + l16;
+    for (int s = 0; s < KSTEPS; ++s) {
+      const int ks = wk * KSTEPS + s;
+      h8 xop[2], wop[4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int r = wm * 32 + i * 16 + l16;
         xop[i] = *reinterpret_cast<const h8 *>(xs + (r * XGR + ((ks * 4 + g) ^ (r & 15))) * 8);
       }
       const int k = ks * 32 + g * 8 + (l16 >> 2);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int c = ((wn0 + j * 16) >> 3) + ((l16 & 3) >> 1);
+      for (int j = 0; j < 4; ++j) {
+        const int c = j * 2 + ((l16 & 3) >> 1);
         const half_t *p = ws + (k * 8 + (c ^ (k & 2))) * 8 + (l16 & 1) * 4;
         const h4 lo = lds_read_tr16(p), hi = lds_read_tr16(p + 4 * 64);
         wop[j] = h8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = mfma_16x16x32(wop[j], xop[i], acc[i][j]);
+        for (int j = 0; j < 4; ++j) acc[i][j] = mfma_16x16x32(wop[j], xop[i], acc[i][j]);
     }
+    __syncthreads();                       // X and W slices are dead from here on
+    after_mfma();
+    float *red = reinterpret_cast<float *>(lds_x);
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) epi(wm0 + i * 16 + l16, wn0 + j * 16 + g * 4, acc[i][j]);
+      for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<f4 *>(red + (wk * BM + wm * 32 + i * 16 + l16) * RED_LD + j * 16 + g * 4) = acc[i][j];
+    __syncthreads();
+    constexpr int TPR = 64 / CPT;           // threads per output row
+    const int row = tid / TPR, col0 = (tid % TPR) * CPT;
+#pragma unroll
+    for (int c = 0; c < CPT / 4; ++c) {
+      f4 v = *reinterpret_cast<const f4 *>(red + row * RED_LD + col0 + c * 4);
+#pragma unroll
+      for (int w = 1; w < WAVES_K; ++w) v += *reinterpret_cast<const f4 *>(red + (w * BM + row) * RED_LD + col0 + c * 4);
+      epi(row, col0 + c * 4, v);
+    }
   }
 };
 

@@ -9,7 +9,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libsouffle_hip.so")
+LIB_PATH = os.environ.get("SOUFFLE_HIP_LIB") or os.path.join(_HERE, "libsouffle_hip.so")
 
 ACT_GELU_TANH, ACT_RELU = 0, 1
 GATES_IFGO, GATES_IGFO = 0, 1
