@@ -21,11 +21,11 @@ _workspaces = {}
 
 def _workspace(cfg, device):
     key = (device, cfg.batch, cfg.seq_len)
+    nbytes = sh.lib().souffle_bert_workspace_bytes(C.byref(cfg))
+    if nbytes == 0:
+        raise sh.SouffleError(-2, sh.last_error())
     ws = _workspaces.get(key)
-    if ws is None:
-        nbytes = sh.lib().souffle_bert_workspace_bytes(C.byref(cfg))
-        if nbytes == 0:
-            raise sh.SouffleError(-2, sh.last_error())
+    if ws is None or ws.nbytes < nbytes:          # grows with the number of layers
         ws = _workspaces[key] = sh.Workspace(nbytes, device)
     return ws
 

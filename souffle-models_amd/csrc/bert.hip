@@ -28,28 +28,45 @@ struct LayerW {
   const half_t *w_qkv, *b_qkv, *w_o, *b_o, *ln1_g, *ln1_b, *w_fc1, *b_fc1, *w_fc2, *b_fc2, *ln2_g, *ln2_b;
 };
 
-struct Args {
+// Per-launch parameters.  The inter-stage buffers (qkv .. yl) are given per layer
+// (`layer_stride` bytes apart) so that inside one launch every address is written by exactly
+// one stage of one layer and read only afterwards: readers can then use ordinary cached
+// loads (an XCD's L2 never holds an older version of a line) and each XCD fetches a line of
+// an activation once instead of every workgroup fetching it from memory.
+struct Params {
   int B, S, M, act, num_layers, splitk_o, splitk_f;
   float scale, eps;
   const half_t *x, *mask;
   half_t *y;
-  half_t *qkv, *ctx, *z1, *y1, *h, *xa, *xb, *probs;
+  half_t *qkv, *ctx, *z1, *y1, *h, *yl, *probs;
   float *part;
   unsigned *ctl;
   unsigned long long *trace;
   int trace_cap;
+  size_t layer_stride;
+};
+struct Args : Params {
   LayerW layers[kMaxLayers];
 };
 
+__device__ __forceinline__ Params layer_params(const Params &a, int l) {
+  Params p = a;
+  const size_t off = (size_t)l * a.layer_stride;
+  auto adv = [&](half_t *q) { return reinterpret_cast<half_t *>(reinterpret_cast<char *>(q) + off); };
+  p.qkv = adv(a.qkv); p.ctx = adv(a.ctx); p.z1 = adv(a.z1); p.y1 = adv(a.y1); p.h = adv(a.h); p.yl = adv(a.yl);
+  p.part = reinterpret_cast<float *>(reinterpret_cast<char *>(a.part) + off);
+  return p;
+}
+
 // ------------------------------------------------------------------ stages ----
 template <bool COH, class Tile>
-__device__ __forceinline__ void stage_qkv(half_t *lds, const Args &a, const LayerW &w, const half_t *xin,
+__device__ __forceinline__ void stage_qkv(half_t *lds, const Params &a, const LayerW &w, const half_t *xin,
                                           int first, int stride) {
   constexpr int BM = Tile::kBM, BN = Tile::kBN, BK = Tile::kBK;
   const int tiles_n = 3 * H / BN, items = (a.M / BM) * tiles_n;
   for (int item = first; item < items; item += stride) {
     const int tm = item / tiles_n, n0 = (item % tiles_n) * BN, j = n0 / H, nn0 = n0 % H;
-    auto aload = [&](int m, int k) { return ld16<COH>(xin, (m * H + k) * 2); };
+    auto aload = [&](int m, int k) { return ld16<false>(xin, (m * H + k) * 2); };
     auto epi = [&](int m, int n, f4 v) {
       if (w.b_qkv) {
         const h4 bb = *reinterpret_cast<const h4 *>(w.b_qkv + j * H + n);
@@ -64,12 +81,12 @@ __device__ __forceinline__ void stage_qkv(half_t *lds, const Args &a, const Laye
 
 // Y = act(X.W + b), fp16 out (FC1).
 template <bool COH, class Tile>
-__device__ __forceinline__ void stage_fc1(half_t *lds, const Args &a, const LayerW &w, int first, int stride) {
+__device__ __forceinline__ void stage_fc1(half_t *lds, const Params &a, const LayerW &w, int first, int stride) {
   constexpr int BM = Tile::kBM, BN = Tile::kBN, BK = Tile::kBK;
   const int tiles_n = F / BN, items = (a.M / BM) * tiles_n;
   for (int item = first; item < items; item += stride) {
     const int tm = item / tiles_n, n0 = (item % tiles_n) * BN;
-    auto aload = [&](int m, int k) { return ld16<COH>(a.y1, (m * H + k) * 2); };
+    auto aload = [&](int m, int k) { return ld16<false>(a.y1, (m * H + k) * 2); };
     auto epi = [&](int m, int n, f4 v) {
       if (w.b_fc1) {
         const h4 bb = *reinterpret_cast<const h4 *>(w.b_fc1 + n);
@@ -85,13 +102,13 @@ __device__ __forceinline__ void stage_fc1(half_t *lds, const Args &a, const Laye
 
 // fp32 split-K partials of X[M][K].W[K][H]: part[ks][m][n].
 template <bool COH, class Tile>
-__device__ __forceinline__ void stage_partial(half_t *lds, const Args &a, const half_t *X, int K,
+__device__ __forceinline__ void stage_partial(half_t *lds, const Params &a, const half_t *X, int K,
                                               const half_t *W, int splitk, int first, int stride) {
   constexpr int BM = Tile::kBM, BN = Tile::kBN, BK = Tile::kBK;
   const int tiles_n = H / BN, items = (a.M / BM) * tiles_n * splitk, kper = K / splitk;
   for (int item = first; item < items; item += stride) {
     const int ks = item % splitk, t = item / splitk, tm = t / tiles_n, n0 = (t % tiles_n) * BN;
-    auto aload = [&](int m, int k) { return ld16<COH>(X, (m * K + k) * 2); };
+    auto aload = [&](int m, int k) { return ld16<false>(X, (m * K + k) * 2); };
     auto epi = [&](int m, int n, f4 v) {
       st16<COH>(a.part, ((ks * a.M + m) * H + n) * 4, __builtin_bit_cast(u4, v));
     };
@@ -101,7 +118,7 @@ __device__ __forceinline__ void stage_partial(half_t *lds, const Args &a, const 
 
 // out[m] = LN(sum_ks part[ks][m] + bias + resid[m]) * g + b; one wave per row.
 template <bool COH, int SPLITK>
-__device__ __forceinline__ void stage_ln_t(const Args &a, const half_t *bias, const half_t *resid,
+__device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, const half_t *resid,
                                          const half_t *gam, const half_t *bet, half_t *out,
                                          int first_row, int row_stride) {
   const int lane = threadIdx.x & 63;
@@ -114,8 +131,8 @@ __device__ __forceinline__ void stage_ln_t(const Args &a, const half_t *bias, co
     for (int c = 0; c < 3; ++c) {
       const int n = c * 256 + lane * 4;
 #pragma unroll
-      for (int ks = 0; ks < SPLITK; ++ks) raw[c][ks] = ld16<COH>(a.part, ((ks * a.M + m) * H + n) * 4);
-      rres[c] = ld8<COH>(resid, (m * H + n) * 2);
+      for (int ks = 0; ks < SPLITK; ++ks) raw[c][ks] = ld16<false>(a.part, ((ks * a.M + m) * H + n) * 4);
+      rres[c] = ld8<false>(resid, (m * H + n) * 2);
     }
 #pragma unroll
     for (int c = 0; c < 3; ++c) {
@@ -174,71 +191,101 @@ struct Item {
   const half_t *W;      // weight matrix the slice comes from
   int ldw, k0;          // its row pitch, first row of the K slice
   int aux;              // stage specific (q/k/v index, K-slice index)
+  int rot;              // rotation of the weight-row request order (see GemmOneShot::issue_w)
 };
 
-// Items are dealt m-tile fastest: the workgroups that share a weight slice are neighbours,
-// i.e. sit on different XCDs, so no L2 sees the same line requested twice at once.
+// Workgroup b runs on XCD b % 8 (each XCD has its own L2).  The m-tiles that share one weight
+// slice are dealt to workgroups of ONE XCD in the same pass, so the slice crosses the fabric
+// once per XCD instead of once per workgroup.  Returns false when `it` names no item.
+__device__ __forceinline__ bool xcd_item(int it, int m_tiles, int w_slices, int *mt, int *ws) {
+  if ((gridDim.x & 7) != 0) { *mt = it % m_tiles; *ws = it / m_tiles; return it < m_tiles * w_slices; }
+  const int xcd = it & 7, j = it >> 3;
+  *mt = j % m_tiles;
+  *ws = (j / m_tiles) * 8 + xcd;
+  return *ws < w_slices;
+}
+__device__ __forceinline__ int xcd_item_span(int m_tiles, int w_slices) {   // exclusive upper bound of valid `it`
+  return (gridDim.x & 7) != 0 ? m_tiles * w_slices : ((w_slices + 7) >> 3) * m_tiles * 8;
+}
+
 struct QkvItems {
   const half_t *w_qkv; int M;
-  __device__ int count() const { return (M / OsFull::kBM) * (3 * H / 64); }
-  __device__ Item at(int it) const {
-    const int mt = M / OsFull::kBM, n0 = (it / mt) * 64, j = n0 / H;
-    return Item{(it % mt) * OsFull::kBM, n0 % H, w_qkv + (size_t)j * H * H, H, 0, j};
+  __device__ int span() const { return xcd_item_span(M / OsFull::kBM, 3 * H / 64); }
+  __device__ bool at(int it, Item &d) const {
+    int mt, ws;
+    if (!xcd_item(it, M / OsFull::kBM, 3 * H / 64, &mt, &ws)) return false;
+    const int n0 = ws * 64, j = n0 / H;
+    d = Item{mt * OsFull::kBM, n0 % H, w_qkv + (size_t)j * H * H, H, 0, j, mt * (OsFull::W_INSTR / 4) / (M / OsFull::kBM)};
+    return true;
   }
 };
 struct OutItems {
   const half_t *w_o; int M;
-  __device__ int count() const { return (M / OsFull::kBM) * (H / 64); }
-  __device__ Item at(int it) const { const int mt = M / OsFull::kBM; return Item{(it % mt) * OsFull::kBM, (it / mt) * 64, w_o, H, 0, 0}; }
+  __device__ int span() const { return xcd_item_span(M / OsFull::kBM, H / 64); }
+  __device__ bool at(int it, Item &d) const {
+    int mt, ws;
+    if (!xcd_item(it, M / OsFull::kBM, H / 64, &mt, &ws)) return false;
+    d = Item{mt * OsFull::kBM, ws * 64, w_o, H, 0, 0, mt * (OsFull::W_INSTR / 4) / (M / OsFull::kBM)};
+    return true;
+  }
 };
 struct Fc1Items {
   const half_t *w_fc1; int M;
-  __device__ int count() const { return (M / OsFull::kBM) * (F / 64); }
-  __device__ Item at(int it) const { const int mt = M / OsFull::kBM; return Item{(it % mt) * OsFull::kBM, (it / mt) * 64, w_fc1, F, 0, 0}; }
+  __device__ int span() const { return xcd_item_span(M / OsFull::kBM, F / 64); }
+  __device__ bool at(int it, Item &d) const {
+    int mt, ws;
+    if (!xcd_item(it, M / OsFull::kBM, F / 64, &mt, &ws)) return false;
+    d = Item{mt * OsFull::kBM, ws * 64, w_fc1, F, 0, 0, mt * (OsFull::W_INSTR / 4) / (M / OsFull::kBM)};
+    return true;
+  }
 };
 struct Fc2Items {
   const half_t *w_fc2; int M;
-  __device__ int count() const { return (M / OsFc2::kBM) * (H / 64) * kSplitFc2Small; }
-  __device__ Item at(int it) const {
-    const int mt = M / OsFc2::kBM, ws = it / mt, ks = ws % kSplitFc2Small;
-    return Item{(it % mt) * OsFc2::kBM, (ws / kSplitFc2Small) * 64, w_fc2, H, ks * OsFc2::kKS, ks};
+  __device__ int span() const { return xcd_item_span(M / OsFc2::kBM, (H / 64) * kSplitFc2Small); }
+  __device__ bool at(int it, Item &d) const {
+    int mt, ws;
+    if (!xcd_item(it, M / OsFc2::kBM, (H / 64) * kSplitFc2Small, &mt, &ws)) return false;
+    const int ks = ws % kSplitFc2Small;
+    d = Item{mt * OsFc2::kBM, (ws / kSplitFc2Small) * 64, w_fc2, H, ks * OsFc2::kKS, ks, mt * (OsFc2::W_INSTR / 4) / (M / OsFc2::kBM)};
+    return true;
   }
 };
-struct NoItems {
-  __device__ int count() const { return 0; }
-  __device__ Item at(int) const { return Item{0, 0, nullptr, 0, 0, 0}; }
-};
+
+// Whether the weight slice of the next stage is queued before the grid barrier.  Measured on
+// MI355X this does not pay: the CU's vector memory pipeline is in order across its waves, so
+// the barrier's own atomics and polling loads queue up behind the ~100 KB in flight and the
+// barrier stretches by as much as the prefetch saves.
+constexpr bool kPrefetchAcrossBarrier = false;
 
 // Queue the weight slice of this workgroup's first item of a stage (if it has one).
 template <class G, class Items>
 __device__ __forceinline__ bool preissue_w(unsigned char *lds, const Items &items) {
-  if ((int)blockIdx.x >= items.count()) return false;
-  const Item d = items.at(blockIdx.x);
-  G::issue_w(lds + kXRegion, d.W, d.ldw, d.n0, d.k0);
+  Item d;
+  if (!kPrefetchAcrossBarrier || (int)blockIdx.x >= items.span() || !items.at(blockIdx.x, d)) return false;
+  G::issue_w_prefetch(lds + kXRegion, d.W, d.ldw, d.n0, d.k0);
   return true;
 }
 
 // Driver of a skinny GEMM stage.  `w_ready`: the weight slice of this workgroup's first item
 // was queued before the preceding grid barrier.  `pre(item)` runs after the operands have
 // landed (LayerNorm on load), `epi(item, m, n, v)` receives 4 consecutive columns of a row,
-// `next()` queues the first weight slice of the FOLLOWING stage as soon as the W region is free.
+// `next()` queues the first weight slice of the FOLLOWING stage once the stage's stores are issued.
 template <class G, bool COH, class Items, class Pre, class Epi, class Next>
 __device__ __forceinline__ void gemm_stage(unsigned char *lds, const Items &items, const half_t *X, int ldx, bool w_ready,
                                            Pre pre, Epi epi, Next next) {
-  const int n = items.count();
-  int it = blockIdx.x;
-  if (it >= n) { next(); return; }
-  for (; it < n; it += gridDim.x) {
-    const Item d = items.at(it);
+  const int span = items.span();
+  for (int it = blockIdx.x; it < span; it += gridDim.x) {
+    Item d;
+    if (!items.at(it, d)) { w_ready = false; continue; }
     __syncthreads();                       // LDS reuse
-    if (!w_ready) G::issue_w(lds + kXRegion, d.W, d.ldw, d.n0, d.k0);
-    G::template issue_x<COH>(lds, X, ldx, d.m0, d.k0);
+    if (!w_ready) G::issue_w(lds + kXRegion, d.W, d.ldw, d.n0, d.k0, d.rot);
+    G::template issue_x<false>(lds, X, ldx, d.m0, d.k0);
     G::wait_loads();
     pre(d);
-    const bool last = it + (int)gridDim.x >= n;
-    G::compute(lds, lds + kXRegion, [&]() { if (last) next(); }, [&](int mm, int nn, f4 v) { epi(d, d.m0 + mm, d.n0 + nn, v); });
+    G::compute(lds, lds + kXRegion, [&](int mm, int nn, f4 v) { epi(d, d.m0 + mm, d.n0 + nn, v); });
     w_ready = false;
   }
+  next();     // after the last store of the stage, so that only these loads are younger than it
 }
 
 __device__ __forceinline__ f4 add_bias4(f4 v, const half_t *bias, int n) {
@@ -303,7 +350,7 @@ __device__ __forceinline__ void ln_rows_in_lds(unsigned char *lds_x, const half_
 }
 
 template <bool COH>
-__device__ __forceinline__ void stage_ln(const Args &a, int splitk, const half_t *bias, const half_t *resid,
+__device__ __forceinline__ void stage_ln(const Params &a, int splitk, const half_t *bias, const half_t *resid,
                                          const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
   if (splitk == 1) stage_ln_t<COH, 1>(a, bias, resid, gam, bet, out, first_row, row_stride);
   else stage_ln_t<COH, kSplitFc2Small>(a, bias, resid, gam, bet, out, first_row, row_stride);
@@ -311,7 +358,7 @@ __device__ __forceinline__ void stage_ln(const Args &a, int splitk, const half_t
 
 // The four skinny GEMM stages (shared by the megakernel and the per-op kernels).
 template <bool COH, class Next>
-__device__ __forceinline__ void small_qkv(unsigned char *lds, const Args &a, const LayerW &w, const half_t *xin, bool w_ready, Next next) {
+__device__ __forceinline__ void small_qkv(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, Next next) {
   gemm_stage<OsFull, COH>(lds, QkvItems{w.w_qkv, a.M}, xin, H, w_ready, [](const Item &) {},
     [&](const Item &d, int m, int n, f4 v) {
       v = add_bias4(v, w.b_qkv ? w.b_qkv + d.aux * H : nullptr, n);
@@ -321,11 +368,11 @@ __device__ __forceinline__ void small_qkv(unsigned char *lds, const Args &a, con
 }
 // z1 = ctx.Wo + b_o + x (pre-LayerNorm, fp16)
 template <bool COH, class Next>
-__device__ __forceinline__ void small_outproj(unsigned char *lds, const Args &a, const LayerW &w, const half_t *xin, bool w_ready, Next next) {
+__device__ __forceinline__ void small_outproj(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, Next next) {
   gemm_stage<OsFull, COH>(lds, OutItems{w.w_o, a.M}, a.ctx, H, w_ready, [](const Item &) {},
     [&](const Item &, int m, int n, f4 v) {
       v = add_bias4(v, w.b_o, n);
-      const h4 r = as_h4(ld8<COH>(xin, (m * H + n) * 2));
+      const h4 r = as_h4(ld8<false>(xin, (m * H + n) * 2));
       v += f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
       st8<COH>(a.z1, (m * H + n) * 2, pack_h4(v));
     }, next);
@@ -333,7 +380,7 @@ __device__ __forceinline__ void small_outproj(unsigned char *lds, const Args &a,
 // h = act(LN1(z1).W1 + b1): LayerNorm is applied to the X tile in LDS (every workgroup has
 // complete rows); the workgroups of the first n-tile also publish y1 = LN1(z1).
 template <bool COH, class Next>
-__device__ __forceinline__ void small_fc1(unsigned char *lds, const Args &a, const LayerW &w, bool w_ready, Next next) {
+__device__ __forceinline__ void small_fc1(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, Next next) {
   gemm_stage<OsFull, COH>(lds, Fc1Items{w.w_fc1, a.M}, a.z1, H, w_ready,
     [&](const Item &d) { ln_rows_in_lds<COH>(lds, w.ln1_g, w.ln1_b, a.eps, d.n0 == 0 ? a.y1 : nullptr, d.m0); },
     [&](const Item &, int m, int n, f4 v) {
@@ -345,7 +392,7 @@ __device__ __forceinline__ void small_fc1(unsigned char *lds, const Args &a, con
 }
 // fp32 partials of h.W2 over 8 K slices
 template <bool COH, class Next>
-__device__ __forceinline__ void small_fc2(unsigned char *lds, const Args &a, const LayerW &w, bool w_ready, Next next) {
+__device__ __forceinline__ void small_fc2(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, Next next) {
   gemm_stage<OsFc2, COH>(lds, Fc2Items{w.w_fc2, a.M}, a.h, F, w_ready, [](const Item &) {},
     [&](const Item &d, int m, int n, f4 v) { st16<COH>(a.part, ((d.aux * a.M + m) * H + n) * 4, __builtin_bit_cast(u4, v)); }, next);
 }
@@ -370,7 +417,7 @@ __device__ __forceinline__ void issue_rows64(unsigned char *lds, const half_t *s
 }
 
 template <bool COH, int NKT>
-__device__ __forceinline__ void attn_item(half_t *lds_h, const Args &a, int item) {
+__device__ __forceinline__ void attn_item(half_t *lds_h, const Params &a, int item) {
   constexpr int S = NKT * 16;
   unsigned char *lds = reinterpret_cast<unsigned char *>(lds_h);
   unsigned char *ks_ = lds, *vs_ = lds + S * 128, *qs_ = lds + 2 * S * 128;
@@ -382,9 +429,9 @@ __device__ __forceinline__ void attn_item(half_t *lds_h, const Args &a, int item
   const half_t *Q = a.qkv + head_off + (size_t)qb * 64 * HD, *K = a.qkv + plane + head_off, *V = a.qkv + 2 * plane + head_off;
 
   __syncthreads();   // LDS reuse
-  issue_rows64<COH, 0>(ks_, K, S);
-  issue_rows64<COH, 1>(vs_, V, S);
-  issue_rows64<COH, 0>(qs_, Q, 64);
+  issue_rows64<false, 0>(ks_, K, S);
+  issue_rows64<false, 1>(vs_, V, S);
+  issue_rows64<false, 0>(qs_, Q, 64);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
@@ -456,8 +503,13 @@ __device__ __forceinline__ void attn_item(half_t *lds_h, const Args &a, int item
     st8<COH>(a.ctx, ((b * S + q) * H + hh * HD + dt * 16 + g * 4) * 2, pack_h4(o[dt]));
 }
 
+template <bool COH, int NKT>
+__device__ __forceinline__ void stage_attn_t(half_t *lds, const Params &a, int first, int stride) {
+  const int items = a.B * NH * (a.S / 64);
+  for (int item = first; item < items; item += stride) attn_item<COH, NKT>(lds, a, item);
+}
 template <bool COH>
-__device__ __forceinline__ void stage_attn(half_t *lds, const Args &a, int first, int stride) {
+__device__ __forceinline__ void stage_attn(half_t *lds, const Params &a, int first, int stride) {
   const int items = a.B * NH * (a.S / 64);
   for (int item = first; item < items; item += stride) {
     switch (a.S) {
@@ -479,26 +531,27 @@ constexpr int lds_bytes(bool large) {
 }
 
 // ------------------------------------------------------------ megakernel ----
-template <bool LARGE>
-__global__ void __launch_bounds__(256) k_encoder_mega(Args a) {
+template <bool LARGE, int NKT>
+__global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   half_t *lds = reinterpret_cast<half_t *>(lds_raw);
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
   GridBarrier bar;
-  grid_barrier_begin(bar, a.ctl);
-  bar.trace = a.trace;
-  bar.trace_cap = a.trace_cap;
+  grid_barrier_begin(bar, args.ctl);
+  bar.trace = args.trace;
+  bar.trace_cap = args.trace_cap;
   const int first = blockIdx.x, stride = gridDim.x;
   const int wave = threadIdx.x >> 6;
-  const half_t *xin = a.x;
+  const half_t *xin = args.x;
   bool qkv_ready = false;
-  for (int l = 0; l < a.num_layers; ++l) {
-    const LayerW w = a.layers[l];
-    half_t *yout = (l == a.num_layers - 1) ? a.y : ((l & 1) ? a.xb : a.xa);
+  for (int l = 0; l < args.num_layers; ++l) {
+    const LayerW w = args.layers[l];
+    const Params a = layer_params(args, l);
+    half_t *yout = (l == a.num_layers - 1) ? a.y : a.yl;
     if constexpr (LARGE) {
       stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
       grid_sync(bar);
-      stage_attn<true>(lds, a, first, stride);
+      stage_attn_t<true, NKT>(lds, a, first, stride);
       grid_sync(bar);
       stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
       grid_sync(bar);
@@ -519,23 +572,23 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args a) {
       const Fc2Items fc2_items{w.w_fc2, a.M};
       bool out_ready = false;
       small_qkv<true>(lds_raw, a, w, xin, qkv_ready, [&]() { if (attn_fits) out_ready = preissue_w<OsFull>(lds_raw, out_items); });
-      grid_sync(bar);
-      stage_attn<true>(lds, a, first, stride);
+      grid_sync(bar, out_ready ? OsFull::PREFETCH_INSTR : 0);
+      stage_attn_t<true, NKT>(lds, a, first, stride);
       if (!attn_fits) { __syncthreads(); out_ready = preissue_w<OsFull>(lds_raw, out_items); }
-      grid_sync(bar);
+      grid_sync(bar, attn_fits ? 0 : (out_ready ? OsFull::PREFETCH_INSTR : 0));
       bool fc1_ready = false, fc2_ready = false;
       small_outproj<true>(lds_raw, a, w, xin, out_ready, [&]() { fc1_ready = preissue_w<OsFull>(lds_raw, fc1_items); });
-      grid_sync(bar);
+      grid_sync(bar, fc1_ready ? OsFull::PREFETCH_INSTR : 0);
       small_fc1<true>(lds_raw, a, w, fc1_ready, [&]() { fc2_ready = preissue_w<OsFc2>(lds_raw, fc2_items); });
-      grid_sync(bar);
+      grid_sync(bar, fc2_ready ? OsFc2::PREFETCH_INSTR : 0);
       qkv_ready = false;
       small_fc2<true>(lds_raw, a, w, fc2_ready, [&]() {
-        if (l + 1 < a.num_layers) qkv_ready = preissue_w<OsFull>(lds_raw, QkvItems{a.layers[l + 1].w_qkv, a.M});
+        if (l + 1 < a.num_layers) qkv_ready = preissue_w<OsFull>(lds_raw, QkvItems{args.layers[l + 1].w_qkv, a.M});
       });
-      grid_sync(bar);
+      grid_sync(bar, qkv_ready ? OsFull::PREFETCH_INSTR : 0);
       stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
     }
-    if (l + 1 < a.num_layers) grid_sync(bar);
+    if (l + 1 < a.num_layers) grid_sync(bar);   // (a prefetched QKV slice is older than the LN2 stores: wait for everything)
     xin = yout;
   }
   grid_barrier_end(bar);
@@ -584,7 +637,7 @@ __global__ void __launch_bounds__(256) k_outproj_small(Args a, int l, const half
 struct Plan {
   bool large;
   int splitk_o, splitk_f;
-  size_t off_ctl, off_qkv, off_ctx, off_z1, off_y1, off_h, off_xa, off_xb, off_part, total;
+  size_t off_ctl, off_qkv, off_ctx, off_z1, off_y1, off_h, off_yl, off_part, layer_stride, total;
 };
 
 static int validate(const souffle_bert_cfg *c) {
@@ -603,7 +656,7 @@ static int validate(const souffle_bert_cfg *c) {
   return SOUFFLE_OK;
 }
 
-static Plan make_plan(const souffle_bert_cfg *c) {
+static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   Plan p;
   const size_t M = (size_t)c->batch * c->seq_len;
   p.large = M >= 1024;
@@ -612,15 +665,16 @@ static Plan make_plan(const souffle_bert_cfg *c) {
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += round_up(bytes, 256); return o; };
   p.off_ctl = take(kCtlWords * 4);
+  const size_t first = off;
   p.off_qkv = take(3 * M * H * 2);
   p.off_ctx = take(M * H * 2);
   p.off_z1 = take(M * H * 2);
   p.off_y1 = take(M * H * 2);
   p.off_h = take(M * F * 2);
-  p.off_xa = take(M * H * 2);
-  p.off_xb = take(M * H * 2);
+  p.off_yl = take(M * H * 2);
   p.off_part = take((size_t)(p.splitk_f > p.splitk_o ? p.splitk_f : p.splitk_o) * M * H * 4);
-  p.total = off;
+  p.layer_stride = off - first;                       // one set of inter-stage buffers per layer
+  p.total = first + p.layer_stride * (size_t)(num_layers < 1 ? 1 : num_layers);
   return p;
 }
 
@@ -643,8 +697,8 @@ static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_laye
   a.z1 = reinterpret_cast<half_t *>(base + p.off_z1);
   a.y1 = reinterpret_cast<half_t *>(base + p.off_y1);
   a.h = reinterpret_cast<half_t *>(base + p.off_h);
-  a.xa = reinterpret_cast<half_t *>(base + p.off_xa);
-  a.xb = reinterpret_cast<half_t *>(base + p.off_xb);
+  a.yl = reinterpret_cast<half_t *>(base + p.off_yl);
+  a.layer_stride = p.layer_stride;
   a.part = reinterpret_cast<float *>(base + p.off_part);
   a.probs = nullptr;
   a.trace = nullptr;
@@ -672,17 +726,28 @@ static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_laye
   return SOUFFLE_OK;
 }
 
-template <bool LARGE>
-static int launch_mega(Args &a, int grid, hipStream_t st) {
+template <bool LARGE, int NKT>
+static int launch_mega_t(Args &a, int grid, hipStream_t st) {
   const int lds = lds_bytes(LARGE);
   static bool attr_done = false;
   if (!attr_done) {
-    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_encoder_mega<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_encoder_mega<LARGE, NKT>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     attr_done = true;
   }
   void *args[] = {&a};
-  SOUFFLE_HIP_TRY(hipLaunchCooperativeKernel((const void *)k_encoder_mega<LARGE>, dim3(grid), dim3(256), args, lds, st));
+  SOUFFLE_HIP_TRY(hipLaunchCooperativeKernel((const void *)k_encoder_mega<LARGE, NKT>, dim3(grid), dim3(256), args, lds, st));
   return SOUFFLE_OK;
+}
+// one kernel per supported sequence length, so that each carries only its own attention tile
+template <bool LARGE>
+static int launch_mega(Args &a, int grid, hipStream_t st) {
+  switch (a.S) {
+    case 64: return launch_mega_t<LARGE, 4>(a, grid, st);
+    case 128: return launch_mega_t<LARGE, 8>(a, grid, st);
+    case 256: return launch_mega_t<LARGE, 16>(a, grid, st);
+    case 384: return launch_mega_t<LARGE, 24>(a, grid, st);
+    default: return launch_mega_t<LARGE, 32>(a, grid, st);
+  }
 }
 
 static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *layers, int nl, const void *x,
@@ -692,7 +757,7 @@ static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *laye
   DeviceFacts df;
   if (int rc = device_facts(&df)) return rc;
   if (!df.cooperative) return fail(SOUFFLE_ERR_DEVICE, "device does not support cooperative launch");
-  const Plan p = make_plan(c);
+  const Plan p = make_plan(c, nl);
   static thread_local Args a;
   if (int rc = fill_args(a, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
   stage_trace(&a.trace, &a.trace_cap, df.num_cus);
@@ -719,7 +784,7 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
   const half_t *xin = a.x;
   for (int l = 0; l < nl; ++l) {
     const LayerW &w = a.layers[l];
-    half_t *yout = (l == nl - 1) ? a.y : ((l & 1) ? a.xb : a.xa);
+    half_t *yout = (l == nl - 1) ? a.y : a.yl;
     hipLaunchKernelGGL(k_qkv<LARGE>, dim3(grid_for((a.M / BM_QKV) * (3 * H / BN))), dim3(256), GEMM_LDS, st, a, l, xin);
     hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), 2 * a.S * 128 + 64 * 128, st, a);
     if (LARGE) {
@@ -743,7 +808,7 @@ static int run_unfused(const souffle_bert_cfg *c, const souffle_bert_layer_w *la
   if (int rc = validate(c)) return rc;
   DeviceFacts df;
   if (int rc = device_facts(&df)) return rc;
-  const Plan p = make_plan(c);
+  const Plan p = make_plan(c, nl);
   static thread_local Args a;
   if (int rc = fill_args(a, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -757,7 +822,8 @@ using namespace souffle;
 
 extern "C" size_t souffle_bert_workspace_bytes(const souffle_bert_cfg *cfg) {
   if (bert::validate(cfg)) return 0;
-  return bert::make_plan(cfg).total;
+  const int nl = cfg->num_layers < 1 ? 1 : (cfg->num_layers > bert::kMaxLayers ? bert::kMaxLayers : cfg->num_layers);
+  return bert::make_plan(cfg, nl).total;
 }
 extern "C" int souffle_bert_layer_fused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *w, const void *x,
                                         const void *mask, void *y, const souffle_bert_dump *dump, void *ws,

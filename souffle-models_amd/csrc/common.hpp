@@ -175,11 +175,26 @@ __device__ __forceinline__ void grid_barrier_begin(GridBarrier &b, unsigned *ctl
   b.target = __hip_atomic_load(ctl + 256 + 32 * x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-__device__ __forceinline__ void grid_sync(GridBarrier &b) {
+// s_waitcnt with only the vector-memory counter: all but the youngest N vector memory
+// instructions of this wave have completed (they complete in issue order).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// `pending`: number of vector loads (0, 16 or 32) that every wave except wave 0 queued AFTER
+// its last store of the stage and that may stay in flight across the barrier (prefetch of the
+// next stage's weight slice into LDS); everything older, i.e. every store, must be
+// acknowledged.  Wave 0 polls the barrier and therefore never has such loads.
+__device__ __forceinline__ void grid_sync(GridBarrier &b, int pending = 0) {
   const bool tr = b.trace && b.trace_idx < b.trace_cap && threadIdx.x == 0;
   if (tr) b.trace[(size_t)(2 * b.trace_idx) * b.nblk + blockIdx.x] = wall_clock64();
-  __builtin_amdgcn_s_waitcnt(0);   // this wave's write-through stores are acknowledged
-  __syncthreads();
+  if (threadIdx.x < 64 || pending == 0) __builtin_amdgcn_s_waitcnt(0);   // write-through stores are acknowledged
+  else if (pending == 32) wait_vmcnt<32>();
+  else if (pending == 16) wait_vmcnt<16>();
+  else __builtin_amdgcn_s_waitcnt(0);
+  __builtin_amdgcn_s_barrier();
   b.target += b.gsz;
   if (threadIdx.x < 64) {
     if (threadIdx.x == 0)
@@ -195,7 +210,8 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b) {
   b.count++;
   if (tr) b.trace[(size_t)(2 * b.trace_idx + 1) * b.nblk + blockIdx.x] = wall_clock64();
   b.trace_idx++;
-  __syncthreads();
+  __builtin_amdgcn_s_barrier();          // no memory wait here: prefetch loads may still be in flight
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
 // Call once by every workgroup before the kernel returns.

@@ -42,19 +42,44 @@ struct GemmOneShot {
   typedef __attribute__((address_space(1))) const void *gptr_t;
   typedef __attribute__((address_space(3))) void *lptr_t;
 
+  // The lane id as a value the optimiser cannot see through: keeps the dozens of per-load
+  // addresses from being hoisted out of the layer loop (and spilled) in the megakernel.
+  __device__ static __forceinline__ int opaque_tid() {
+    int t = threadIdx.x;
+    asm volatile("" : "+v"(t));
+    return t;
+  }
   // Queue the loads of W[k0 .. k0+KS)[n0 .. n0+64) (plain cached loads: weights are never written).
-  __device__ static __forceinline__ void issue_w(unsigned char *lds_w, const half_t *__restrict__ W, int ldw, int n0, int k0) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // `rot` rotates the order in which the rows are requested: workgroups of one XCD that load
+  // the same slice start at different rows, so at any moment they ask their L2 for different
+  // lines and everybody but the first requester of a line hits.
+  __device__ static __forceinline__ void issue_w(unsigned char *lds_w, const half_t *__restrict__ W, int ldw, int n0, int k0, int rot = 0) {
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
 #pragma unroll
-    for (int q = 0; q < W_INSTR / 4; ++q) {
+    for (int q0 = 0; q0 < W_INSTR / 4; ++q0) {
+      int q = q0 + rot;
+      if (q >= W_INSTR / 4) q -= W_INSTR / 4;
       const int inst = q * 4 + wave, s = inst * 64 + lane, k = s >> 3, c = (s & 7) ^ (k & 2);
+      __builtin_amdgcn_global_load_lds((gptr_t)(W + (size_t)(k0 + k) * ldw + n0 + c * 8), (lptr_t)(lds_w + inst * 1024), 16, 0, 0);
+    }
+  }
+  // The same slice queued by waves 1..3 only (PREFETCH_INSTR loads each): wave 0 polls the grid
+  // barrier, and its polling loads must not queue up behind a weight slice that is still in flight.
+  static constexpr int PREFETCH_INSTR = W_INSTR / 3;
+  static_assert(W_INSTR % 3 == 0 && PREFETCH_INSTR < 64, "prefetch split over three waves");
+  __device__ static __forceinline__ void issue_w_prefetch(unsigned char *lds_w, const half_t *__restrict__ W, int ldw, int n0, int k0) {
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
+    if (wave == 0) return;
+#pragma unroll
+    for (int q = 0; q < PREFETCH_INSTR; ++q) {
+      const int inst = q * 3 + wave - 1, s = inst * 64 + lane, k = s >> 3, c = (s & 7) ^ (k & 2);
       __builtin_amdgcn_global_load_lds((gptr_t)(W + (size_t)(k0 + k) * ldw + n0 + c * 8), (lptr_t)(lds_w + inst * 1024), 16, 0, 0);
     }
   }
   // Queue the loads of X[m0 .. m0+BM)[k0 .. k0+KS); COH selects agent-coherent loads.
   template <bool COH>
   __device__ static __forceinline__ void issue_x(unsigned char *lds_x, const half_t *X, int ldx, int m0, int k0) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
 #pragma unroll
     for (int q = 0; q < X_INSTR / 4; ++q) {
       const int inst = q * 4 + wave, s = inst * 64 + lane, r = s / XGR, j = (s % XGR) ^ (r & 15);
@@ -68,14 +93,14 @@ struct GemmOneShot {
     __syncthreads();
   }
 
-  // MFMA over this wave's share of the slice; then every wave is done reading X and W
-  // (so the caller may queue new loads into the W region), the partial tiles are summed
-  // through the X region, and epi(m, n, v) is called with v[i] = Y[m][n+i], i = 0..3,
-  // m and n relative to the tile origin, CPT/4 times per thread.
-  template <class AfterMfma, class Epi>
-  __device__ static __forceinline__ void compute(unsigned char *lds_x, const unsigned char *lds_w, AfterMfma after_mfma, Epi epi) {
+  // MFMA over this wave's share of the slice; then every wave is done reading X and W, the
+  // partial tiles are summed through the X region, and epi(m, n, v) is called with
+  // v[i] = Y[m][n+i], i = 0..3, m and n relative to the tile origin, CPT/4 times per thread.
+  // On return the W region is free (new loads may be queued into it).
+  template <class Epi>
+  __device__ static __forceinline__ void compute(unsigned char *lds_x, const unsigned char *lds_w, Epi epi) {
     const half_t *xs = reinterpret_cast<const half_t *>(lds_x), *ws = reinterpret_cast<const half_t *>(lds_w);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+    const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
     const int wm = wave / WAVES_K, wk = wave % WAVES_K;
     f4 acc[2][4];
 #pragma unroll
@@ -105,7 +130,6 @@ struct GemmOneShot {
         for (int j = 0; j < 4; ++j) acc[i][j] = mfma_16x16x32(wop[j], xop[i], acc[i][j]);
     }
     __syncthreads();                       // X and W slices are dead from here on
-    after_mfma();
     float *red = reinterpret_cast<float *>(lds_x);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
