@@ -34,7 +34,8 @@ int device_facts(DeviceFacts *out) {
     if (hipGetDeviceProperties(&p, dev) != hipSuccess) { (void)hipGetLastError(); return fail(SOUFFLE_ERR_DEVICE, "hipGetDeviceProperties failed"); }
     if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
       return fail(SOUFFLE_ERR_DEVICE, "built for gfx950 only, device is %s", p.gcnArchName);
-    cached[dev].num_cus = p.multiProcessorCount;
+    // cooperative grids are sized by this number; the grid barrier has 256 arrival flags
+    cached[dev].num_cus = p.multiProcessorCount < 256 ? p.multiProcessorCount : 256;
     cached[dev].lds_per_cu = (int)p.maxSharedMemoryPerMultiProcessor;
     cached[dev].cooperative = p.cooperativeLaunch;
     strncpy(cached[dev].arch, p.gcnArchName, 63);

@@ -251,6 +251,39 @@ struct Fc2Items {
   }
 };
 
+// ---- weight streamers ----
+// With at most 128 rows no stage of the skinny path has more than 192 items, so on a 256-CU
+// grid the workgroups 192..255 (eight per XCD) never compute.  They run ahead instead: while
+// the others work on a stage they touch one word of every 128-byte line of the weight slices
+// that THEIR XCD will multiply in a later stage, so those slices are already in that XCD's L2
+// when the stage starts.  Waves 1..3 issue the touches (direct-to-LDS loads into a dummy
+// region: no destination registers, nothing ever waits for them except the throttle in
+// grid_sync); wave 0 only takes part in the grid barriers.
+constexpr int kFirstStreamer = 192, kStreamersPerXcd = 8, kStreamerThreads = 192;
+__device__ __forceinline__ bool is_streamer(int M) { return M <= 128 && gridDim.x == 256 && (int)blockIdx.x >= kFirstStreamer; }
+__device__ __forceinline__ void touch_line(const half_t *p, unsigned char *lds) {
+  typedef __attribute__((address_space(1))) const void *gptr_t;
+  typedef __attribute__((address_space(3))) void *lptr_t;
+  __builtin_amdgcn_global_load_lds((gptr_t)p, (lptr_t)(lds + (threadIdx.x >> 6) * 256), 4, 0, 0);
+}
+// Column slices of W[K=768][ldw]: slice cs (64 columns) is item slice `ws_base + cs`, owned by XCD (ws_base + cs) % 8.
+__device__ __forceinline__ void warm_col_slices(unsigned char *lds, const half_t *W, int ldw, int n_slices, int ws_base) {
+  if (threadIdx.x < 64) return;
+  const int xcd = blockIdx.x & 7, sidx = ((int)blockIdx.x - kFirstStreamer) >> 3;
+  const int k = sidx * kStreamerThreads + (int)threadIdx.x - 64;
+  if (k >= H) return;
+  for (int cs = 0; cs < n_slices; ++cs)
+    if (((ws_base + cs) & 7) == xcd) touch_line(W + (size_t)k * ldw + cs * 64, lds);
+}
+// FC2: item slice (cs, ks) is owned by XCD ks, i.e. rows [ks*384, ks*384+384) of every column slice.
+__device__ __forceinline__ void warm_fc2_slices(unsigned char *lds, const half_t *W) {
+  if (threadIdx.x < 64) return;
+  static_assert(kSplitFc2Small == 8, "one K slice per XCD");
+  const int xcd = blockIdx.x & 7, sidx = ((int)blockIdx.x - kFirstStreamer) >> 3;
+  for (int i = sidx * kStreamerThreads + (int)threadIdx.x - 64; i < OsFc2::kKS * (H / 64); i += kStreamersPerXcd * kStreamerThreads)
+    touch_line(W + (size_t)(xcd * OsFc2::kKS + i / (H / 64)) * H + (i % (H / 64)) * 64, lds);
+}
+
 // Whether the weight slice of the next stage is queued before the grid barrier.  Measured on
 // MI355X this does not pay: the CU's vector memory pipeline is in order across its waves, so
 // the barrier's own atomics and polling loads queue up behind the ~100 KB in flight and the
@@ -266,23 +299,41 @@ __device__ __forceinline__ bool preissue_w(unsigned char *lds, const Items &item
   return true;
 }
 
+// Fine-grained time stamps inside a stage (development builds only: they cost scalar registers).
+#ifdef SOUFFLE_STAGE_MARKS
+#define STAGE_MARK(tb, id) do { if (tb) trace_mark(*(tb), (id)); } while (0)
+#else
+#define STAGE_MARK(tb, id) do { (void)(tb); } while (0)
+#endif
+
 // Driver of a skinny GEMM stage.  `w_ready`: the weight slice of this workgroup's first item
 // was queued before the preceding grid barrier.  `pre(item)` runs after the operands have
-// landed (LayerNorm on load), `epi(item, m, n, v)` receives 4 consecutive columns of a row,
+// landed (LayerNorm on load), `epi(item, m, n, lo, hi)` receives 8 consecutive columns of a row,
 // `next()` queues the first weight slice of the FOLLOWING stage once the stage's stores are issued.
 template <class G, bool COH, class Items, class Pre, class Epi, class Next>
 __device__ __forceinline__ void gemm_stage(unsigned char *lds, const Items &items, const half_t *X, int ldx, bool w_ready,
-                                           Pre pre, Epi epi, Next next) {
+                                           Pre pre, Epi epi, Next next, const GridBarrier *tb = nullptr) {
   const int span = items.span();
   for (int it = blockIdx.x; it < span; it += gridDim.x) {
     Item d;
     if (!items.at(it, d)) { w_ready = false; continue; }
     __syncthreads();                       // LDS reuse
+    STAGE_MARK(tb, 0);
     if (!w_ready) G::issue_w(lds + kXRegion, d.W, d.ldw, d.n0, d.k0, d.rot);
     G::template issue_x<false>(lds, X, ldx, d.m0, d.k0);
+    STAGE_MARK(tb, 1);
+#ifdef SOUFFLE_STAGE_MARKS
+    if (tb && tb->trace) { wait_vmcnt<G::X_INSTR / 4>(); trace_mark(*tb, 2); }
+#endif
     G::wait_loads();
+    STAGE_MARK(tb, 3);
     pre(d);
-    G::compute(lds, lds + kXRegion, [&](int mm, int nn, f4 v) { epi(d, d.m0 + mm, d.n0 + nn, v); });
+    STAGE_MARK(tb, 4);
+    G::compute(lds, lds + kXRegion, [&](int mm, int nn, f4 lo, f4 hi) { epi(d, d.m0 + mm, d.n0 + nn, lo, hi); });
+    STAGE_MARK(tb, 5);
+#ifdef SOUFFLE_STAGE_MARKS
+    if (tb && tb->trace) { __builtin_amdgcn_s_waitcnt(0); trace_mark(*tb, 6); }
+#endif
     w_ready = false;
   }
   next();     // after the last store of the stage, so that only these loads are younger than it
@@ -294,6 +345,18 @@ __device__ __forceinline__ f4 add_bias4(f4 v, const half_t *bias, int n) {
     v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
   }
   return v;
+}
+
+__device__ __forceinline__ void add_bias8(f4 &lo, f4 &hi, const half_t *bias, int n) {
+  if (bias) {
+    const h8 bb = *reinterpret_cast<const h8 *>(bias + n);
+    lo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+    hi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]};
+  }
+}
+__device__ __forceinline__ u4 pack_h8(f4 lo, f4 hi) {
+  const h8 r = {(half_t)lo[0], (half_t)lo[1], (half_t)lo[2], (half_t)lo[3], (half_t)hi[0], (half_t)hi[1], (half_t)hi[2], (half_t)hi[3]};
+  return as_u4(r);
 }
 
 // LayerNorm of the 32 complete rows of an OsFull X tile, in place in LDS.  Eight lanes
@@ -358,43 +421,50 @@ __device__ __forceinline__ void stage_ln(const Params &a, int splitk, const half
 
 // The four skinny GEMM stages (shared by the megakernel and the per-op kernels).
 template <bool COH, class Next>
-__device__ __forceinline__ void small_qkv(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, Next next) {
+__device__ __forceinline__ void small_qkv(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, Next next, const GridBarrier *tb = nullptr) {
   gemm_stage<OsFull, COH>(lds, QkvItems{w.w_qkv, a.M}, xin, H, w_ready, [](const Item &) {},
-    [&](const Item &d, int m, int n, f4 v) {
-      v = add_bias4(v, w.b_qkv ? w.b_qkv + d.aux * H : nullptr, n);
+    [&](const Item &d, int m, int n, f4 lo, f4 hi) {
+      add_bias8(lo, hi, w.b_qkv ? w.b_qkv + d.aux * H : nullptr, n);
       const int b = m / a.S, s = m % a.S, hh = n / HD, dd = n % HD;
-      st8<COH>(a.qkv, ((((d.aux * a.B + b) * NH + hh) * a.S + s) * HD + dd) * 2, pack_h4(v));
-    }, next);
+      st16<COH>(a.qkv, ((((d.aux * a.B + b) * NH + hh) * a.S + s) * HD + dd) * 2, pack_h8(lo, hi));
+    }, next, tb);
 }
 // z1 = ctx.Wo + b_o + x (pre-LayerNorm, fp16)
 template <bool COH, class Next>
-__device__ __forceinline__ void small_outproj(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, Next next) {
+__device__ __forceinline__ void small_outproj(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, Next next, const GridBarrier *tb = nullptr) {
   gemm_stage<OsFull, COH>(lds, OutItems{w.w_o, a.M}, a.ctx, H, w_ready, [](const Item &) {},
-    [&](const Item &, int m, int n, f4 v) {
-      v = add_bias4(v, w.b_o, n);
-      const h4 r = as_h4(ld8<false>(xin, (m * H + n) * 2));
-      v += f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
-      st8<COH>(a.z1, (m * H + n) * 2, pack_h4(v));
-    }, next);
+    [&](const Item &, int m, int n, f4 lo, f4 hi) {
+      add_bias8(lo, hi, w.b_o, n);
+      const h8 r = as_h8(ld16<false>(xin, (m * H + n) * 2));
+      lo += f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+      hi += f4{(float)r[4], (float)r[5], (float)r[6], (float)r[7]};
+      st16<COH>(a.z1, (m * H + n) * 2, pack_h8(lo, hi));
+    }, next, tb);
 }
 // h = act(LN1(z1).W1 + b1): LayerNorm is applied to the X tile in LDS (every workgroup has
 // complete rows); the workgroups of the first n-tile also publish y1 = LN1(z1).
 template <bool COH, class Next>
-__device__ __forceinline__ void small_fc1(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, Next next) {
+__device__ __forceinline__ void small_fc1(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, Next next, const GridBarrier *tb = nullptr) {
   gemm_stage<OsFull, COH>(lds, Fc1Items{w.w_fc1, a.M}, a.z1, H, w_ready,
     [&](const Item &d) { ln_rows_in_lds<COH>(lds, w.ln1_g, w.ln1_b, a.eps, d.n0 == 0 ? a.y1 : nullptr, d.m0); },
-    [&](const Item &, int m, int n, f4 v) {
-      v = add_bias4(v, w.b_fc1, n);
+    [&](const Item &, int m, int n, f4 lo, f4 hi) {
+      add_bias8(lo, hi, w.b_fc1, n);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(v[i], 0.f) : gelu_tanh(v[i]);
-      st8<COH>(a.h, (m * F + n) * 2, pack_h4(v));
-    }, next);
+      for (int i = 0; i < 4; ++i) {
+        lo[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(lo[i], 0.f) : gelu_tanh(lo[i]);
+        hi[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(hi[i], 0.f) : gelu_tanh(hi[i]);
+      }
+      st16<COH>(a.h, (m * F + n) * 2, pack_h8(lo, hi));
+    }, next, tb);
 }
 // fp32 partials of h.W2 over 8 K slices
 template <bool COH, class Next>
-__device__ __forceinline__ void small_fc2(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, Next next) {
+__device__ __forceinline__ void small_fc2(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, Next next, const GridBarrier *tb = nullptr) {
   gemm_stage<OsFc2, COH>(lds, Fc2Items{w.w_fc2, a.M}, a.h, F, w_ready, [](const Item &) {},
-    [&](const Item &d, int m, int n, f4 v) { st16<COH>(a.part, ((d.aux * a.M + m) * H + n) * 4, __builtin_bit_cast(u4, v)); }, next);
+    [&](const Item &d, int m, int n, f4 lo, f4 hi) {
+      st16<COH>(a.part, ((d.aux * a.M + m) * H + n) * 4, __builtin_bit_cast(u4, lo));
+      st16<COH>(a.part, ((d.aux * a.M + m) * H + n + 4) * 4, __builtin_bit_cast(u4, hi));
+    }, next, tb);
 }
 
 // One (batch, head, 64-query block) per workgroup pass; each wave owns 16 queries.
@@ -566,25 +636,41 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       // Weight slices are queued one stage ahead: right after a stage's MFMA loop has
       // released the W region, the slice of the next stage is requested, so it crosses HBM
       // while the epilogue stores drain and the grid barrier is crossed.
+      if (is_streamer(a.M)) {
+        // Weight traffic is moved into the stages that leave HBM idle; every slice is requested
+        // at least one full stage before it is multiplied.
+        grid_sync(bar, 16);                                           // QKV runs
+        warm_col_slices(lds_raw, w.w_o, H, H / 64, 0);
+        warm_col_slices(lds_raw, w.w_fc1, F, F / 64, 0);
+        grid_sync(bar, 16);                                           // attention runs
+        warm_fc2_slices(lds_raw, w.w_fc2);
+        grid_sync(bar, 16);                                           // out-projection runs
+        if (l + 1 < a.num_layers)
+          for (int j = 0; j < 3; ++j) warm_col_slices(lds_raw, args.layers[l + 1].w_qkv + (size_t)j * H * H, H, H / 64, j * (H / 64));
+        grid_sync(bar, 16);                                           // FC1 runs
+        grid_sync(bar, 16);                                           // FC2 runs
+        if (l + 1 < a.num_layers) grid_sync(bar, 16);                 // LayerNorm 2 runs
+        continue;
+      }
       const bool attn_fits = 2 * a.S * 128 + 64 * 128 <= kXRegion;   // attention tiles stay below the W region
       const OutItems out_items{w.w_o, a.M};
       const Fc1Items fc1_items{w.w_fc1, a.M};
       const Fc2Items fc2_items{w.w_fc2, a.M};
       bool out_ready = false;
-      small_qkv<true>(lds_raw, a, w, xin, qkv_ready, [&]() { if (attn_fits) out_ready = preissue_w<OsFull>(lds_raw, out_items); });
+      small_qkv<true>(lds_raw, a, w, xin, qkv_ready, [&]() { if (attn_fits) out_ready = preissue_w<OsFull>(lds_raw, out_items); }, &bar);
       grid_sync(bar, out_ready ? OsFull::PREFETCH_INSTR : 0);
       stage_attn_t<true, NKT>(lds, a, first, stride);
       if (!attn_fits) { __syncthreads(); out_ready = preissue_w<OsFull>(lds_raw, out_items); }
       grid_sync(bar, attn_fits ? 0 : (out_ready ? OsFull::PREFETCH_INSTR : 0));
       bool fc1_ready = false, fc2_ready = false;
-      small_outproj<true>(lds_raw, a, w, xin, out_ready, [&]() { fc1_ready = preissue_w<OsFull>(lds_raw, fc1_items); });
+      small_outproj<true>(lds_raw, a, w, xin, out_ready, [&]() { fc1_ready = preissue_w<OsFull>(lds_raw, fc1_items); }, &bar);
       grid_sync(bar, fc1_ready ? OsFull::PREFETCH_INSTR : 0);
-      small_fc1<true>(lds_raw, a, w, fc1_ready, [&]() { fc2_ready = preissue_w<OsFc2>(lds_raw, fc2_items); });
+      small_fc1<true>(lds_raw, a, w, fc1_ready, [&]() { fc2_ready = preissue_w<OsFc2>(lds_raw, fc2_items); }, &bar);
       grid_sync(bar, fc2_ready ? OsFc2::PREFETCH_INSTR : 0);
       qkv_ready = false;
       small_fc2<true>(lds_raw, a, w, fc2_ready, [&]() {
         if (l + 1 < a.num_layers) qkv_ready = preissue_w<OsFull>(lds_raw, QkvItems{args.layers[l + 1].w_qkv, a.M});
-      });
+      }, &bar);
       grid_sync(bar, qkv_ready ? OsFull::PREFETCH_INSTR : 0);
       stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
     }

@@ -127,27 +127,34 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 }
 
 // -------------------------------------------------------- grid barrier ----
-// One arrival counter per XCD (workgroup b runs on XCD b % 8 and adds 1 to counter b % 8
-// with a relaxed agent-scope atomic whose result is not awaited) and no release flag:
-// every workgroup polls all eight counters with one 8-lane load until each has reached its
-// target.  Counters only ever grow and are compared as signed differences, so a fast
-// workgroup arriving at the next barrier never disturbs a slow one that is still polling.
-// The critical path is one atomic on its way to memory plus one polling round trip.
+// Two kinds of words, never mixed on one cache line:
+//  * arrival counter x (x = workgroup % 8, the XCD the workgroup runs on): incremented with an
+//    atomic whose result IS awaited, and read by nobody else.  The line therefore stays with
+//    the L2 of that XCD and the increments of its workgroups do not compete with pollers for it
+//    (with polled counters every poll from another XCD pulls the line away between two
+//    increments, and a barrier after a balanced stage takes 4 us instead of 1.5);
+//  * done flag x: the workgroup whose increment completes the count of XCD x stores the barrier
+//    number there once (write-through), and every workgroup polls the eight flags with one
+//    8-lane load until all have reached that number.
+// Counters and barrier numbers only grow (across launches too) and are compared as signed
+// differences, so a fast workgroup arriving at the next barrier never disturbs a slow one.
 // Control block (uint32 words, zeroed once before first use):
-//   [32*x]        arrival counter of XCD x, x < 8 (one 128-byte line each)
-//   [256 + 32*x]  value counter x holds between launches; rewritten by grid_barrier_end()
-//                 (all workgroups read it before their first arrival, nobody writes it
-//                 before the last barrier of the launch has completed)
-//   [48]          sticky error flag for kernels with bounded spin loops
-// All data exchanged across a barrier must be written with st*<true> and read with
-// ld*<true>; the barrier itself carries no cache write-back or invalidate.
+//   [32*x]        arrival counter x              [256 + 32*x]  done flag x
+//   [384 + x]     value counter x holds between launches, [392] barrier number between launches:
+//                 rewritten by grid_barrier_end() (all workgroups read them before their first
+//                 arrival, nobody writes them before the last barrier of the launch has completed)
+//   [kCtlErrWord] sticky error flag for kernels with bounded spin loops
+// Data exchanged across a barrier must be written with st*<true> (write-through); the barrier
+// itself carries no cache write-back or invalidate.
 constexpr int kCtlWords = 512;
+constexpr int kCtlErrWord = 400;
 constexpr int kMaxBarrierSpin = 1 << 24;
 
 struct GridBarrier {
   unsigned *ctl;
-  unsigned target;   // lane x < 8 of wave 0: value counter x reaches at the next barrier
-  unsigned gsz;      // lane x < 8 of wave 0: workgroups on XCD x
+  unsigned target;   // value this workgroup's arrival counter holds once its XCD is complete
+  unsigned gsz;      // workgroups that share this workgroup's counter
+  unsigned epoch;    // number of the last barrier passed
   unsigned nblk;
   int count;         // barriers passed in this launch
   // optional stage trace: thread 0 stamps the 100 MHz wall clock on entry to and exit from
@@ -170,9 +177,10 @@ __device__ __forceinline__ void grid_barrier_begin(GridBarrier &b, unsigned *ctl
   b.trace = nullptr;
   b.trace_idx = 0;
   b.trace_cap = 0;
-  const unsigned x = threadIdx.x & 7;
+  const unsigned x = blockIdx.x & 7;
   b.gsz = (b.nblk + 7 - x) >> 3;
-  b.target = __hip_atomic_load(ctl + 256 + 32 * x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  b.target = __hip_atomic_load(ctl + 384 + x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  b.epoch = __hip_atomic_load(ctl + 392, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // s_waitcnt with only the vector-memory counter: all but the youngest N vector memory
@@ -195,14 +203,21 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b, int pending = 0) {
   else if (pending == 16) wait_vmcnt<16>();
   else __builtin_amdgcn_s_waitcnt(0);
   __builtin_amdgcn_s_barrier();
+#ifdef SOUFFLE_STAGE_MARKS
+  trace_mark(b, 7);
+#endif
   b.target += b.gsz;
+  b.epoch += 1;
   if (threadIdx.x < 64) {
-    if (threadIdx.x == 0)
-      (void)__hip_atomic_fetch_add(b.ctl + 32 * (blockIdx.x & 7), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) {
+      const unsigned x = blockIdx.x & 7;
+      const unsigned old = __hip_atomic_fetch_add(b.ctl + 32 * x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (old + 1 == b.target) __hip_atomic_store(b.ctl + 256 + 32 * x, b.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     for (int spin = 0; spin < kMaxBarrierSpin; ++spin) {
       bool ok = true;
-      if (threadIdx.x < 8)
-        ok = (int)(__hip_atomic_load(b.ctl + 32 * threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - b.target) >= 0;
+      if (threadIdx.x < 8 && threadIdx.x < b.nblk)
+        ok = (int)(__hip_atomic_load(b.ctl + 256 + 32 * threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - b.epoch) >= 0;
       if (__all(ok)) break;
       __builtin_amdgcn_s_sleep(1);
     }
@@ -216,8 +231,10 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b, int pending = 0) {
 
 // Call once by every workgroup before the kernel returns.
 __device__ __forceinline__ void grid_barrier_end(GridBarrier &b) {
-  if (b.count > 0 && blockIdx.x < 8 && threadIdx.x == blockIdx.x)
-    __hip_atomic_store(b.ctl + 256 + 32 * blockIdx.x, b.target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (b.count > 0 && blockIdx.x < 8 && threadIdx.x == 0) {
+    __hip_atomic_store(b.ctl + 384 + blockIdx.x, b.target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (blockIdx.x == 0) __hip_atomic_store(b.ctl + 392, b.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
 }  // namespace souffle

@@ -94,8 +94,9 @@ struct GemmOneShot {
   }
 
   // MFMA over this wave's share of the slice; then every wave is done reading X and W, the
-  // partial tiles are summed through the X region, and epi(m, n, v) is called with
-  // v[i] = Y[m][n+i], i = 0..3, m and n relative to the tile origin, CPT/4 times per thread.
+  // partial tiles are summed through the X region, and epi(m, n, lo, hi) is called with
+  // lo[i] = Y[m][n+i], hi[i] = Y[m][n+4+i], i = 0..3 (8 consecutive columns of one row, m and n
+  // relative to the tile origin), CPT/8 times per thread.
   // On return the W region is free (new loads may be queued into it).
   template <class Epi>
   __device__ static __forceinline__ void compute(unsigned char *lds_x, const unsigned char *lds_w, Epi epi) {
@@ -140,11 +141,15 @@ struct GemmOneShot {
     constexpr int TPR = 64 / CPT;           // threads per output row
     const int row = tid / TPR, col0 = (tid % TPR) * CPT;
 #pragma unroll
-    for (int c = 0; c < CPT / 4; ++c) {
-      f4 v = *reinterpret_cast<const f4 *>(red + row * RED_LD + col0 + c * 4);
+    for (int c = 0; c < CPT / 8; ++c) {
+      const float *src = red + row * RED_LD + col0 + c * 8;
+      f4 lo = *reinterpret_cast<const f4 *>(src), hi = *reinterpret_cast<const f4 *>(src + 4);
 #pragma unroll
-      for (int w = 1; w < WAVES_K; ++w) v += *reinterpret_cast<const f4 *>(red + (w * BM + row) * RED_LD + col0 + c * 4);
-      epi(row, col0 + c * 4, v);
+      for (int w = 1; w < WAVES_K; ++w) {
+        lo += *reinterpret_cast<const f4 *>(src + w * BM * RED_LD);
+        hi += *reinterpret_cast<const f4 *>(src + w * BM * RED_LD + 4);
+      }
+      epi(row, col0 + c * 8, lo, hi);
     }
   }
 };

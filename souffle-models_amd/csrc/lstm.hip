@@ -29,7 +29,7 @@ struct Args {
   const float *bias, *x;
   float *y;
   u2 *hbuf;          // [layers][timesteps][256] of (value bits, step tag)
-  unsigned *ctl;     // grid-barrier control block; word 48 = sticky error flag
+  unsigned *ctl;     // grid-barrier control block; word kCtlErrWord = sticky error flag
 };
 
 __device__ __forceinline__ float sigmoidf_(float v) { return 1.0f / (1.0f + __expf(-v)); }
@@ -116,7 +116,7 @@ __global__ void __launch_bounds__(256) k_lstm(Args a) {
       if (l == a.layers - 1) a.y[(size_t)t * HID + unit] = h;
     }
   }
-  if (failed) atomicOr(a.ctl + 48, 1u);
+  if (failed) atomicOr(a.ctl + kCtlErrWord, 1u);
   // everything has been consumed once every workgroup is here: clear this workgroup's
   // published slots so that the next launch (or a graph replay) starts from empty tags
   grid_sync(bar);
