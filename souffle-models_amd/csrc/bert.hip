@@ -183,7 +183,8 @@ using OsFc2 = GemmOneShot<64, 384>;     // FC2: 8 K slices as fp32 partials
 constexpr int kSplitFc2Small = F / OsFc2::kKS;
 constexpr int kXRegion = 49152;         // LDS: [0, 48 KB) X slice / attention tiles / reduction, [48 KB, 144 KB) W slice
 static_assert(OsFull::X_BYTES <= kXRegion && OsFc2::X_BYTES <= kXRegion, "X region");
-constexpr int kSmallGemmLds = kXRegion + (OsFull::W_BYTES > OsFc2::W_BYTES ? OsFull::W_BYTES : OsFc2::W_BYTES);
+constexpr int kLnParamOff = kXRegion + (OsFull::W_BYTES > OsFc2::W_BYTES ? OsFull::W_BYTES : OsFc2::W_BYTES);   // gamma[768], beta[768]
+constexpr int kSmallGemmLds = kLnParamOff + 2 * H * 2;
 
 // One work item of a skinny GEMM stage: output tile origin, weight slice, activation slice.
 struct Item {
@@ -251,51 +252,17 @@ struct Fc2Items {
   }
 };
 
-// ---- weight streamers ----
-// With at most 128 rows no stage of the skinny path has more than 192 items, so on a 256-CU
-// grid the workgroups 192..255 (eight per XCD) never compute.  They run ahead instead: while
-// the others work on a stage they touch one word of every 128-byte line of the weight slices
-// that THEIR XCD will multiply in a later stage, so those slices are already in that XCD's L2
-// when the stage starts.  Waves 1..3 issue the touches (direct-to-LDS loads into a dummy
-// region: no destination registers, nothing ever waits for them except the throttle in
-// grid_sync); wave 0 only takes part in the grid barriers.
-constexpr int kFirstStreamer = 192, kStreamersPerXcd = 8, kStreamerThreads = 192;
-__device__ __forceinline__ bool is_streamer(int M) { return M <= 128 && gridDim.x == 256 && (int)blockIdx.x >= kFirstStreamer; }
-__device__ __forceinline__ void touch_line(const half_t *p, unsigned char *lds) {
-  typedef __attribute__((address_space(1))) const void *gptr_t;
-  typedef __attribute__((address_space(3))) void *lptr_t;
-  __builtin_amdgcn_global_load_lds((gptr_t)p, (lptr_t)(lds + (threadIdx.x >> 6) * 256), 4, 0, 0);
-}
-// Column slices of W[K=768][ldw]: slice cs (64 columns) is item slice `ws_base + cs`, owned by XCD (ws_base + cs) % 8.
-__device__ __forceinline__ void warm_col_slices(unsigned char *lds, const half_t *W, int ldw, int n_slices, int ws_base) {
-  if (threadIdx.x < 64) return;
-  const int xcd = blockIdx.x & 7, sidx = ((int)blockIdx.x - kFirstStreamer) >> 3;
-  const int k = sidx * kStreamerThreads + (int)threadIdx.x - 64;
-  if (k >= H) return;
-  for (int cs = 0; cs < n_slices; ++cs)
-    if (((ws_base + cs) & 7) == xcd) touch_line(W + (size_t)k * ldw + cs * 64, lds);
-}
-// FC2: item slice (cs, ks) is owned by XCD ks, i.e. rows [ks*384, ks*384+384) of every column slice.
-__device__ __forceinline__ void warm_fc2_slices(unsigned char *lds, const half_t *W) {
-  if (threadIdx.x < 64) return;
-  static_assert(kSplitFc2Small == 8, "one K slice per XCD");
-  const int xcd = blockIdx.x & 7, sidx = ((int)blockIdx.x - kFirstStreamer) >> 3;
-  for (int i = sidx * kStreamerThreads + (int)threadIdx.x - 64; i < OsFc2::kKS * (H / 64); i += kStreamersPerXcd * kStreamerThreads)
-    touch_line(W + (size_t)(xcd * OsFc2::kKS + i / (H / 64)) * H + (i % (H / 64)) * 64, lds);
-}
-
-// Whether the weight slice of the next stage is queued before the grid barrier.  Measured on
-// MI355X this does not pay: the CU's vector memory pipeline is in order across its waves, so
-// the barrier's own atomics and polling loads queue up behind the ~100 KB in flight and the
-// barrier stretches by as much as the prefetch saves.
-constexpr bool kPrefetchAcrossBarrier = false;
+// The weight slice of a workgroup's first item of the NEXT stage is queued from inside the grid
+// barrier (after the arrival, before the wait), by waves 1..3: it needs nothing from other
+// workgroups, and the ~1.3 us its requests take to issue are hidden in the barrier.
+constexpr bool kPrefetchAcrossBarrier = true;
 
 // Queue the weight slice of this workgroup's first item of a stage (if it has one).
 template <class G, class Items>
 __device__ __forceinline__ bool preissue_w(unsigned char *lds, const Items &items) {
   Item d;
   if (!kPrefetchAcrossBarrier || (int)blockIdx.x >= items.span() || !items.at(blockIdx.x, d)) return false;
-  G::issue_w_prefetch(lds + kXRegion, d.W, d.ldw, d.n0, d.k0);
+  G::issue_w_prefetch(lds + kXRegion, d.W, d.ldw, d.n0, d.k0, d.rot);
   return true;
 }
 
@@ -307,12 +274,12 @@ __device__ __forceinline__ bool preissue_w(unsigned char *lds, const Items &item
 #endif
 
 // Driver of a skinny GEMM stage.  `w_ready`: the weight slice of this workgroup's first item
-// was queued before the preceding grid barrier.  `pre(item)` runs after the operands have
+// was queued inside the preceding grid barrier.  `extra()` queues further direct-to-LDS loads
+// with the operands, `pre(item)` runs after the operands have
 // landed (LayerNorm on load), `epi(item, m, n, lo, hi)` receives 8 consecutive columns of a row,
-// `next()` queues the first weight slice of the FOLLOWING stage once the stage's stores are issued.
-template <class G, bool COH, class Items, class Pre, class Epi, class Next>
+template <class G, bool COH, class Items, class Extra, class Pre, class Epi>
 __device__ __forceinline__ void gemm_stage(unsigned char *lds, const Items &items, const half_t *X, int ldx, bool w_ready,
-                                           Pre pre, Epi epi, Next next, const GridBarrier *tb = nullptr) {
+                                           Extra extra, Pre pre, Epi epi, const GridBarrier *tb = nullptr) {
   const int span = items.span();
   for (int it = blockIdx.x; it < span; it += gridDim.x) {
     Item d;
@@ -321,6 +288,7 @@ __device__ __forceinline__ void gemm_stage(unsigned char *lds, const Items &item
     STAGE_MARK(tb, 0);
     if (!w_ready) G::issue_w(lds + kXRegion, d.W, d.ldw, d.n0, d.k0, d.rot);
     G::template issue_x<false>(lds, X, ldx, d.m0, d.k0);
+    extra();
     STAGE_MARK(tb, 1);
 #ifdef SOUFFLE_STAGE_MARKS
     if (tb && tb->trace) { wait_vmcnt<G::X_INSTR / 4>(); trace_mark(*tb, 2); }
@@ -336,7 +304,6 @@ __device__ __forceinline__ void gemm_stage(unsigned char *lds, const Items &item
 #endif
     w_ready = false;
   }
-  next();     // after the last store of the stage, so that only these loads are younger than it
 }
 
 __device__ __forceinline__ f4 add_bias4(f4 v, const half_t *bias, int n) {
@@ -362,22 +329,40 @@ __device__ __forceinline__ u4 pack_h8(f4 lo, f4 hi) {
 // LayerNorm of the 32 complete rows of an OsFull X tile, in place in LDS.  Eight lanes
 // share a row; slot s of row r holds columns 8*(s ^ (r & 15)) .. +7.  Statistics and the
 // normalisation (one FMA per element) are fp32.  When `out` is given the normalised rows are also written to out[m0 + r][:].
+// gamma and beta come from LDS (queued with the operands by issue_ln_params), not from global
+// memory: a dependent global load after the row statistics would cost another memory latency.
+__device__ __forceinline__ void issue_ln_params(unsigned char *lds, const half_t *gam, const half_t *bet) {
+  typedef __attribute__((address_space(1))) const void *gptr_t;
+  typedef __attribute__((address_space(3))) void *lptr_t;
+  const int tid = threadIdx.x, wave = tid >> 6;       // 192 slots of 16 bytes: gamma 0..95, beta 96..191
+  if (wave < 3) {
+    const int s = tid;
+    const half_t *src = s < 96 ? (gam ? gam + s * 8 : nullptr) : (bet ? bet + (s - 96) * 8 : nullptr);
+    if (src) __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + kLnParamOff + wave * 1024), 16, 0, 0);
+  }
+}
 template <bool COH>
-__device__ __forceinline__ void ln_rows_in_lds(unsigned char *lds_x, const half_t *gam, const half_t *bet, float eps,
+__device__ __forceinline__ void ln_rows_in_lds(unsigned char *lds_x, bool has_gam, bool has_bet, float eps,
                                                half_t *out, int m0) {
   constexpr int XGR = OsFull::XGR, PER = XGR / 8;
   const int tid = threadIdx.x, r = tid >> 3, t8 = tid & 7;
   h8 *row = reinterpret_cast<h8 *>(lds_x) + r * XGR;
-  float f[PER][8];
+  const half_t *gam = has_gam ? reinterpret_cast<const half_t *>(lds_x + kLnParamOff) : nullptr;
+  const half_t *bet = has_bet ? reinterpret_cast<const half_t *>(lds_x + kLnParamOff + H * 2) : nullptr;
+  // Statistics with the packed dot product (fp16 products are exact in fp32, fp32 accumulation),
+  // normalisation with two mixed-precision FMAs per element (fp16 operands, fp32 arithmetic,
+  // one rounding at the end): the stage is bound by vector ALU issue, not by LDS.
+  h8 x[PER];
   float sum = 0.f, sq = 0.f;
+  const h2 ones = {(half_t)1.f, (half_t)1.f};
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
-    const h8 x = row[t8 + 8 * i];
+    x[i] = row[t8 + 8 * i];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      f[i][e] = (float)x[e];
-      sum += f[i][e];
-      sq += f[i][e] * f[i][e];
+    for (int e = 0; e < 8; e += 2) {
+      const h2 p = {x[i][e], x[i][e + 1]};
+      sum = __builtin_amdgcn_fdot2(p, ones, sum, false);
+      sq = __builtin_amdgcn_fdot2(p, p, sq, false);
     }
   }
   sum += wave_xor(sum, 1); sum += wave_xor(sum, 2); sum += wave_xor(sum, 4);
@@ -397,14 +382,12 @@ __device__ __forceinline__ void ln_rows_in_lds(unsigned char *lds_x, const half_
       if (bet) b8 = *reinterpret_cast<const h8 *>(bet + k);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        float t = f[i][e] * rstd + shift;
-        if (gam) t *= (float)g8[e];
-        if (bet) t += (float)b8[e];
-        o[e] = (half_t)t;
+        const float t = __builtin_fmaf((float)x[i][e], rstd, shift);
+        o[e] = (half_t)__builtin_fmaf(t, gam ? (float)g8[e] : 1.0f, bet ? (float)b8[e] : 0.0f);
       }
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = (half_t)(f[i][e] * rstd + shift);
+      for (int e = 0; e < 8; ++e) o[e] = (half_t)__builtin_fmaf((float)x[i][e], rstd, shift);
     }
     row[sl] = o;
     if (out) st16<COH>(out, ((m0 + r) * H + k) * 2, as_u4(o));
@@ -420,33 +403,34 @@ __device__ __forceinline__ void stage_ln(const Params &a, int splitk, const half
 }
 
 // The four skinny GEMM stages (shared by the megakernel and the per-op kernels).
-template <bool COH, class Next>
-__device__ __forceinline__ void small_qkv(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, Next next, const GridBarrier *tb = nullptr) {
-  gemm_stage<OsFull, COH>(lds, QkvItems{w.w_qkv, a.M}, xin, H, w_ready, [](const Item &) {},
+template <bool COH>
+__device__ __forceinline__ void small_qkv(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, const GridBarrier *tb = nullptr) {
+  gemm_stage<OsFull, COH>(lds, QkvItems{w.w_qkv, a.M}, xin, H, w_ready, []() {}, [](const Item &) {},
     [&](const Item &d, int m, int n, f4 lo, f4 hi) {
       add_bias8(lo, hi, w.b_qkv ? w.b_qkv + d.aux * H : nullptr, n);
       const int b = m / a.S, s = m % a.S, hh = n / HD, dd = n % HD;
       st16<COH>(a.qkv, ((((d.aux * a.B + b) * NH + hh) * a.S + s) * HD + dd) * 2, pack_h8(lo, hi));
-    }, next, tb);
+    }, tb);
 }
 // z1 = ctx.Wo + b_o + x (pre-LayerNorm, fp16)
-template <bool COH, class Next>
-__device__ __forceinline__ void small_outproj(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, Next next, const GridBarrier *tb = nullptr) {
-  gemm_stage<OsFull, COH>(lds, OutItems{w.w_o, a.M}, a.ctx, H, w_ready, [](const Item &) {},
+template <bool COH>
+__device__ __forceinline__ void small_outproj(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, const GridBarrier *tb = nullptr) {
+  gemm_stage<OsFull, COH>(lds, OutItems{w.w_o, a.M}, a.ctx, H, w_ready, []() {}, [](const Item &) {},
     [&](const Item &, int m, int n, f4 lo, f4 hi) {
       add_bias8(lo, hi, w.b_o, n);
       const h8 r = as_h8(ld16<false>(xin, (m * H + n) * 2));
       lo += f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
       hi += f4{(float)r[4], (float)r[5], (float)r[6], (float)r[7]};
       st16<COH>(a.z1, (m * H + n) * 2, pack_h8(lo, hi));
-    }, next, tb);
+    }, tb);
 }
 // h = act(LN1(z1).W1 + b1): LayerNorm is applied to the X tile in LDS (every workgroup has
 // complete rows); the workgroups of the first n-tile also publish y1 = LN1(z1).
-template <bool COH, class Next>
-__device__ __forceinline__ void small_fc1(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, Next next, const GridBarrier *tb = nullptr) {
+template <bool COH>
+__device__ __forceinline__ void small_fc1(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, const GridBarrier *tb = nullptr) {
   gemm_stage<OsFull, COH>(lds, Fc1Items{w.w_fc1, a.M}, a.z1, H, w_ready,
-    [&](const Item &d) { ln_rows_in_lds<COH>(lds, w.ln1_g, w.ln1_b, a.eps, d.n0 == 0 ? a.y1 : nullptr, d.m0); },
+    [&]() { issue_ln_params(lds, w.ln1_g, w.ln1_b); },
+    [&](const Item &d) { ln_rows_in_lds<COH>(lds, w.ln1_g != nullptr, w.ln1_b != nullptr, a.eps, d.n0 == 0 ? a.y1 : nullptr, d.m0); },
     [&](const Item &, int m, int n, f4 lo, f4 hi) {
       add_bias8(lo, hi, w.b_fc1, n);
 #pragma unroll
@@ -455,16 +439,16 @@ __device__ __forceinline__ void small_fc1(unsigned char *lds, const Params &a, c
         hi[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(hi[i], 0.f) : gelu_tanh(hi[i]);
       }
       st16<COH>(a.h, (m * F + n) * 2, pack_h8(lo, hi));
-    }, next, tb);
+    }, tb);
 }
 // fp32 partials of h.W2 over 8 K slices
-template <bool COH, class Next>
-__device__ __forceinline__ void small_fc2(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, Next next, const GridBarrier *tb = nullptr) {
-  gemm_stage<OsFc2, COH>(lds, Fc2Items{w.w_fc2, a.M}, a.h, F, w_ready, [](const Item &) {},
+template <bool COH>
+__device__ __forceinline__ void small_fc2(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, const GridBarrier *tb = nullptr) {
+  gemm_stage<OsFc2, COH>(lds, Fc2Items{w.w_fc2, a.M}, a.h, F, w_ready, []() {}, [](const Item &) {},
     [&](const Item &d, int m, int n, f4 lo, f4 hi) {
       st16<COH>(a.part, ((d.aux * a.M + m) * H + n) * 4, __builtin_bit_cast(u4, lo));
       st16<COH>(a.part, ((d.aux * a.M + m) * H + n + 4) * 4, __builtin_bit_cast(u4, hi));
-    }, next, tb);
+    }, tb);
 }
 
 // One (batch, head, 64-query block) per workgroup pass; each wave owns 16 queries.
@@ -633,48 +617,33 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       grid_sync(bar);
       stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
     } else {
-      // Weight slices are queued one stage ahead: right after a stage's MFMA loop has
-      // released the W region, the slice of the next stage is requested, so it crosses HBM
-      // while the epilogue stores drain and the grid barrier is crossed.
-      if (is_streamer(a.M)) {
-        // Weight traffic is moved into the stages that leave HBM idle; every slice is requested
-        // at least one full stage before it is multiplied.
-        grid_sync(bar, 16);                                           // QKV runs
-        warm_col_slices(lds_raw, w.w_o, H, H / 64, 0);
-        warm_col_slices(lds_raw, w.w_fc1, F, F / 64, 0);
-        grid_sync(bar, 16);                                           // attention runs
-        warm_fc2_slices(lds_raw, w.w_fc2);
-        grid_sync(bar, 16);                                           // out-projection runs
-        if (l + 1 < a.num_layers)
-          for (int j = 0; j < 3; ++j) warm_col_slices(lds_raw, args.layers[l + 1].w_qkv + (size_t)j * H * H, H, H / 64, j * (H / 64));
-        grid_sync(bar, 16);                                           // FC1 runs
-        grid_sync(bar, 16);                                           // FC2 runs
-        if (l + 1 < a.num_layers) grid_sync(bar, 16);                 // LayerNorm 2 runs
-        continue;
-      }
-      const bool attn_fits = 2 * a.S * 128 + 64 * 128 <= kXRegion;   // attention tiles stay below the W region
+      // Weight slices are queued one stage ahead, from inside the grid barrier that precedes
+      // the stage (during attention the out-projection slice waits in the W region, which the
+      // attention tiles do not reach when S <= 128).
+      const bool attn_fits = 2 * a.S * 128 + 64 * 128 <= kXRegion;
       const OutItems out_items{w.w_o, a.M};
       const Fc1Items fc1_items{w.w_fc1, a.M};
       const Fc2Items fc2_items{w.w_fc2, a.M};
-      bool out_ready = false;
-      small_qkv<true>(lds_raw, a, w, xin, qkv_ready, [&]() { if (attn_fits) out_ready = preissue_w<OsFull>(lds_raw, out_items); }, &bar);
-      grid_sync(bar, out_ready ? OsFull::PREFETCH_INSTR : 0);
+      bool out_ready = false, fc1_ready = false, fc2_ready = false;
+      small_qkv<true>(lds_raw, a, w, xin, qkv_ready, &bar);
+      // (a workgroup that has an attention item would wait for the slice inside attention: it asks later)
+      const bool attn_busy = first < a.B * NH * (a.S / 64);
+      grid_sync(bar, [&]() { if (attn_fits && !attn_busy) out_ready = preissue_w<OsFull>(lds_raw, out_items); });
       stage_attn_t<true, NKT>(lds, a, first, stride);
-      if (!attn_fits) { __syncthreads(); out_ready = preissue_w<OsFull>(lds_raw, out_items); }
-      grid_sync(bar, attn_fits ? 0 : (out_ready ? OsFull::PREFETCH_INSTR : 0));
-      bool fc1_ready = false, fc2_ready = false;
-      small_outproj<true>(lds_raw, a, w, xin, out_ready, [&]() { fc1_ready = preissue_w<OsFull>(lds_raw, fc1_items); }, &bar);
-      grid_sync(bar, fc1_ready ? OsFull::PREFETCH_INSTR : 0);
-      small_fc1<true>(lds_raw, a, w, fc1_ready, [&]() { fc2_ready = preissue_w<OsFc2>(lds_raw, fc2_items); }, &bar);
-      grid_sync(bar, fc2_ready ? OsFc2::PREFETCH_INSTR : 0);
-      qkv_ready = false;
-      small_fc2<true>(lds_raw, a, w, fc2_ready, [&]() {
-        if (l + 1 < a.num_layers) qkv_ready = preissue_w<OsFull>(lds_raw, QkvItems{args.layers[l + 1].w_qkv, a.M});
-      }, &bar);
-      grid_sync(bar, qkv_ready ? OsFull::PREFETCH_INSTR : 0);
+      grid_sync(bar, [&]() { if (!out_ready) out_ready = preissue_w<OsFull>(lds_raw, out_items); });
+      small_outproj<true>(lds_raw, a, w, xin, out_ready, &bar);
+      grid_sync(bar, [&]() { fc1_ready = preissue_w<OsFull>(lds_raw, fc1_items); });
+      small_fc1<true>(lds_raw, a, w, fc1_ready, &bar);
+      grid_sync(bar, [&]() { fc2_ready = preissue_w<OsFc2>(lds_raw, fc2_items); });
+      small_fc2<true>(lds_raw, a, w, fc2_ready, &bar);
+      grid_sync(bar);
       stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
     }
-    if (l + 1 < a.num_layers) grid_sync(bar);   // (a prefetched QKV slice is older than the LN2 stores: wait for everything)
+    qkv_ready = false;
+    if (l + 1 < a.num_layers) {
+      if constexpr (LARGE) grid_sync(bar);
+      else grid_sync(bar, [&]() { qkv_ready = preissue_w<OsFull>(lds_raw, QkvItems{args.layers[l + 1].w_qkv, a.M}); });
+    }
     xin = yout;
   }
   grid_barrier_end(bar);
@@ -686,7 +655,7 @@ __global__ void __launch_bounds__(256) k_qkv(Args a, int l, const half_t *xin) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
   if constexpr (LARGE) stage_qkv<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], xin, blockIdx.x, gridDim.x);
-  else small_qkv<false>(lds_raw, a, a.layers[l], xin, false, []() {});
+  else small_qkv<false>(lds_raw, a, a.layers[l], xin, false);
 }
 __global__ void __launch_bounds__(256) k_attn(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -700,7 +669,7 @@ __global__ void __launch_bounds__(256) k_partial(Args a, const half_t *X, int K,
   else {
     LayerW w{};
     w.w_fc2 = W;
-    small_fc2<false>(lds_raw, a, w, false, []() {});
+    small_fc2<false>(lds_raw, a, w, false);
   }
 }
 __global__ void __launch_bounds__(256) k_ln(Args a, int splitk, const half_t *bias, const half_t *resid,
@@ -712,11 +681,11 @@ __global__ void __launch_bounds__(256) k_fc1(Args a, int l) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
   if constexpr (LARGE) stage_fc1<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], blockIdx.x, gridDim.x);
-  else small_fc1<false>(lds_raw, a, a.layers[l], false, []() {});
+  else small_fc1<false>(lds_raw, a, a.layers[l], false);
 }
 __global__ void __launch_bounds__(256) k_outproj_small(Args a, int l, const half_t *xin) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  small_outproj<false>(lds_raw, a, a.layers[l], xin, false, []() {});
+  small_outproj<false>(lds_raw, a, a.layers[l], xin, false);
 }
 
 // ------------------------------------------------------------------- host ----

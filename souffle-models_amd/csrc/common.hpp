@@ -191,29 +191,29 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-// `pending`: number of vector loads (0, 16 or 32) that every wave except wave 0 queued AFTER
-// its last store of the stage and that may stay in flight across the barrier (prefetch of the
-// next stage's weight slice into LDS); everything older, i.e. every store, must be
-// acknowledged.  Wave 0 polls the barrier and therefore never has such loads.
-__device__ __forceinline__ void grid_sync(GridBarrier &b, int pending = 0) {
+// `mid()` is called by every wave after the workgroup has arrived and before it starts to wait:
+// the place to queue loads that do not depend on other workgroups (the next stage's weight
+// slice), so that they travel while the barrier completes.  Wave 0 polls; its polling loads
+// return in issue order, so it must not queue anything slow in mid() itself.
+template <class Mid>
+__device__ __forceinline__ void grid_sync(GridBarrier &b, Mid mid) {
   const bool tr = b.trace && b.trace_idx < b.trace_cap && threadIdx.x == 0;
   if (tr) b.trace[(size_t)(2 * b.trace_idx) * b.nblk + blockIdx.x] = wall_clock64();
-  if (threadIdx.x < 64 || pending == 0) __builtin_amdgcn_s_waitcnt(0);   // write-through stores are acknowledged
-  else if (pending == 32) wait_vmcnt<32>();
-  else if (pending == 16) wait_vmcnt<16>();
-  else __builtin_amdgcn_s_waitcnt(0);
+  __builtin_amdgcn_s_waitcnt(0);           // write-through stores are acknowledged
   __builtin_amdgcn_s_barrier();
 #ifdef SOUFFLE_STAGE_MARKS
   trace_mark(b, 7);
 #endif
   b.target += b.gsz;
   b.epoch += 1;
+  if (threadIdx.x == 0) {
+    const unsigned x = blockIdx.x & 7;
+    const unsigned old = __hip_atomic_fetch_add(b.ctl + 32 * x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old + 1 == b.target) __hip_atomic_store(b.ctl + 256 + 32 * x, b.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __builtin_amdgcn_s_barrier();            // the arrival (and the done flag) precede whatever mid() queues
+  mid();
   if (threadIdx.x < 64) {
-    if (threadIdx.x == 0) {
-      const unsigned x = blockIdx.x & 7;
-      const unsigned old = __hip_atomic_fetch_add(b.ctl + 32 * x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (old + 1 == b.target) __hip_atomic_store(b.ctl + 256 + 32 * x, b.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
     for (int spin = 0; spin < kMaxBarrierSpin; ++spin) {
       bool ok = true;
       if (threadIdx.x < 8 && threadIdx.x < b.nblk)
@@ -225,9 +225,10 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b, int pending = 0) {
   b.count++;
   if (tr) b.trace[(size_t)(2 * b.trace_idx + 1) * b.nblk + blockIdx.x] = wall_clock64();
   b.trace_idx++;
-  __builtin_amdgcn_s_barrier();          // no memory wait here: prefetch loads may still be in flight
+  __builtin_amdgcn_s_barrier();            // no memory wait here: loads queued by mid() may still be in flight
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
+__device__ __forceinline__ void grid_sync(GridBarrier &b) { grid_sync(b, []() {}); }
 
 // Call once by every workgroup before the kernel returns.
 __device__ __forceinline__ void grid_barrier_end(GridBarrier &b) {

@@ -4,7 +4,7 @@
 // Both operand slices fit in LDS, so ALL of their loads are queued at once with the direct
 // global->LDS instruction (no register staging, ~100 KB in flight per CU): an item costs
 // one memory latency instead of one per K step, and the weight slice of the NEXT stage can
-// be queued before a grid barrier and land while the barrier is crossed.
+// be queued inside a grid barrier and land while the barrier completes.
 //
 // LDS layouts are unpadded (the direct load writes 64 consecutive 16-byte slots per wave
 // instruction) and XOR-swizzled at slot granularity instead:
@@ -67,11 +67,13 @@ struct GemmOneShot {
   // barrier, and its polling loads must not queue up behind a weight slice that is still in flight.
   static constexpr int PREFETCH_INSTR = W_INSTR / 3;
   static_assert(W_INSTR % 3 == 0 && PREFETCH_INSTR < 64, "prefetch split over three waves");
-  __device__ static __forceinline__ void issue_w_prefetch(unsigned char *lds_w, const half_t *__restrict__ W, int ldw, int n0, int k0) {
+  __device__ static __forceinline__ void issue_w_prefetch(unsigned char *lds_w, const half_t *__restrict__ W, int ldw, int n0, int k0, int rot = 0) {
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6;
     if (wave == 0) return;
 #pragma unroll
-    for (int q = 0; q < PREFETCH_INSTR; ++q) {
+    for (int q0 = 0; q0 < PREFETCH_INSTR; ++q0) {
+      int q = q0 + (rot * 4) / 3;
+      if (q >= PREFETCH_INSTR) q -= PREFETCH_INSTR;
       const int inst = q * 3 + wave - 1, s = inst * 64 + lane, k = s >> 3, c = (s & 7) ^ (k & 2);
       __builtin_amdgcn_global_load_lds((gptr_t)(W + (size_t)(k0 + k) * ldw + n0 + c * 8), (lptr_t)(lds_w + inst * 1024), 16, 0, 0);
     }
