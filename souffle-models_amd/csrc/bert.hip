@@ -179,7 +179,7 @@ __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, 
 
 // ---- skinny (small M) path: one-shot operand loads, see gemm_oneshot.hpp ----
 using OsFull = GemmOneShot<32, 768>;    // QKV, out-projection, FC1: whole K in one shot
-using OsFc2 = GemmOneShot<64, 384>;     // FC2: 8 K slices as fp32 partials
+using OsFc2 = GemmOneShot<32, 768>;     // FC2: 4 K slices as fp32 partials
 constexpr int kSplitFc2Small = F / OsFc2::kKS;
 constexpr int kXRegion = 49152;         // LDS: [0, 48 KB) X slice / attention tiles / reduction, [48 KB, 144 KB) W slice
 static_assert(OsFull::X_BYTES <= kXRegion && OsFc2::X_BYTES <= kXRegion, "X region");
@@ -557,6 +557,158 @@ __device__ __forceinline__ void attn_item(half_t *lds_h, const Params &a, int it
     st8<COH>(a.ctx, ((b * S + q) * H + hh * HD + dt * 16 + g * 4) * 2, pack_h4(o[dt]));
 }
 
+// ---- attention for the skinny path: one item = one head x 16 queries, keys split over the waves ----
+// With few rows the 64-query item above leaves most CUs idle and its per-wave chain
+// (scores -> softmax -> P.V over ALL keys) is the stage's critical path.  Here each wave
+// handles a quarter of the keys for the same 16 queries and loads exactly the K/V rows it
+// multiplies (no workgroup barrier before the MFMAs); the four partial results are merged
+// through LDS the flash-attention way (running maximum, rescaled sums).
+constexpr int kAttnCombLd = 68;                                   // floats per row of a wave's partial context
+constexpr int attn_small_lds_bytes(int S) { return 2 * S * 128 + 4 * 2048 + 4 * 16 * kAttnCombLd * 4 + 512; }
+
+template <int MODE>
+__device__ __forceinline__ void issue_rows64_wave(unsigned char *lds_tile, const half_t *src, int row0, int rows) {
+  typedef __attribute__((address_space(1))) const void *gptr_t;
+  typedef __attribute__((address_space(3))) void *lptr_t;
+  const int lane = threadIdx.x & 63;
+  for (int inst = 0; inst < rows / 8; ++inst) {
+    const int r = row0 + inst * 8 + (lane >> 3), c = (lane & 7) ^ (MODE == 0 ? ((r >> 1) & 7) : (r & 2));
+    __builtin_amdgcn_global_load_lds((gptr_t)(src + (size_t)r * HD + c * 8), (lptr_t)(lds_tile + (row0 + inst * 8) * 128), 16, 0, 0);
+  }
+}
+
+template <bool COH, int NKT>
+__device__ __forceinline__ void attn_item_split(unsigned char *lds, const Params &a, int bh, int qb) {
+  constexpr int S = NKT * 16, TPW = NKT / 4;                       // key tiles per wave
+  static_assert(NKT % 4 == 0, "keys split evenly over four waves");
+  unsigned char *ks_ = lds, *vs_ = lds + S * 128, *qs_ = lds + 2 * S * 128;
+  float *comb = reinterpret_cast<float *>(lds + 2 * S * 128 + 4 * 2048);
+  float *stats = comb + 4 * 16 * kAttnCombLd;                      // [wave][query][max, sum]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+  const int b = bh / NH, hh = bh % NH;
+  const int head_off = ((b * NH + hh) * S) * HD;                   // halves, within one of q/k/v
+  const size_t plane = (size_t)a.B * NH * S * HD;
+  const half_t *Q = a.qkv + head_off + (size_t)qb * 16 * HD, *K = a.qkv + plane + head_off, *V = a.qkv + 2 * plane + head_off;
+
+  __syncthreads();   // LDS reuse
+  issue_rows64_wave<0>(qs_ + wave * 2048, Q, 0, 16);               // every wave its own copy of the queries
+  issue_rows64_wave<0>(ks_, K, wave * TPW * 16, TPW * 16);
+  issue_rows64_wave<1>(vs_, V, wave * TPW * 16, TPW * 16);
+  __builtin_amdgcn_s_waitcnt(0);                                   // this wave's rows only: no barrier needed
+
+  const half_t *kh = reinterpret_cast<const half_t *>(ks_), *vh = reinterpret_cast<const half_t *>(vs_),
+               *qh = reinterpret_cast<const half_t *>(qs_ + wave * 2048);
+  const int q = qb * 16 + l16;
+  h8 qop[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) qop[ks] = *reinterpret_cast<const h8 *>(qh + (l16 * 8 + ((ks * 4 + g) ^ ((l16 >> 1) & 7))) * 8);
+  f4 sc[TPW];
+  float mx = -1e30f;                                               // finite: a fully masked quarter contributes nothing
+#pragma unroll
+  for (int tt = 0; tt < TPW; ++tt) {
+    const int t = wave * TPW + tt, r = t * 16 + l16, sw = (r >> 1) & 7;
+    const h8 k0 = *reinterpret_cast<const h8 *>(kh + (r * 8 + (g ^ sw)) * 8);
+    const h8 k1 = *reinterpret_cast<const h8 *>(kh + (r * 8 + ((4 + g) ^ sw)) * 8);
+    f4 sv = mfma_16x16x32(k1, qop[1], mfma_16x16x32(k0, qop[0], f4{0.f, 0.f, 0.f, 0.f})) * a.scale;
+    // sv[v] = score(key = 16t + 4g + v, query = q)
+    if (a.mask) {
+      const h4 mk = *reinterpret_cast<const h4 *>(a.mask + ((size_t)b * S + q) * S + t * 16 + g * 4);
+      sv += f4{(float)mk[0], (float)mk[1], (float)mk[2], (float)mk[3]};
+    }
+    sc[tt] = sv;
+    mx = fmaxf(mx, fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
+  }
+  mx = fmaxf(mx, wave_xor(mx, 16));
+  mx = fmaxf(mx, wave_xor(mx, 32));
+  float sum = 0.f;
+  h4 p[TPW];
+#pragma unroll
+  for (int tt = 0; tt < TPW; ++tt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { sc[tt][i] = __expf(sc[tt][i] - mx); sum += sc[tt][i]; }
+    p[tt] = h4{(half_t)sc[tt][0], (half_t)sc[tt][1], (half_t)sc[tt][2], (half_t)sc[tt][3]};
+  }
+  sum += wave_xor(sum, 16);
+  sum += wave_xor(sum, 32);
+  f4 o[HD / 16];
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt) o[dt] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int tt = 0; tt < TPW; ++tt) {
+    const int kr = (wave * TPW + tt) * 16 + g * 4 + (l16 >> 2);
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) {
+      const int c = dt * 2 + ((l16 & 3) >> 1);
+      const h4 vop = lds_read_tr16(vh + (kr * 8 + (c ^ (kr & 2))) * 8 + (l16 & 1) * 4);
+      o[dt] = mfma_16x16x16(vop, p[tt], o[dt]);
+    }
+  }
+  // o[dt][v] = sum over this wave's keys of exp(score - mx) * V[key][16dt + 4g + v], query q
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt)
+    *reinterpret_cast<f4 *>(comb + (wave * 16 + l16) * kAttnCombLd + dt * 16 + g * 4) = o[dt];
+  if (g == 0) { stats[(wave * 16 + l16) * 2] = mx; stats[(wave * 16 + l16) * 2 + 1] = sum; }
+  __syncthreads();
+  float wmx[4], wsum[4];
+  auto merged = [&](int qq, float *scale) {                        // scale[w] = exp(mx_w - max) / total
+    float m = -1e30f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) { wmx[w] = stats[(w * 16 + qq) * 2]; wsum[w] = stats[(w * 16 + qq) * 2 + 1]; m = fmaxf(m, wmx[w]); }
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) { scale[w] = __expf(wmx[w] - m); total += wsum[w] * scale[w]; }
+    const float inv = 1.0f / total;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) scale[w] *= inv;
+  };
+  {
+    const int qq = tid >> 4, d0 = (tid & 15) * 4;
+    float scale[4];
+    merged(qq, scale);
+    f4 r = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) r += *reinterpret_cast<const f4 *>(comb + (w * 16 + qq) * kAttnCombLd + d0) * scale[w];
+    st8<COH>(a.ctx, ((b * S + qb * 16 + qq) * H + hh * HD + d0) * 2, pack_h4(r));
+  }
+  if (a.probs) {
+    float scale[4];
+    merged(l16, scale);
+#pragma unroll
+    for (int tt = 0; tt < TPW; ++tt) {
+      const f4 pr = sc[tt] * scale[wave];
+      const h4 ph = {(half_t)pr[0], (half_t)pr[1], (half_t)pr[2], (half_t)pr[3]};
+      st8<false>(a.probs, (int)((((size_t)(b * NH + hh) * S + q) * S + (wave * TPW + tt) * 16 + g * 4) * 2), as_u2(ph));
+    }
+  }
+}
+
+// Items are dealt so that the 16-query blocks of one head run on one XCD (they share K and V),
+// and, when the grid is large enough, on workgroups 64.. so that the workgroups of the
+// out-projection can fetch their weight slice meanwhile.
+__device__ __forceinline__ void attn_small_range(const Params &a, int stride, int *off, int *span) {
+  *span = xcd_item_span(a.S / 16, a.B * NH);
+  *off = (*span + 64 <= stride) ? 64 : 0;
+}
+template <bool COH, int NKT>
+__device__ __forceinline__ void stage_attn_small_t(unsigned char *lds, const Params &a, int first, int stride) {
+  int off, span;
+  attn_small_range(a, stride, &off, &span);
+  for (int it = first - off; it < span; it += stride) {
+    int qb, bh;
+    if (it >= 0 && xcd_item(it, a.S / 16, a.B * NH, &qb, &bh)) attn_item_split<COH, NKT>(lds, a, bh, qb);
+  }
+}
+template <bool COH>
+__device__ __forceinline__ void stage_attn_small(unsigned char *lds, const Params &a, int first, int stride) {
+  switch (a.S) {
+    case 64: stage_attn_small_t<COH, 4>(lds, a, first, stride); break;
+    case 128: stage_attn_small_t<COH, 8>(lds, a, first, stride); break;
+    case 256: stage_attn_small_t<COH, 16>(lds, a, first, stride); break;
+    case 384: stage_attn_small_t<COH, 24>(lds, a, first, stride); break;
+    default: stage_attn_small_t<COH, 32>(lds, a, first, stride); break;   // 512 (validated on the host)
+  }
+}
+
 template <bool COH, int NKT>
 __device__ __forceinline__ void stage_attn_t(half_t *lds, const Params &a, int first, int stride) {
   const int items = a.B * NH * (a.S / 64);
@@ -578,7 +730,7 @@ __device__ __forceinline__ void stage_attn(half_t *lds, const Params &a, int fir
 
 using TileSmall = GemmTile<64, 64, 64, 2, 2>;
 using TileLarge = GemmTile<128, 128, 64, 2, 2>;
-constexpr int kAttnLdsBytes = 2 * 512 * 128 + 64 * 128;
+constexpr int kAttnLdsBytes = attn_small_lds_bytes(512) > 2 * 512 * 128 + 64 * 128 ? attn_small_lds_bytes(512) : 2 * 512 * 128 + 64 * 128;
 constexpr int lds_bytes(bool large) {
   const int t = large ? TileLarge::LDS_BYTES : kSmallGemmLds;
   return t > kAttnLdsBytes ? t : kAttnLdsBytes;
@@ -618,18 +770,18 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
     } else {
       // Weight slices are queued one stage ahead, from inside the grid barrier that precedes
-      // the stage (during attention the out-projection slice waits in the W region, which the
-      // attention tiles do not reach when S <= 128).
-      const bool attn_fits = 2 * a.S * 128 + 64 * 128 <= kXRegion;
+      // the stage.
       const OutItems out_items{w.w_o, a.M};
       const Fc1Items fc1_items{w.w_fc1, a.M};
       const Fc2Items fc2_items{w.w_fc2, a.M};
       bool out_ready = false, fc1_ready = false, fc2_ready = false;
       small_qkv<true>(lds_raw, a, w, xin, qkv_ready, &bar);
       // (a workgroup that has an attention item would wait for the slice inside attention: it asks later)
-      const bool attn_busy = first < a.B * NH * (a.S / 64);
-      grid_sync(bar, [&]() { if (attn_fits && !attn_busy) out_ready = preissue_w<OsFull>(lds_raw, out_items); });
-      stage_attn_t<true, NKT>(lds, a, first, stride);
+      int attn_off, attn_span;
+      attn_small_range(a, stride, &attn_off, &attn_span);
+      const bool attn_busy = first >= attn_off && first < attn_off + attn_span;
+      grid_sync(bar, [&]() { if (!attn_busy) out_ready = preissue_w<OsFull>(lds_raw, out_items); });
+      stage_attn_small_t<true, NKT>(lds_raw, a, first, stride);
       grid_sync(bar, [&]() { if (!out_ready) out_ready = preissue_w<OsFull>(lds_raw, out_items); });
       small_outproj<true>(lds_raw, a, w, xin, out_ready, &bar);
       grid_sync(bar, [&]() { fc1_ready = preissue_w<OsFull>(lds_raw, fc1_items); });
@@ -637,7 +789,7 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       grid_sync(bar, [&]() { fc2_ready = preissue_w<OsFc2>(lds_raw, fc2_items); });
       small_fc2<true>(lds_raw, a, w, fc2_ready, &bar);
       grid_sync(bar);
-      stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
+      stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, wave * stride + first, stride * 4);
     }
     qkv_ready = false;
     if (l + 1 < a.num_layers) {
@@ -660,6 +812,10 @@ __global__ void __launch_bounds__(256) k_qkv(Args a, int l, const half_t *xin) {
 __global__ void __launch_bounds__(256) k_attn(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   stage_attn<false>(reinterpret_cast<half_t *>(lds_raw), a, blockIdx.x, gridDim.x);
+}
+__global__ void __launch_bounds__(256) k_attn_small(Args a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  stage_attn_small<false>(lds_raw, a, blockIdx.x, gridDim.x);
 }
 template <bool LARGE>
 __global__ void __launch_bounds__(256) k_partial(Args a, const half_t *X, int K, const half_t *W, int splitk) {
@@ -831,6 +987,7 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_partial<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_fc1<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_attn, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLdsBytes));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_attn_small, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLdsBytes));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_outproj_small, hipFuncAttributeMaxDynamicSharedMemorySize, kSmallGemmLds));
     attr_done = true;
   }
@@ -841,7 +998,8 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     const LayerW &w = a.layers[l];
     half_t *yout = (l == nl - 1) ? a.y : a.yl;
     hipLaunchKernelGGL(k_qkv<LARGE>, dim3(grid_for((a.M / BM_QKV) * (3 * H / BN))), dim3(256), GEMM_LDS, st, a, l, xin);
-    hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), 2 * a.S * 128 + 64 * 128, st, a);
+    if (LARGE) hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), 2 * a.S * 128 + 64 * 128, st, a);
+    else hipLaunchKernelGGL(k_attn_small, dim3(grid_for((a.B * NH + 7) / 8 * 8 * (a.S / 16))), dim3(256), attn_small_lds_bytes(a.S), st, a);
     if (LARGE) {
       hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, 1);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, 1, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
