@@ -150,7 +150,7 @@ def bench_encoder(args, B, S, L, name):
         "extra": {"per_layer_us_cold": cold_ev * 1e3 / L, "warm_cache_us": warm_ev * 1e3, "per_layer_us_warm": warm_ev * 1e3 / L,
                   "unfused_per_op_us": unf_ev * 1e3, "fused_speedup_vs_unfused": unf_ev / cold_ev,
                   "min_of_means_us_warm": mn, "median_us_warm": med, "parity": parity,
-                  "launches_fused": 1, "launches_unfused": 7 * L},
+                  "launches_fused": 1, "launches_unfused": (6 if M < 1024 else 7) * L},
     }
     if cpu:
         res["cpu_baseline"] = cpu
@@ -176,6 +176,16 @@ def main():
     elif args.workload == "encoder_b32":
         args.weight_sets = 1
         res = bench_encoder(args, 32, 128, 12, "BERT-base 12-layer encoder, B=32, S=128, fp16 (MFMA-bound shape)")
+    elif args.workload == "copy":
+        # A plain device copy of known size: the calibration run for the FETCH_SIZE / WRITE_SIZE
+        # counters (counter reading per byte actually read / written).
+        n = 256 << 20
+        a = torch.empty(n, dtype=torch.uint8, device="cuda:0").fill_(1)
+        b = torch.empty_like(a)
+        for _ in range(max(1, args.steps // 20)):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        res = {"workload": "copy", "bytes_read_per_copy": n, "bytes_written_per_copy": n, "copies": max(1, args.steps // 20)}
     else:
         import bench_extra
         res = bench_extra.run(args)

@@ -65,6 +65,17 @@ int souffle_workspace_init(void *workspace, size_t workspace_bytes, souffle_stre
  * buf[(2*cap + 8*i + id) * grid + block].  Pass NULL to switch tracing off (the default). */
 int souffle_set_stage_trace(void *device_buf, size_t bytes);
 
+/* How the persistent (grid-barrier) kernels are launched.  The reference launches its fused
+ * kernels with cudaLaunchCooperativeKernel (cpp/swin_transformer/swin_transformer_binding.cu:95,
+ * cpp/efficientnet/efficientnet_se_module_main.cu:62).  On MI355X a cooperative launch costs
+ * ~20 us against ~4 us for a plain one, which is most of a 30 us encoder layer, so the default
+ * (on = 0) is a plain launch of a grid that the occupancy query has shown to be co-resident on
+ * an otherwise idle device.  Fused calls must then not overlap in time with other fused calls
+ * on another stream (two half-resident grids would wait for each other until the bounded
+ * barrier spin gives up and the call's output is invalid).  on = 1 restores the runtime's
+ * guarantee.  The environment variable SOUFFLE_COOPERATIVE_LAUNCH=1 sets the initial value. */
+int souffle_set_cooperative_launch(int on);
+
 /* ------------------------------------------------------------------ BERT ---- */
 enum { SOUFFLE_ACT_GELU_TANH = 0, SOUFFLE_ACT_RELU = 1 };
 

@@ -2,7 +2,10 @@
 // workspace initialisation, the event-timing helper and the plain GEMM.
 #include <algorithm>
 #include <cstring>
+#include <atomic>
+#include <map>
 #include <mutex>
+#include <cstdlib>
 #include <type_traits>
 #include <vector>
 #include "gemm_tile.hpp"
@@ -47,6 +50,43 @@ int device_facts(DeviceFacts *out) {
 
 static void *g_trace_buf = nullptr;
 static size_t g_trace_bytes = 0;
+static std::atomic<int> g_cooperative{-1};
+static bool cooperative_mode() {
+  int v = g_cooperative.load();
+  if (v < 0) {
+    const char *e = getenv("SOUFFLE_COOPERATIVE_LAUNCH");
+    v = (e && e[0] == '1') ? 1 : 0;
+    g_cooperative.store(v);
+  }
+  return v == 1;
+}
+
+int launch_persistent(const void *fn, int grid, int block, void **args, size_t lds_bytes, hipStream_t st) {
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  {
+    static std::mutex mu;
+    static std::map<std::pair<const void *, size_t>, int> per_cu;     // (function, LDS bytes) -> workgroups per CU
+    std::lock_guard<std::mutex> lk(mu);
+    auto key = std::make_pair(fn, lds_bytes);
+    auto it = per_cu.find(key);
+    if (it == per_cu.end()) {
+      int n = 0;
+      SOUFFLE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, block, lds_bytes));
+      it = per_cu.emplace(key, n).first;
+    }
+    if ((long long)it->second * df.num_cus < grid)
+      return fail(SOUFFLE_ERR_DEVICE, "a grid of %d workgroups cannot be resident at once (%d per CU on %d CUs)", grid, it->second, df.num_cus);
+  }
+  if (cooperative_mode()) {
+    if (!df.cooperative) return fail(SOUFFLE_ERR_DEVICE, "device does not support cooperative launches");
+    SOUFFLE_HIP_TRY(hipLaunchCooperativeKernel(fn, dim3(grid), dim3(block), args, lds_bytes, st));
+  } else {
+    SOUFFLE_HIP_TRY(hipLaunchKernel(fn, dim3(grid), dim3(block), args, lds_bytes, st));
+  }
+  return SOUFFLE_OK;
+}
+
 void stage_trace(unsigned long long **buf, int *max_barriers, int nblk) {
   *buf = static_cast<unsigned long long *>(g_trace_buf);
   *max_barriers = g_trace_buf ? (int)(g_trace_bytes / ((size_t)nblk * 80)) : 0;   // 2 stamps + 8 marks per barrier
@@ -106,6 +146,11 @@ extern "C" int souffle_device_info(souffle_devinfo *out) {
   out->cooperative_launch = p.cooperativeLaunch;
   out->wavefront_size = p.warpSize;
   strncpy(out->arch, p.gcnArchName, sizeof(out->arch) - 1);
+  return SOUFFLE_OK;
+}
+
+extern "C" int souffle_set_cooperative_launch(int on) {
+  souffle::g_cooperative.store(on ? 1 : 0);
   return SOUFFLE_OK;
 }
 

@@ -946,8 +946,7 @@ static int launch_mega_t(Args &a, int grid, hipStream_t st) {
     attr_done = true;
   }
   void *args[] = {&a};
-  SOUFFLE_HIP_TRY(hipLaunchCooperativeKernel((const void *)k_encoder_mega<LARGE, NKT>, dim3(grid), dim3(256), args, lds, st));
-  return SOUFFLE_OK;
+  return launch_persistent((const void *)k_encoder_mega<LARGE, NKT>, grid, 256, args, lds, st);
 }
 // one kernel per supported sequence length, so that each carries only its own attention tile
 template <bool LARGE>

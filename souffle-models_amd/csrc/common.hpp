@@ -220,6 +220,8 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b, Mid mid) {
         ok = (int)(__hip_atomic_load(b.ctl + 256 + 32 * threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - b.epoch) >= 0;
       if (__all(ok)) break;
       __builtin_amdgcn_s_sleep(1);
+      if (spin == kMaxBarrierSpin - 1 && threadIdx.x == 0)   // gave up: the launch's output is invalid
+        (void)__hip_atomic_fetch_or(b.ctl + kCtlErrWord, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
   b.count++;

@@ -26,6 +26,12 @@ int device_facts(DeviceFacts *out);
 // Process-wide stage-trace buffer set by souffle_set_stage_trace (NULL = tracing off).
 void stage_trace(unsigned long long **buf, int *max_barriers, int nblk);
 
+// Launch of a persistent kernel whose workgroups synchronise through the grid barrier: all
+// `grid` workgroups must be resident at once.  Checks that with the occupancy query (cached
+// per function), then launches plainly or, when souffle_set_cooperative_launch(1) was called,
+// cooperatively.
+int launch_persistent(const void *fn, int grid, int block, void **args, size_t lds_bytes, hipStream_t st);
+
 inline size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 #define SOUFFLE_HIP_TRY(expr)                                                            \

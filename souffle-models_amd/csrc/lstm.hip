@@ -172,7 +172,5 @@ extern "C" int souffle_lstm_fused(const souffle_lstm_cfg *cfg, const void *w_ih,
   a.ctl = static_cast<unsigned *>(ws);
   a.hbuf = reinterpret_cast<u2 *>(static_cast<char *>(ws) + round_up(kCtlWords * 4, 256));
   void *args[] = {&a};
-  SOUFFLE_HIP_TRY(hipLaunchCooperativeKernel((const void *)lstm::k_lstm, dim3(grid), dim3(256), args, 0,
-                                             static_cast<hipStream_t>(stream)));
-  return SOUFFLE_OK;
+  return launch_persistent((const void *)lstm::k_lstm, grid, 256, args, 0, static_cast<hipStream_t>(stream));
 }

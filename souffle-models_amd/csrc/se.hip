@@ -139,7 +139,5 @@ extern "C" int souffle_se_module_fused(const float *x, const float *w_reduce, co
   se::Args a{C, HW, R, chunks, combine, x, w_reduce, b_reduce, w_expand, b_expand, y, pooled,
              reinterpret_cast<float *>(static_cast<char *>(ws) + round_up(kCtlWords * 4, 256)), static_cast<unsigned *>(ws)};
   void *args[] = {&a};
-  SOUFFLE_HIP_TRY(hipLaunchCooperativeKernel((const void *)se::k_se, dim3(df.num_cus), dim3(256), args, 0,
-                                             static_cast<hipStream_t>(stream)));
-  return SOUFFLE_OK;
+  return launch_persistent((const void *)se::k_se, df.num_cus, 256, args, 0, static_cast<hipStream_t>(stream));
 }

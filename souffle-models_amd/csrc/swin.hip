@@ -334,9 +334,8 @@ extern "C" int souffle_swin_block_pair_fused(const souffle_swin_cfg *cfg, const 
   }
   const int nwin = (cfg->height / swin::WS) * (cfg->width / swin::WS);
   void *args[] = {&a};
-  SOUFFLE_HIP_TRY(hipLaunchCooperativeKernel((const void *)swin::k_block_pair, dim3(std::min(nwin, df.num_cus)), dim3(256), args,
-                                             swin::LDS_BYTES, static_cast<hipStream_t>(stream)));
-  return SOUFFLE_OK;
+  return launch_persistent((const void *)swin::k_block_pair, std::min(nwin, df.num_cus), 256, args, swin::LDS_BYTES,
+                           static_cast<hipStream_t>(stream));
 }
 
 // Closed forms of torch.roll(-shift) + view/permute window partition, its inverse, the
@@ -384,7 +383,5 @@ extern "C" int souffle_swin_ffn_fused(const void *x, const void *w1, const void 
     attr_done = true;
   }
   void *args[] = {&a};
-  SOUFFLE_HIP_TRY(hipLaunchCooperativeKernel((const void *)swin::k_ffn, dim3(df.num_cus), dim3(256), args, swin::Tile::LDS_BYTES,
-                                             static_cast<hipStream_t>(stream)));
-  return SOUFFLE_OK;
+  return launch_persistent((const void *)swin::k_ffn, df.num_cus, 256, args, swin::Tile::LDS_BYTES, static_cast<hipStream_t>(stream));
 }

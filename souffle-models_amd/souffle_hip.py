@@ -67,6 +67,7 @@ SIGNATURES = {
     "souffle_version": (C.c_char_p, []),
     "souffle_device_info": (C.c_int, [C.POINTER(DevInfo)]),
     "souffle_set_stage_trace": (C.c_int, [C.c_void_p, C.c_size_t]),
+    "souffle_set_cooperative_launch": (C.c_int, [C.c_int]),
     "souffle_workspace_init": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "souffle_bert_workspace_bytes": (C.c_size_t, [C.POINTER(BertCfg)]),
     "souffle_bert_layer_fused": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
@@ -159,6 +160,11 @@ def set_stage_trace(tensor):
         check(lib().souffle_set_stage_trace(None, 0))
     else:
         check(lib().souffle_set_stage_trace(tensor.data_ptr(), tensor.numel() * tensor.element_size()))
+
+
+def set_cooperative_launch(on):
+    """Launch the persistent kernels cooperatively (True) or plainly (False, the default)."""
+    check(lib().souffle_set_cooperative_launch(1 if on else 0))
 
 
 def device_info():
