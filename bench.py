@@ -136,7 +136,11 @@ def bench_encoder(args, B, S, L, name):
         ach = bytes_alg / (cold_ev * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS,
                 "traffic": None}
-    roof["kernel"] = "k_encoder_mega (one cooperative launch = %d layers)" % L
+    if (B, S, L) == (1, 128, 12):
+        # L2<->fabric bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a device
+        # copy of known size (profiles/k_encoder_mega_bert_encoder_b1_s128_hbm_traffic.txt)
+        roof["traffic"] = 339.6e6
+    roof["kernel"] = "k_encoder_mega (one launch = %d layers)" % L
     roof["algorithmic_bytes_per_launch"] = bytes_alg
     roof["algorithmic_flops_per_launch"] = flops
     roof["avg_launch_us"] = cold_ev * 1e3
