@@ -50,6 +50,16 @@ int device_facts(DeviceFacts *out) {
 
 static void *g_trace_buf = nullptr;
 static size_t g_trace_bytes = 0;
+static std::atomic<int> g_bert_sync{-1};
+int bert_sync_mode() {
+  int v = g_bert_sync.load();
+  if (v < 0) {
+    const char *e = getenv("SOUFFLE_BERT_SYNC");
+    v = (e && (e[0] == 'd' || e[0] == 'D')) ? SOUFFLE_SYNC_DATAFLOW : SOUFFLE_SYNC_BARRIER;
+    g_bert_sync.store(v);
+  }
+  return v;
+}
 static std::atomic<int> g_cooperative{-1};
 static bool cooperative_mode() {
   int v = g_cooperative.load();
@@ -151,6 +161,25 @@ extern "C" int souffle_device_info(souffle_devinfo *out) {
 
 extern "C" int souffle_set_cooperative_launch(int on) {
   souffle::g_cooperative.store(on ? 1 : 0);
+  return SOUFFLE_OK;
+}
+
+extern "C" int souffle_set_bert_sync(int mode) {
+  if (mode != SOUFFLE_SYNC_DATAFLOW && mode != SOUFFLE_SYNC_BARRIER) return fail(SOUFFLE_ERR_SHAPE, "unknown synchronisation mode %d", mode);
+  souffle::g_bert_sync.store(mode);
+  return SOUFFLE_OK;
+}
+
+extern "C" int souffle_workspace_status(void *ws, souffle_stream_t stream, unsigned *flags, int clear) {
+  if (!ws || !flags) return fail(SOUFFLE_ERR_NULL, "workspace and flags must not be NULL");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  unsigned *word = static_cast<unsigned *>(ws) + kCtlErrWord;
+  SOUFFLE_HIP_TRY(hipMemcpyAsync(flags, word, sizeof(unsigned), hipMemcpyDeviceToHost, st));
+  SOUFFLE_HIP_TRY(hipStreamSynchronize(st));
+  if (clear && *flags) {
+    hipLaunchKernelGGL(k_zero_words, dim3(1), dim3(64), 0, st, word, 1);
+    SOUFFLE_HIP_TRY(hipGetLastError());
+  }
   return SOUFFLE_OK;
 }
 

@@ -44,6 +44,10 @@ struct Params {
   unsigned long long *trace;
   int trace_cap;
   size_t layer_stride;
+  // dataflow kernel: bytes of one layer's buffers from `qkv` up to (not including) `yl`, and the
+  // marker the control block holds while all buffers of this layout are in the unwritten state
+  size_t flow_bytes;
+  unsigned flow_marker;
 };
 struct Args : Params {
   LayerW layers[kMaxLayers];
@@ -56,6 +60,86 @@ __device__ __forceinline__ Params layer_params(const Params &a, int l) {
   p.qkv = adv(a.qkv); p.ctx = adv(a.ctx); p.z1 = adv(a.z1); p.y1 = adv(a.y1); p.h = adv(a.h); p.yl = adv(a.yl);
   p.part = reinterpret_cast<float *>(reinterpret_cast<char *>(a.part) + off);
   return p;
+}
+
+// ---- dataflow synchronisation (skinny path) ----
+// Instead of a grid barrier between stages, a consumer polls the data it needs.  Every
+// inter-stage buffer holds the pattern 0xffffffff in each 32-bit word (two fp16 NaNs that no
+// conversion from fp32 produces, or an fp32 NaN no arithmetic here produces) until its producer
+// has written it; producers write through (sc1), consumers load with sc1 straight from the
+// memory side and re-request whatever still shows the pattern.  One load round trip thus both
+// detects and fetches the data; there is no arrival counter, no flag and no wait for store
+// acknowledgements on the critical path.  Waits are bounded: after kMaxFlowSpin retries the
+// workgroup gives up, flags the control block and stops waiting for the rest of the launch.
+constexpr int kMaxFlowSpin = 1 << 15;
+struct Flow {
+  bool failed;
+  unsigned long long *trace;   // optional stamps, same layout as the barrier trace: (ready, done) per stage
+  int trace_cap, stage;
+};
+__device__ __forceinline__ void flow_stamp(Flow &fl, int which) {
+  if (fl.trace && fl.stage < fl.trace_cap && threadIdx.x == 0)
+    fl.trace[(size_t)(2 * fl.stage + which) * gridDim.x + blockIdx.x] = wall_clock64();
+}
+__device__ __forceinline__ bool has_unwritten(u4 v) {
+  return (v[0] == ~0u) | (v[1] == ~0u) | (v[2] == ~0u) | (v[3] == ~0u);
+}
+__device__ __forceinline__ bool has_unwritten(u2 v) { return (v[0] == ~0u) | (v[1] == ~0u); }
+
+// A wave fetches N direct-to-LDS loads (issue(i): load i, 64 lanes x 16 bytes; slot(i): where this
+// lane's 16 bytes of load i land).  Loads in PROBE are repeated until none of their lanes sees
+// the pattern; only then are the others requested, and repeated individually while incomplete.
+// The probe loads are chosen to touch the last rows of the producers the wave depends on, so
+// that waiting costs a few KB per round trip and not the whole operand (polling the whole
+// operand from every waiting workgroup saturates the fabric and delays the very stores it waits for).
+template <int N, unsigned long long PROBE, class Issue, class Slot>
+__device__ __forceinline__ void poll_direct_loads(Issue issue, Slot slot, Flow &fl) {
+  static_assert(N >= 1 && N <= 64, "one mask bit per load");
+  constexpr unsigned long long ALL = N == 64 ? ~0ull : ((1ull << N) - 1);
+  static_assert(PROBE != 0 && (PROBE & ~ALL) == 0, "probe loads are a non-empty subset");
+  unsigned long long pending = PROBE;
+  bool rest_issued = false;
+#pragma unroll
+  for (int i = 0; i < N; ++i)
+    if ((PROBE >> i) & 1) issue(i);
+  for (int spin = 0;; ++spin) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    unsigned long long still = 0;
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      if ((pending >> i) & 1) {
+        const u4 v = *reinterpret_cast<const u4 *>(slot(i));
+        if (__any(has_unwritten(v))) still |= 1ull << i;
+      }
+    if (fl.failed || spin >= kMaxFlowSpin) { fl.failed = true; still = 0; }
+    if (!still) {
+      if (rest_issued || PROBE == ALL) return;
+      rest_issued = true;
+      still = ALL & ~PROBE;
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      if ((still >> i) & 1) issue(i);
+    pending = still;
+  }
+}
+
+// The X slice of a one-shot GEMM item, polled (layout as GemmOneShot::issue_x).
+template <class G>
+__device__ __forceinline__ void poll_x(unsigned char *lds_x, const half_t *X, int ldx, int m0, int k0, Flow &fl) {
+  typedef __attribute__((address_space(1))) const void *gptr_t;
+  typedef __attribute__((address_space(3))) void *lptr_t;
+  const int tid = G::opaque_tid(), lane = tid & 63, wave = tid >> 6;
+  auto issue = [&](int q) {
+    const int inst = q * 4 + wave, sl = inst * 64 + lane, r = sl / G::XGR, j = (sl % G::XGR) ^ (r & 15);
+    __builtin_amdgcn_global_load_lds((gptr_t)(X + (size_t)(m0 + r) * ldx + k0 + j * 8), (lptr_t)(lds_x + inst * 1024), 16, 0, kAuxSc1);
+  };
+  auto slot = [&](int q) { return lds_x + (q * 4 + wave) * 1024 + lane * 16; };
+  // Everything is requested at once.  (Waiting on a probe first - this wave's last load, which lies in
+  // the last rows of the slice - costs a second memory round trip once the data is there: measured
+  // 378 us against 350 us for the 12-layer encoder.)
+  constexpr int PER = G::X_INSTR / 4;
+  poll_direct_loads<PER, (1ull << PER) - 1>(issue, slot, fl);
 }
 
 // ------------------------------------------------------------------ stages ----
@@ -120,19 +204,41 @@ __device__ __forceinline__ void stage_partial(half_t *lds, const Params &a, cons
 template <bool COH, int SPLITK>
 __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, const half_t *resid,
                                          const half_t *gam, const half_t *bet, half_t *out,
-                                         int first_row, int row_stride) {
+                                         int first_row, int row_stride, Flow *fl = nullptr) {
   const int lane = threadIdx.x & 63;
   for (int m = first_row; m < a.M; m += row_stride) {
     f4 v[3];
     u4 raw[3][SPLITK];
     u2 rres[3];
     // every load of the row is issued before the first use
+    if (fl) {   // dataflow kernel: partials and residual come from the memory side and are polled
+      for (int spin = 0;; ++spin) {
+        asm volatile("" ::: "memory");     // the loads below are repeated, not hoisted
+        bool bad = false;
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+          const int n = c * 256 + lane * 4;
+#pragma unroll
+          for (int ks = 0; ks < SPLITK; ++ks) raw[c][ks] = ld16<true>(a.part, ((ks * a.M + m) * H + n) * 4);
+          rres[c] = ld8<true>(resid, (m * H + n) * 2);
+        }
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+#pragma unroll
+          for (int ks = 0; ks < SPLITK; ++ks) bad |= has_unwritten(raw[c][ks]);
+          bad |= has_unwritten(rres[c]);
+        }
+        if (!__any(bad)) break;
+        if (fl->failed || spin >= kMaxFlowSpin) { fl->failed = true; break; }
+      }
+    } else {
 #pragma unroll
     for (int c = 0; c < 3; ++c) {
       const int n = c * 256 + lane * 4;
 #pragma unroll
       for (int ks = 0; ks < SPLITK; ++ks) raw[c][ks] = ld16<false>(a.part, ((ks * a.M + m) * H + n) * 4);
       rres[c] = ld8<false>(resid, (m * H + n) * 2);
+    }
     }
 #pragma unroll
     for (int c = 0; c < 3; ++c) {
@@ -274,12 +380,15 @@ __device__ __forceinline__ bool preissue_w(unsigned char *lds, const Items &item
 #endif
 
 // Driver of a skinny GEMM stage.  `w_ready`: the weight slice of this workgroup's first item
-// was queued inside the preceding grid barrier.  `extra()` queues further direct-to-LDS loads
+// was queued earlier (inside the preceding grid barrier, or after the previous stage in the
+// dataflow kernel).  `extra()` queues further direct-to-LDS loads
 // with the operands, `pre(item)` runs after the operands have
-// landed (LayerNorm on load), `epi(item, m, n, lo, hi)` receives 8 consecutive columns of a row,
+// landed (LayerNorm on load), `epi(item, m, n, lo, hi)` receives 8 consecutive columns of a row.
+// With `fl` the X slice is polled (dataflow kernel) unless `x_is_input` (it is then read plainly).
 template <class G, bool COH, class Items, class Extra, class Pre, class Epi>
 __device__ __forceinline__ void gemm_stage(unsigned char *lds, const Items &items, const half_t *X, int ldx, bool w_ready,
-                                           Extra extra, Pre pre, Epi epi, const GridBarrier *tb = nullptr) {
+                                           Extra extra, Pre pre, Epi epi, const GridBarrier *tb = nullptr,
+                                           Flow *fl = nullptr, bool x_is_input = false) {
   const int span = items.span();
   for (int it = blockIdx.x; it < span; it += gridDim.x) {
     Item d;
@@ -287,13 +396,15 @@ __device__ __forceinline__ void gemm_stage(unsigned char *lds, const Items &item
     __syncthreads();                       // LDS reuse
     STAGE_MARK(tb, 0);
     if (!w_ready) G::issue_w(lds + kXRegion, d.W, d.ldw, d.n0, d.k0, d.rot);
-    G::template issue_x<false>(lds, X, ldx, d.m0, d.k0);
     extra();
+    if (fl && !x_is_input) poll_x<G>(lds, X, ldx, d.m0, d.k0, *fl);
+    else G::template issue_x<false>(lds, X, ldx, d.m0, d.k0);
     STAGE_MARK(tb, 1);
 #ifdef SOUFFLE_STAGE_MARKS
     if (tb && tb->trace) { wait_vmcnt<G::X_INSTR / 4>(); trace_mark(*tb, 2); }
 #endif
     G::wait_loads();
+    if (fl) flow_stamp(*fl, 0);
     STAGE_MARK(tb, 3);
     pre(d);
     STAGE_MARK(tb, 4);
@@ -397,37 +508,51 @@ __device__ __forceinline__ void ln_rows_in_lds(unsigned char *lds_x, bool has_ga
 
 template <bool COH>
 __device__ __forceinline__ void stage_ln(const Params &a, int splitk, const half_t *bias, const half_t *resid,
-                                         const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
-  if (splitk == 1) stage_ln_t<COH, 1>(a, bias, resid, gam, bet, out, first_row, row_stride);
-  else stage_ln_t<COH, kSplitFc2Small>(a, bias, resid, gam, bet, out, first_row, row_stride);
+                                         const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride,
+                                         Flow *fl = nullptr) {
+  if (splitk == 1) stage_ln_t<COH, 1>(a, bias, resid, gam, bet, out, first_row, row_stride, fl);
+  else stage_ln_t<COH, kSplitFc2Small>(a, bias, resid, gam, bet, out, first_row, row_stride, fl);
 }
 
-// The four skinny GEMM stages (shared by the megakernel and the per-op kernels).
+// The four skinny GEMM stages (shared by the megakernels and the per-op kernels).  With `fl`
+// (dataflow kernel) the activation slice is polled instead of being loaded after a barrier.
 template <bool COH>
-__device__ __forceinline__ void small_qkv(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, const GridBarrier *tb = nullptr) {
+__device__ __forceinline__ void small_qkv(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready,
+                                          const GridBarrier *tb = nullptr, Flow *fl = nullptr, bool x_is_input = false) {
   gemm_stage<OsFull, COH>(lds, QkvItems{w.w_qkv, a.M}, xin, H, w_ready, []() {}, [](const Item &) {},
     [&](const Item &d, int m, int n, f4 lo, f4 hi) {
       add_bias8(lo, hi, w.b_qkv ? w.b_qkv + d.aux * H : nullptr, n);
       const int b = m / a.S, s = m % a.S, hh = n / HD, dd = n % HD;
       st16<COH>(a.qkv, ((((d.aux * a.B + b) * NH + hh) * a.S + s) * HD + dd) * 2, pack_h8(lo, hi));
-    }, tb);
+    }, tb, fl, x_is_input);
 }
-// z1 = ctx.Wo + b_o + x (pre-LayerNorm, fp16)
+// z1 = ctx.Wo + b_o + x (pre-LayerNorm, fp16).  The residual values of a thread's 8 output
+// columns are requested before the MFMAs and used after them.  In the dataflow kernel the rows
+// of x are known to be complete (the context rows being there implies it) but may be absent
+// from this XCD's L2 or stale in it, hence the memory-side load.
 template <bool COH>
-__device__ __forceinline__ void small_outproj(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready, const GridBarrier *tb = nullptr) {
-  gemm_stage<OsFull, COH>(lds, OutItems{w.w_o, a.M}, a.ctx, H, w_ready, []() {}, [](const Item &) {},
+__device__ __forceinline__ void small_outproj(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, bool w_ready,
+                                              const GridBarrier *tb = nullptr, Flow *fl = nullptr, bool x_is_input = false) {
+  static_assert(OsFull::CPT == 8, "one epilogue call per thread");
+  u4 resid;
+  gemm_stage<OsFull, COH>(lds, OutItems{w.w_o, a.M}, a.ctx, H, w_ready, []() {},
+    [&](const Item &d) {
+      const int tid = threadIdx.x, off = ((d.m0 + tid / 8) * H + d.n0 + (tid % 8) * 8) * 2;
+      resid = (fl && !x_is_input) ? ld16<true>(xin, off) : ld16<false>(xin, off);
+    },
     [&](const Item &, int m, int n, f4 lo, f4 hi) {
       add_bias8(lo, hi, w.b_o, n);
-      const h8 r = as_h8(ld16<false>(xin, (m * H + n) * 2));
+      const h8 r = as_h8(resid);
       lo += f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
       hi += f4{(float)r[4], (float)r[5], (float)r[6], (float)r[7]};
       st16<COH>(a.z1, (m * H + n) * 2, pack_h8(lo, hi));
-    }, tb);
+    }, tb, fl);
 }
 // h = act(LN1(z1).W1 + b1): LayerNorm is applied to the X tile in LDS (every workgroup has
 // complete rows); the workgroups of the first n-tile also publish y1 = LN1(z1).
 template <bool COH>
-__device__ __forceinline__ void small_fc1(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, const GridBarrier *tb = nullptr) {
+__device__ __forceinline__ void small_fc1(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready,
+                                          const GridBarrier *tb = nullptr, Flow *fl = nullptr) {
   gemm_stage<OsFull, COH>(lds, Fc1Items{w.w_fc1, a.M}, a.z1, H, w_ready,
     [&]() { issue_ln_params(lds, w.ln1_g, w.ln1_b); },
     [&](const Item &d) { ln_rows_in_lds<COH>(lds, w.ln1_g != nullptr, w.ln1_b != nullptr, a.eps, d.n0 == 0 ? a.y1 : nullptr, d.m0); },
@@ -439,16 +564,17 @@ __device__ __forceinline__ void small_fc1(unsigned char *lds, const Params &a, c
         hi[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(hi[i], 0.f) : gelu_tanh(hi[i]);
       }
       st16<COH>(a.h, (m * F + n) * 2, pack_h8(lo, hi));
-    }, tb);
+    }, tb, fl);
 }
-// fp32 partials of h.W2 over 8 K slices
+// fp32 partials of h.W2 over 4 K slices
 template <bool COH>
-__device__ __forceinline__ void small_fc2(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready, const GridBarrier *tb = nullptr) {
+__device__ __forceinline__ void small_fc2(unsigned char *lds, const Params &a, const LayerW &w, bool w_ready,
+                                          const GridBarrier *tb = nullptr, Flow *fl = nullptr) {
   gemm_stage<OsFc2, COH>(lds, Fc2Items{w.w_fc2, a.M}, a.h, F, w_ready, []() {}, [](const Item &) {},
     [&](const Item &d, int m, int n, f4 lo, f4 hi) {
       st16<COH>(a.part, ((d.aux * a.M + m) * H + n) * 4, __builtin_bit_cast(u4, lo));
       st16<COH>(a.part, ((d.aux * a.M + m) * H + n + 4) * 4, __builtin_bit_cast(u4, hi));
-    }, tb);
+    }, tb, fl);
 }
 
 // One (batch, head, 64-query block) per workgroup pass; each wave owns 16 queries.
@@ -577,8 +703,17 @@ __device__ __forceinline__ void issue_rows64_wave(unsigned char *lds_tile, const
   }
 }
 
+// One direct-to-LDS load of 8 rows of a [rows][64] fp16 tile, layout as issue_rows64_wave, memory-side.
+template <int MODE>
+__device__ __forceinline__ void issue_row8_sc1(unsigned char *lds_tile, const half_t *src, int r0) {
+  typedef __attribute__((address_space(1))) const void *gptr_t;
+  typedef __attribute__((address_space(3))) void *lptr_t;
+  const int lane = threadIdx.x & 63, r = r0 + (lane >> 3), c = (lane & 7) ^ (MODE == 0 ? ((r >> 1) & 7) : (r & 2));
+  __builtin_amdgcn_global_load_lds((gptr_t)(src + (size_t)r * HD + c * 8), (lptr_t)(lds_tile + r0 * 128), 16, 0, kAuxSc1);
+}
+
 template <bool COH, int NKT>
-__device__ __forceinline__ void attn_item_split(unsigned char *lds, const Params &a, int bh, int qb) {
+__device__ __forceinline__ void attn_item_split(unsigned char *lds, const Params &a, int bh, int qb, Flow *fl = nullptr) {
   constexpr int S = NKT * 16, TPW = NKT / 4;                       // key tiles per wave
   static_assert(NKT % 4 == 0, "keys split evenly over four waves");
   unsigned char *ks_ = lds, *vs_ = lds + S * 128, *qs_ = lds + 2 * S * 128;
@@ -591,10 +726,28 @@ __device__ __forceinline__ void attn_item_split(unsigned char *lds, const Params
   const half_t *Q = a.qkv + head_off + (size_t)qb * 16 * HD, *K = a.qkv + plane + head_off, *V = a.qkv + 2 * plane + head_off;
 
   __syncthreads();   // LDS reuse
-  issue_rows64_wave<0>(qs_ + wave * 2048, Q, 0, 16);               // every wave its own copy of the queries
-  issue_rows64_wave<0>(ks_, K, wave * TPW * 16, TPW * 16);
-  issue_rows64_wave<1>(vs_, V, wave * TPW * 16, TPW * 16);
-  __builtin_amdgcn_s_waitcnt(0);                                   // this wave's rows only: no barrier needed
+  if (fl) {
+    // 2 loads of queries, then TPW*2 of this wave's keys and as many of its values, each polled
+    constexpr int NL = 2 + 4 * TPW;
+    const int lane_b = (threadIdx.x & 63) * 16, kr0 = wave * TPW * 16;
+    auto issue = [&](int i) {
+      if (i < 2) issue_row8_sc1<0>(qs_ + wave * 2048, Q, i * 8);
+      else if (i < 2 + 2 * TPW) issue_row8_sc1<0>(ks_, K, kr0 + (i - 2) * 8);
+      else issue_row8_sc1<1>(vs_, V, kr0 + (i - 2 - 2 * TPW) * 8);
+    };
+    auto slot = [&](int i) {
+      if (i < 2) return qs_ + wave * 2048 + i * 1024 + lane_b;
+      if (i < 2 + 2 * TPW) return ks_ + (kr0 + (i - 2) * 8) * 128 + lane_b;
+      return vs_ + (kr0 + (i - 2 - 2 * TPW) * 8) * 128 + lane_b;
+    };
+    poll_direct_loads<NL, (1ull << NL) - 1>(issue, slot, *fl);
+    flow_stamp(*fl, 0);
+  } else {
+    issue_rows64_wave<0>(qs_ + wave * 2048, Q, 0, 16);             // every wave its own copy of the queries
+    issue_rows64_wave<0>(ks_, K, wave * TPW * 16, TPW * 16);
+    issue_rows64_wave<1>(vs_, V, wave * TPW * 16, TPW * 16);
+    __builtin_amdgcn_s_waitcnt(0);                                 // this wave's rows only: no barrier needed
+  }
 
   const half_t *kh = reinterpret_cast<const half_t *>(ks_), *vh = reinterpret_cast<const half_t *>(vs_),
                *qh = reinterpret_cast<const half_t *>(qs_ + wave * 2048);
@@ -690,13 +843,23 @@ __device__ __forceinline__ void attn_small_range(const Params &a, int stride, in
   *off = (*span + 64 <= stride) ? 64 : 0;
 }
 template <bool COH, int NKT>
-__device__ __forceinline__ void stage_attn_small_t(unsigned char *lds, const Params &a, int first, int stride) {
+__device__ __forceinline__ void stage_attn_small_t(unsigned char *lds, const Params &a, int first, int stride, Flow *fl = nullptr) {
   int off, span;
   attn_small_range(a, stride, &off, &span);
   for (int it = first - off; it < span; it += stride) {
     int qb, bh;
-    if (it >= 0 && xcd_item(it, a.S / 16, a.B * NH, &qb, &bh)) attn_item_split<COH, NKT>(lds, a, bh, qb);
+    if (it >= 0 && xcd_item(it, a.S / 16, a.B * NH, &qb, &bh)) attn_item_split<COH, NKT>(lds, a, bh, qb, fl);
   }
+}
+// Does this workgroup have an attention item?
+__device__ __forceinline__ bool attn_small_busy(const Params &a, int first, int stride) {
+  int off, span;
+  attn_small_range(a, stride, &off, &span);
+  for (int it = first - off; it < span; it += stride) {
+    int qb, bh;
+    if (it >= 0 && xcd_item(it, a.S / 16, a.B * NH, &qb, &bh)) return true;
+  }
+  return false;
 }
 template <bool COH>
 __device__ __forceinline__ void stage_attn_small(unsigned char *lds, const Params &a, int first, int stride) {
@@ -750,6 +913,8 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
   const int wave = threadIdx.x >> 6;
   const half_t *xin = args.x;
   bool qkv_ready = false;
+  // this kernel leaves data in the workspace buffers: the dataflow kernel must refill them
+  if (first == 0 && threadIdx.x == 0) __hip_atomic_store(args.ctl + kCtlFlowWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   for (int l = 0; l < args.num_layers; ++l) {
     const LayerW w = args.layers[l];
     const Params a = layer_params(args, l);
@@ -801,10 +966,128 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
   grid_barrier_end(bar);
 }
 
+// ------------------------------------------------- dataflow megakernel ----
+// The skinny path without grid barriers between stages: every consumer polls its input (see
+// Flow above).  Buffers are per layer; a layer's buffers are put back into the unwritten state
+// by the workgroups that run FC1 items of the NEXT layer, after their own input has arrived:
+// a complete row tile of z1(l+1) implies, through the chain of dependencies (context rows <-
+// all keys and values <- all rows of the layer input <- every LayerNorm-2 row of layer l <- all
+// FC2 partials <- all of h <- all FC1 items <- ...), that every buffer of layer l except its
+// output has been read for the last time.  The layer output is still being read by layer l+1
+// (queries, residual) and is reset one layer later.  What is left at the end is reset after
+// one grid barrier.  Between launches every buffer is therefore in the unwritten state, which
+// the control block records as a layout marker; a launch that does not find its marker (first
+// use, another layout, an earlier failure, or another kernel having used the workspace) fills
+// the buffers first.
+__device__ __forceinline__ void fill_unwritten(void *base, size_t bytes, int part, int parts) {
+  const size_t n16 = bytes / 16, per = (n16 + parts - 1) / parts;
+  const size_t b = per * part, e = b + per < n16 ? b + per : n16;
+  const u4 pat = {~0u, ~0u, ~0u, ~0u};
+  for (size_t i = b + threadIdx.x; i < e; i += 256)
+    st16<true>(base, (int)(i * 16), pat);          // a layer's buffers span far less than 2 GiB
+}
+
+template <int NKT>
+__global__ void __launch_bounds__(256) k_encoder_flow(Args args) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  GridBarrier bar;
+  grid_barrier_begin(bar, args.ctl);
+  Flow fl;
+  fl.failed = false;
+  fl.trace = args.trace;
+  fl.trace_cap = args.trace_cap;
+  fl.stage = 0;
+  const int first = blockIdx.x, stride = gridDim.x, wave = threadIdx.x >> 6;
+  const int L = args.num_layers, M = args.M;
+  if (__hip_atomic_load(args.ctl + kCtlFlowWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != args.flow_marker) {
+    for (int l = 0; l < L; ++l)
+      fill_unwritten(reinterpret_cast<char *>(args.qkv) + (size_t)l * args.layer_stride, args.layer_stride, first, stride);
+    grid_sync(bar);
+  }
+  // Weight slice prefetch: at most one slice is in flight or resident (the W region of LDS); it is
+  // queued as soon as the region is free, for the next GEMM stage in which this workgroup has an
+  // item.  `pf` names that stage (layer * 5 + position; positions 0 QKV, 1 attention, 2 out, 3 FC1, 4 FC2).
+  int pf = -1;
+  const bool attn_busy = attn_small_busy(args, first, stride);
+  auto prefetch_after = [&](int l, int pos) {
+    if (pf >= 0) return;
+    for (int step = 1; step <= 5; ++step) {
+      const int q = pos + step, ll = l + q / 5, pp = q % 5;
+      if (ll >= L) return;
+      if (pp == 1) { if (attn_busy) return; continue; }
+      const LayerW &w = args.layers[ll];
+      Item d;
+      bool ok = false;
+      if (pp == 0) { const QkvItems it{w.w_qkv, M}; ok = first < it.span() && it.at(first, d); }
+      else if (pp == 2) { const OutItems it{w.w_o, M}; ok = first < it.span() && it.at(first, d); }
+      else if (pp == 3) { const Fc1Items it{w.w_fc1, M}; ok = first < it.span() && it.at(first, d); }
+      else { const Fc2Items it{w.w_fc2, M}; ok = first < it.span() && it.at(first, d); }
+      if (ok) {
+        OsFull::issue_w(lds_raw + kXRegion, d.W, d.ldw, d.n0, d.k0, d.rot);
+        pf = ll * 5 + pp;
+        return;
+      }
+    }
+  };
+  auto take = [&](int l, int pos) { const bool r = pf == l * 5 + pos; if (r) pf = -1; return r; };
+  static_assert(std::is_same<OsFull, OsFc2>::value, "one slice shape for every stage");
+  // workgroups that reset: those with an FC1 item (all `it` below the span are valid: 48 slices)
+  const int fc1_span = Fc1Items{nullptr, M}.span();
+  const int resetters = fc1_span < stride ? fc1_span : stride;
+
+  prefetch_after(0, -1);
+  const half_t *xin = args.x;
+  for (int l = 0; l < L; ++l) {
+    const LayerW w = args.layers[l];
+    const Params a = layer_params(args, l);
+    half_t *yout = (l == L - 1) ? a.y : a.yl;
+    const bool in0 = l == 0;                       // the layer input is the caller's tensor: nothing to poll
+
+    small_qkv<true>(lds_raw, a, w, xin, take(l, 0), nullptr, &fl, in0);
+    flow_stamp(fl, 1); fl.stage++;
+    prefetch_after(l, 0);
+
+    stage_attn_small_t<true, NKT>(lds_raw, a, first, stride, &fl);
+    flow_stamp(fl, 1); fl.stage++;
+    if (attn_busy) { __syncthreads(); prefetch_after(l, 1); }
+
+    small_outproj<true>(lds_raw, a, w, xin, take(l, 2), nullptr, &fl, in0);
+    flow_stamp(fl, 1); fl.stage++;
+    prefetch_after(l, 2);
+
+    small_fc1<true>(lds_raw, a, w, take(l, 3), nullptr, &fl);
+    flow_stamp(fl, 1); fl.stage++;
+    prefetch_after(l, 3);
+    if (l >= 1 && first < resetters) {
+      fill_unwritten(reinterpret_cast<char *>(args.qkv) + (size_t)(l - 1) * args.layer_stride, args.flow_bytes, first, resetters);
+      if (l >= 2) fill_unwritten(reinterpret_cast<char *>(args.yl) + (size_t)(l - 2) * args.layer_stride, (size_t)M * H * 2, first, resetters);
+    }
+
+    small_fc2<true>(lds_raw, a, w, take(l, 4), nullptr, &fl);
+    flow_stamp(fl, 1); fl.stage++;
+    prefetch_after(l, 4);
+
+    stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, wave * stride + first, stride * 4, &fl);
+    flow_stamp(fl, 1); fl.stage++;
+    xin = yout;
+  }
+  if (fl.failed && threadIdx.x == 0) (void)__hip_atomic_fetch_or(args.ctl + kCtlErrWord, 4u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  grid_sync(bar);                                  // everything has been consumed
+  fill_unwritten(reinterpret_cast<char *>(args.qkv) + (size_t)(L - 1) * args.layer_stride, args.flow_bytes, first, stride);
+  if (L >= 2) fill_unwritten(reinterpret_cast<char *>(args.yl) + (size_t)(L - 2) * args.layer_stride, (size_t)M * H * 2, first, stride);
+  if (first == 0 && threadIdx.x == 0) {
+    const unsigned err = __hip_atomic_load(args.ctl + kCtlErrWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(args.ctl + kCtlFlowWord, err ? 0u : args.flow_marker, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  grid_barrier_end(bar);
+}
+
 // ------------------------------------------------------ per-op kernels ----
 template <bool LARGE>
 __global__ void __launch_bounds__(256) k_qkv(Args a, int l, const half_t *xin) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  // the per-op chain leaves data in the workspace buffers: the dataflow kernel must refill them
+  if (blockIdx.x == 0 && threadIdx.x == 0) __hip_atomic_store(a.ctl + kCtlFlowWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
   if constexpr (LARGE) stage_qkv<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], xin, blockIdx.x, gridDim.x);
   else small_qkv<false>(lds_raw, a, a.layers[l], xin, false);
@@ -849,6 +1132,8 @@ struct Plan {
   bool large;
   int splitk_o, splitk_f;
   size_t off_ctl, off_qkv, off_ctx, off_z1, off_y1, off_h, off_yl, off_part, layer_stride, total;
+  size_t flow_bytes;      // a layer's buffers without its output (which comes last)
+  unsigned flow_marker;
 };
 
 static int validate(const souffle_bert_cfg *c) {
@@ -882,10 +1167,13 @@ static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   p.off_z1 = take(M * H * 2);
   p.off_y1 = take(M * H * 2);
   p.off_h = take(M * F * 2);
-  p.off_yl = take(M * H * 2);
   p.off_part = take((size_t)(p.splitk_f > p.splitk_o ? p.splitk_f : p.splitk_o) * M * H * 4);
+  p.off_yl = take(M * H * 2);
   p.layer_stride = off - first;                       // one set of inter-stage buffers per layer
+  p.flow_bytes = p.off_yl - p.off_qkv;
   p.total = first + p.layer_stride * (size_t)(num_layers < 1 ? 1 : num_layers);
+  // names the layout (rows, layers, extent) in the control block; never 0
+  p.flow_marker = (unsigned)((M * 2654435761ull) ^ ((size_t)num_layers * 40503ull) ^ (p.total >> 4)) | 0x80000000u;
   return p;
 }
 
@@ -910,6 +1198,8 @@ static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_laye
   a.h = reinterpret_cast<half_t *>(base + p.off_h);
   a.yl = reinterpret_cast<half_t *>(base + p.off_yl);
   a.layer_stride = p.layer_stride;
+  a.flow_bytes = p.flow_bytes;
+  a.flow_marker = p.flow_marker;
   a.part = reinterpret_cast<float *>(base + p.off_part);
   a.probs = nullptr;
   a.trace = nullptr;
@@ -960,6 +1250,27 @@ static int launch_mega(Args &a, int grid, hipStream_t st) {
   }
 }
 
+template <int NKT>
+static int launch_flow_t(Args &a, int grid, hipStream_t st) {
+  const int lds = lds_bytes(false);
+  static bool attr_done = false;
+  if (!attr_done) {
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_encoder_flow<NKT>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    attr_done = true;
+  }
+  void *args[] = {&a};
+  return launch_persistent((const void *)k_encoder_flow<NKT>, grid, 256, args, lds, st);
+}
+static int launch_flow(Args &a, int grid, hipStream_t st) {
+  switch (a.S) {
+    case 64: return launch_flow_t<4>(a, grid, st);
+    case 128: return launch_flow_t<8>(a, grid, st);
+    case 256: return launch_flow_t<16>(a, grid, st);
+    case 384: return launch_flow_t<24>(a, grid, st);
+    default: return launch_flow_t<32>(a, grid, st);
+  }
+}
+
 static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *layers, int nl, const void *x,
                      const void *mask, void *y, const souffle_bert_dump *dump, void *ws, size_t ws_bytes,
                      souffle_stream_t stream) {
@@ -972,6 +1283,9 @@ static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *laye
   if (int rc = fill_args(a, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
   stage_trace(&a.trace, &a.trace_cap, df.num_cus);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  // Skinny shapes run the dataflow kernel unless per-stage tensors are asked for (those are the
+  // caller's buffers, which do not start in the unwritten state) or it has been switched off.
+  if (!p.large && !dump && bert_sync_mode() == SOUFFLE_SYNC_DATAFLOW) return launch_flow(a, df.num_cus, st);
   return p.large ? launch_mega<true>(a, df.num_cus, st) : launch_mega<false>(a, df.num_cus, st);
 }
 

@@ -23,6 +23,9 @@ struct DeviceFacts {
 // Cached per process for the current device; returns a negative status on failure.
 int device_facts(DeviceFacts *out);
 
+// SOUFFLE_SYNC_* selected by souffle_set_bert_sync / SOUFFLE_BERT_SYNC.
+int bert_sync_mode();
+
 // Process-wide stage-trace buffer set by souffle_set_stage_trace (NULL = tracing off).
 void stage_trace(unsigned long long **buf, int *max_barriers, int nblk);
 

@@ -69,6 +69,8 @@ SIGNATURES = {
     "souffle_set_stage_trace": (C.c_int, [C.c_void_p, C.c_size_t]),
     "souffle_set_cooperative_launch": (C.c_int, [C.c_int]),
     "souffle_workspace_init": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
+    "souffle_workspace_status": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_uint), C.c_int]),
+    "souffle_set_bert_sync": (C.c_int, [C.c_int]),
     "souffle_bert_workspace_bytes": (C.c_size_t, [C.POINTER(BertCfg)]),
     "souffle_bert_layer_fused": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
                                            C.c_void_p, C.POINTER(BertDump), C.c_void_p, C.c_size_t, C.c_void_p]),
@@ -153,6 +155,12 @@ class Workspace:
     def ptr(self):
         return self.buf.data_ptr()
 
+    def status(self, clear=False):
+        """Wait for the current stream and return the sticky failure flags (0 = all launches completed)."""
+        flags = C.c_uint(0)
+        check(lib().souffle_workspace_status(self.buf.data_ptr(), current_stream(), C.byref(flags), 1 if clear else 0))
+        return flags.value
+
 
 def set_stage_trace(tensor):
     """Point the in-kernel stage trace at an int64 CUDA tensor (None = off)."""
@@ -160,6 +168,15 @@ def set_stage_trace(tensor):
         check(lib().souffle_set_stage_trace(None, 0))
     else:
         check(lib().souffle_set_stage_trace(tensor.data_ptr(), tensor.numel() * tensor.element_size()))
+
+
+SYNC_DATAFLOW, SYNC_BARRIER = 0, 1
+
+
+def set_bert_sync(mode):
+    """Hand-over between the stages of the skinny fused encoder: "dataflow" (default) or "barrier"."""
+    modes = {"dataflow": SYNC_DATAFLOW, "barrier": SYNC_BARRIER, SYNC_DATAFLOW: SYNC_DATAFLOW, SYNC_BARRIER: SYNC_BARRIER}
+    check(lib().souffle_set_bert_sync(modes[mode]))
 
 
 def set_cooperative_launch(on):

@@ -102,6 +102,32 @@ def test_encoder_matches_oracle(B, S, layers):
     assert torch.equal(y_f, y_u)
 
 
+@pytest.mark.parametrize("B,S,layers", [(1, 128, 12), (1, 384, 2), (2, 64, 3), (1, 128, 1)])
+def test_dataflow_sync_equals_barrier_sync(B, S, layers):
+    """The dataflow hand-over (consumers poll the data) runs the same arithmetic as the grid-barrier
+    one: bit-identical results, also on a second launch (buffers put back into the unwritten state by
+    the first) and after the per-op chain has left data in the shared workspace."""
+    announce("bert encoder dataflow sync B=%d S=%d L=%d" % (B, S, layers))
+    import bert_binding
+    import souffle_hip as sh
+    ws = [synth.bert_layer_weights(2, l) for l in range(layers)]
+    x = dev(synth.bert_input(2, B, S))
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    y_b = enc(x).clone()
+    sh.set_bert_sync("dataflow")
+    try:
+        y_1 = enc(x).clone()
+        y_2 = enc(x).clone()
+        y_u = enc(x, fused=False).clone()
+        y_3 = enc(x).clone()
+        flags = enc.ws.status()
+    finally:
+        sh.set_bert_sync("barrier")
+    assert flags == 0, "a bounded wait gave up (flags %d)" % flags
+    assert torch.equal(y_1, y_b) and torch.equal(y_2, y_b) and torch.equal(y_3, y_b) and torch.equal(y_u, y_b)
+    assert_close("encoder dataflow", y_1, oracle.bert_encoder(synth.bert_input(2, B, S), ws, B, S))
+
+
 def test_layernorm_invariants_at_full_size():
     """Size-independent property: with gamma 1 / beta 0 every output row has mean 0, variance 1."""
     announce("bert LN invariants B=32")
