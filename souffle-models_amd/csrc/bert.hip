@@ -15,6 +15,7 @@
 #include <type_traits>
 #include "gemm_oneshot.hpp"
 #include "gemm_tile.hpp"
+#include "gemm_big.hpp"
 #include "host_util.hpp"
 
 namespace souffle {
@@ -35,6 +36,7 @@ struct LayerW {
 // an activation once instead of every workgroup fetching it from memory.
 struct Params {
   int B, S, M, act, num_layers, splitk_o, splitk_f;
+  int big;             // rows are a multiple of 256 and many: the 256-row GEMM tiles are used
   float scale, eps;
   const half_t *x, *mask;
   half_t *y;
@@ -143,6 +145,27 @@ __device__ __forceinline__ void poll_x(unsigned char *lds_x, const half_t *X, in
 }
 
 // ------------------------------------------------------------------ stages ----
+__device__ __forceinline__ f4 add_bias4(f4 v, const half_t *bias, int n) {
+  if (bias) {
+    const h4 bb = *reinterpret_cast<const h4 *>(bias + n);
+    v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+  }
+  return v;
+}
+
+__device__ __forceinline__ void add_bias8(f4 &lo, f4 &hi, const half_t *bias, int n) {
+  if (bias) {
+    const h8 bb = *reinterpret_cast<const h8 *>(bias + n);
+    lo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+    hi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]};
+  }
+}
+__device__ __forceinline__ u4 pack_h8(f4 lo, f4 hi) {
+  const h8 r = {(half_t)lo[0], (half_t)lo[1], (half_t)lo[2], (half_t)lo[3], (half_t)hi[0], (half_t)hi[1], (half_t)hi[2], (half_t)hi[3]};
+  return as_u4(r);
+}
+
+
 template <bool COH, class Tile>
 __device__ __forceinline__ void stage_qkv(half_t *lds, const Params &a, const LayerW &w, const half_t *xin,
                                           int first, int stride) {
@@ -257,6 +280,133 @@ __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, 
     float sum = 0.f;
 #pragma unroll
     for (int c = 0; c < 3; ++c) sum += v[c][0] + v[c][1] + v[c][2] + v[c][3];
+    const float mean = wave_sum(sum) * (1.0f / H);
+    float sq = 0.f;
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { const float d = v[c][i] - mean; sq += d * d; }
+    const float rstd = rsqrtf(wave_sum(sq) * (1.0f / H) + a.eps);
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      const int n = c * 256 + lane * 4;
+      f4 o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = (v[c][i] - mean) * rstd;
+      if (gam) {
+        const h4 gg = *reinterpret_cast<const h4 *>(gam + n);
+        o *= f4{(float)gg[0], (float)gg[1], (float)gg[2], (float)gg[3]};
+      }
+      if (bet) {
+        const h4 bb = *reinterpret_cast<const h4 *>(bet + n);
+        o += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+      }
+      st8<COH>(out, (m * H + n) * 2, pack_h4(o));
+    }
+  }
+}
+
+// ---- many rows (M a multiple of 256): 256 x BN tiles, see gemm_big.hpp ----
+// BN is chosen per GEMM so that M = 4096 gives exactly 256 tiles, one per CU: 144 for the
+// 2304 QKV columns, 192 for FC1's 3072, 48 for the 768 of the out-projection and FC2.
+using BigQkv = GemmBig<144, 5>;
+using BigFc1 = GemmBig<192, 5>;
+using BigOut = GemmBig<48, 5>;
+constexpr int kBigLds = BigFc1::LDS_BYTES;
+static_assert(BigQkv::LDS_BYTES <= kBigLds && BigOut::LDS_BYTES <= kBigLds, "FC1 has the largest ring");
+
+// Workgroup b runs on XCD b % 8.  An XCD gets a quarter of the row tiles and half of the
+// column tiles, so that its L2 fetches each operand tile it needs once.
+__device__ __forceinline__ void big_tile(int it, int m_tiles, int n_tiles, int *tm, int *tn) {
+  if ((gridDim.x & 7) == 0 && (m_tiles & 3) == 0 && (n_tiles & 1) == 0) {
+    const int x = it & 7, i = it >> 3, mq = m_tiles >> 2;
+    *tm = (x & 3) * mq + i % mq;
+    *tn = (x >> 2) * (n_tiles >> 1) + i / mq;
+  } else {
+    *tm = it / n_tiles;
+    *tn = it % n_tiles;
+  }
+}
+
+template <bool COH>
+__device__ __forceinline__ void big_qkv(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, int first, int stride) {
+  const int m_tiles = a.M / 256, n_tiles = 3 * H / BigQkv::kBN;
+  for (int it = first; it < m_tiles * n_tiles; it += stride) {
+    int tm, tn;
+    big_tile(it, m_tiles, n_tiles, &tm, &tn);
+    const int n0 = tn * BigQkv::kBN;
+    // the three [768][768] matrices are addressed as one [768][2304]
+    auto wptr = [&](int k, int col) {
+      const int c = n0 + col, j = c / H;
+      return w.w_qkv + ((size_t)j * H + k) * H + (c - j * H);
+    };
+    auto cvt = [&](int, int nr, f4 v) {
+      const int c = n0 + nr, j = c / H, n = c - j * H;
+      return pack_h4(add_bias4(v, w.b_qkv ? w.b_qkv + j * H : nullptr, n));
+    };
+    auto store16 = [&](int m, int nr, u4 v) {                // 8 columns never straddle a head (64 columns)
+      const int c = n0 + nr, j = c / H, n = c - j * H;
+      const int b = m / a.S, s = m % a.S, hh = n / HD, d = n % HD;
+      st16<COH>(a.qkv, ((((j * a.B + b) * NH + hh) * a.S + s) * HD + d) * 2, v);
+    };
+    BigQkv::run(lds, xin, H, tm * 256, 0, H / 32, wptr, cvt, store16);
+  }
+}
+template <bool COH>
+__device__ __forceinline__ void big_fc1(unsigned char *lds, const Params &a, const LayerW &w, int first, int stride) {
+  const int m_tiles = a.M / 256, n_tiles = F / BigFc1::kBN;
+  for (int it = first; it < m_tiles * n_tiles; it += stride) {
+    int tm, tn;
+    big_tile(it, m_tiles, n_tiles, &tm, &tn);
+    const int n0 = tn * BigFc1::kBN;
+    auto wptr = [&](int k, int col) { return w.w_fc1 + (size_t)k * F + n0 + col; };
+    auto cvt = [&](int, int nr, f4 v) {
+      v = add_bias4(v, w.b_fc1, n0 + nr);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(v[i], 0.f) : gelu_tanh(v[i]);
+      return pack_h4(v);
+    };
+    auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.h, (m * F + n0 + nr) * 2, v); };
+    BigFc1::run(lds, a.y1, H, tm * 256, 0, H / 32, wptr, cvt, store16);
+  }
+}
+// z = X[M][K].W[K][768] + bias + resid, fp16, into a.z1 (the pre-LayerNorm sum of the out-projection
+// and of FC2; no split of K: 256 tiles already fill the device)
+template <bool COH>
+__device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, const half_t *X, int K, const half_t *W,
+                                           const half_t *bias, const half_t *resid, int first, int stride) {
+  const int m_tiles = a.M / 256, n_tiles = H / BigOut::kBN;
+  for (int it = first; it < m_tiles * n_tiles; it += stride) {
+    int tm, tn;
+    big_tile(it, m_tiles, n_tiles, &tm, &tn);
+    const int n0 = tn * BigOut::kBN;
+    auto wptr = [&](int k, int col) { return W + (size_t)k * H + n0 + col; };
+    auto cvt = [&](int m, int nr, f4 v) {
+      const int n = n0 + nr;
+      const h4 r = as_h4(ld8<false>(resid, (m * H + n) * 2));
+      v = add_bias4(v, bias, n) + f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+      return pack_h4(v);
+    };
+    auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.z1, (m * H + n0 + nr) * 2, v); };
+    BigOut::run(lds, X, K, tm * 256, 0, K / 32, wptr, cvt, store16);
+  }
+}
+// out[m] = LN(z1[m]) * g + b; one wave per row, two-pass statistics in fp32 registers
+template <bool COH>
+__device__ __forceinline__ void big_ln(const Params &a, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
+  const int lane = opaque_thread_id() & 63;
+  for (int m = first_row; m < a.M; m += row_stride) {
+    u2 raw[3];
+#pragma unroll
+    for (int c = 0; c < 3; ++c) raw[c] = ld8<false>(a.z1, (m * H + c * 256 + lane * 4) * 2);
+    f4 v[3];
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      const h4 r = as_h4(raw[c]);
+      v[c] = f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+      sum += v[c][0] + v[c][1] + v[c][2] + v[c][3];
+    }
     const float mean = wave_sum(sum) * (1.0f / H);
     float sq = 0.f;
 #pragma unroll
@@ -415,26 +565,6 @@ __device__ __forceinline__ void gemm_stage(unsigned char *lds, const Items &item
 #endif
     w_ready = false;
   }
-}
-
-__device__ __forceinline__ f4 add_bias4(f4 v, const half_t *bias, int n) {
-  if (bias) {
-    const h4 bb = *reinterpret_cast<const h4 *>(bias + n);
-    v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
-  }
-  return v;
-}
-
-__device__ __forceinline__ void add_bias8(f4 &lo, f4 &hi, const half_t *bias, int n) {
-  if (bias) {
-    const h8 bb = *reinterpret_cast<const h8 *>(bias + n);
-    lo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
-    hi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]};
-  }
-}
-__device__ __forceinline__ u4 pack_h8(f4 lo, f4 hi) {
-  const h8 r = {(half_t)lo[0], (half_t)lo[1], (half_t)lo[2], (half_t)lo[3], (half_t)hi[0], (half_t)hi[1], (half_t)hi[2], (half_t)hi[3]};
-  return as_u4(r);
 }
 
 // LayerNorm of the 32 complete rows of an OsFull X tile, in place in LDS.  Eight lanes
@@ -601,7 +731,7 @@ __device__ __forceinline__ void attn_item(half_t *lds_h, const Params &a, int it
   constexpr int S = NKT * 16;
   unsigned char *lds = reinterpret_cast<unsigned char *>(lds_h);
   unsigned char *ks_ = lds, *vs_ = lds + S * 128, *qs_ = lds + 2 * S * 128;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+  const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
   const int qblocks = S / 64;
   const int qb = item % qblocks, bh = item / qblocks, b = bh / NH, hh = bh % NH;
   const int head_off = ((b * NH + hh) * S) * HD;                 // halves, within one of q/k/v
@@ -895,13 +1025,15 @@ using TileSmall = GemmTile<64, 64, 64, 2, 2>;
 using TileLarge = GemmTile<128, 128, 64, 2, 2>;
 constexpr int kAttnLdsBytes = attn_small_lds_bytes(512) > 2 * 512 * 128 + 64 * 128 ? attn_small_lds_bytes(512) : 2 * 512 * 128 + 64 * 128;
 constexpr int lds_bytes(bool large) {
-  const int t = large ? TileLarge::LDS_BYTES : kSmallGemmLds;
+  const int t = large ? (TileLarge::LDS_BYTES > kBigLds ? TileLarge::LDS_BYTES : kBigLds) : kSmallGemmLds;
   return t > kAttnLdsBytes ? t : kAttnLdsBytes;
 }
 
 // ------------------------------------------------------------ megakernel ----
-template <bool LARGE, int NKT>
+// MODE 0: skinny path (M < 1024); 1: 128 x 128 tiles; 2: 256-row tiles (M >= 2048, a multiple of 256)
+template <int MODE, int NKT>
 __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
+  constexpr bool LARGE = MODE != 0, BIG = MODE == 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   half_t *lds = reinterpret_cast<half_t *>(lds_raw);
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
@@ -920,19 +1052,25 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
     const Params a = layer_params(args, l);
     half_t *yout = (l == a.num_layers - 1) ? a.y : a.yl;
     if constexpr (LARGE) {
-      stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
+      if constexpr (BIG) big_qkv<true>(lds_raw, a, w, xin, first, stride);
+      else stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
       grid_sync(bar);
       stage_attn_t<true, NKT>(lds, a, first, stride);
       grid_sync(bar);
-      stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
+      if constexpr (BIG) big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, xin, first, stride);
+      else stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
       grid_sync(bar);
-      stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
+      if constexpr (BIG) big_ln<true>(a, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
+      else stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
       grid_sync(bar);
-      stage_fc1<true, Tile>(lds, a, w, first, stride);
+      if constexpr (BIG) big_fc1<true>(lds_raw, a, w, first, stride);
+      else stage_fc1<true, Tile>(lds, a, w, first, stride);
       grid_sync(bar);
-      stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
+      if constexpr (BIG) big_presum<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, a.y1, first, stride);
+      else stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
       grid_sync(bar);
-      stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
+      if constexpr (BIG) big_ln<true>(a, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
+      else stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
     } else {
       // Weight slices are queued one stage ahead, from inside the grid barrier that precedes
       // the stage.
@@ -1083,14 +1221,17 @@ __global__ void __launch_bounds__(256) k_encoder_flow(Args args) {
 }
 
 // ------------------------------------------------------ per-op kernels ----
-template <bool LARGE>
+template <int MODE>
 __global__ void __launch_bounds__(256) k_qkv(Args a, int l, const half_t *xin) {
+  constexpr bool LARGE = MODE != 0, BIG = MODE == 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   // the per-op chain leaves data in the workspace buffers: the dataflow kernel must refill them
   if (blockIdx.x == 0 && threadIdx.x == 0) __hip_atomic_store(a.ctl + kCtlFlowWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
-  if constexpr (LARGE) stage_qkv<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], xin, blockIdx.x, gridDim.x);
-  else small_qkv<false>(lds_raw, a, a.layers[l], xin, false);
+  if constexpr (LARGE) {
+    if constexpr (BIG) big_qkv<false>(lds_raw, a, a.layers[l], xin, blockIdx.x, gridDim.x);
+    else stage_qkv<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], xin, blockIdx.x, gridDim.x);
+  } else small_qkv<false>(lds_raw, a, a.layers[l], xin, false);
 }
 __global__ void __launch_bounds__(256) k_attn(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -1100,12 +1241,15 @@ __global__ void __launch_bounds__(256) k_attn_small(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   stage_attn_small<false>(lds_raw, a, blockIdx.x, gridDim.x);
 }
-template <bool LARGE>
+template <int MODE>
 __global__ void __launch_bounds__(256) k_partial(Args a, const half_t *X, int K, const half_t *W, int splitk) {
+  constexpr bool LARGE = MODE != 0, BIG = MODE == 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
-  if constexpr (LARGE) stage_partial<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, X, K, W, splitk, blockIdx.x, gridDim.x);
-  else {
+  if constexpr (LARGE) {
+    static_assert(!BIG, "the 256-row path writes fp16 pre-LayerNorm sums: k_presum_big");
+    stage_partial<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, X, K, W, splitk, blockIdx.x, gridDim.x);
+  } else {
     LayerW w{};
     w.w_fc2 = W;
     small_fc2<false>(lds_raw, a, w, false);
@@ -1115,12 +1259,22 @@ __global__ void __launch_bounds__(256) k_ln(Args a, int splitk, const half_t *bi
                                             const half_t *gam, const half_t *bet, half_t *out) {
   stage_ln<false>(a, splitk, bias, resid, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
 }
-template <bool LARGE>
+__global__ void __launch_bounds__(256) k_presum_big(Args a, const half_t *X, int K, const half_t *W, const half_t *bias, const half_t *resid) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  big_presum<false>(lds_raw, a, X, K, W, bias, resid, blockIdx.x, gridDim.x);
+}
+__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *gam, const half_t *bet, half_t *out) {
+  big_ln<false>(a, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
+}
+template <int MODE>
 __global__ void __launch_bounds__(256) k_fc1(Args a, int l) {
+  constexpr bool LARGE = MODE != 0, BIG = MODE == 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   using Tile = typename std::conditional<LARGE, TileLarge, TileSmall>::type;
-  if constexpr (LARGE) stage_fc1<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], blockIdx.x, gridDim.x);
-  else small_fc1<false>(lds_raw, a, a.layers[l], false);
+  if constexpr (LARGE) {
+    if constexpr (BIG) big_fc1<false>(lds_raw, a, a.layers[l], blockIdx.x, gridDim.x);
+    else stage_fc1<false, Tile>(reinterpret_cast<half_t *>(lds_raw), a, a.layers[l], blockIdx.x, gridDim.x);
+  } else small_fc1<false>(lds_raw, a, a.layers[l], false);
 }
 __global__ void __launch_bounds__(256) k_outproj_small(Args a, int l, const half_t *xin) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -1129,7 +1283,7 @@ __global__ void __launch_bounds__(256) k_outproj_small(Args a, int l, const half
 
 // ------------------------------------------------------------------- host ----
 struct Plan {
-  bool large;
+  bool large, big;
   int splitk_o, splitk_f;
   size_t off_ctl, off_qkv, off_ctx, off_z1, off_y1, off_h, off_yl, off_part, layer_stride, total;
   size_t flow_bytes;      // a layer's buffers without its output (which comes last)
@@ -1156,6 +1310,7 @@ static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   Plan p;
   const size_t M = (size_t)c->batch * c->seq_len;
   p.large = M >= 1024;
+  p.big = M >= 2048 && M % 256 == 0;
   p.splitk_o = 1;
   p.splitk_f = p.large ? 1 : kSplitFc2Small;
   size_t off = 0;
@@ -1189,6 +1344,7 @@ static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_laye
   char *base = static_cast<char *>(ws);
   a.B = c->batch; a.S = c->seq_len; a.M = c->batch * c->seq_len; a.act = c->act; a.num_layers = nl;
   a.splitk_o = p.splitk_o; a.splitk_f = p.splitk_f; a.scale = c->scale; a.eps = c->ln_eps;
+  a.big = p.big ? 1 : 0;
   a.x = static_cast<const half_t *>(x); a.mask = static_cast<const half_t *>(mask); a.y = static_cast<half_t *>(y);
   a.ctl = reinterpret_cast<unsigned *>(base + p.off_ctl);
   a.qkv = reinterpret_cast<half_t *>(base + p.off_qkv);
@@ -1227,26 +1383,26 @@ static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_laye
   return SOUFFLE_OK;
 }
 
-template <bool LARGE, int NKT>
+template <int MODE, int NKT>
 static int launch_mega_t(Args &a, int grid, hipStream_t st) {
-  const int lds = lds_bytes(LARGE);
+  const int lds = lds_bytes(MODE != 0);
   static bool attr_done = false;
   if (!attr_done) {
-    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_encoder_mega<LARGE, NKT>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_encoder_mega<MODE, NKT>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     attr_done = true;
   }
   void *args[] = {&a};
-  return launch_persistent((const void *)k_encoder_mega<LARGE, NKT>, grid, 256, args, lds, st);
+  return launch_persistent((const void *)k_encoder_mega<MODE, NKT>, grid, 256, args, lds, st);
 }
 // one kernel per supported sequence length, so that each carries only its own attention tile
-template <bool LARGE>
+template <int MODE>
 static int launch_mega(Args &a, int grid, hipStream_t st) {
   switch (a.S) {
-    case 64: return launch_mega_t<LARGE, 4>(a, grid, st);
-    case 128: return launch_mega_t<LARGE, 8>(a, grid, st);
-    case 256: return launch_mega_t<LARGE, 16>(a, grid, st);
-    case 384: return launch_mega_t<LARGE, 24>(a, grid, st);
-    default: return launch_mega_t<LARGE, 32>(a, grid, st);
+    case 64: return launch_mega_t<MODE, 4>(a, grid, st);
+    case 128: return launch_mega_t<MODE, 8>(a, grid, st);
+    case 256: return launch_mega_t<MODE, 16>(a, grid, st);
+    case 384: return launch_mega_t<MODE, 24>(a, grid, st);
+    default: return launch_mega_t<MODE, 32>(a, grid, st);
   }
 }
 
@@ -1286,19 +1442,21 @@ static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *laye
   // Skinny shapes run the dataflow kernel unless per-stage tensors are asked for (those are the
   // caller's buffers, which do not start in the unwritten state) or it has been switched off.
   if (!p.large && !dump && bert_sync_mode() == SOUFFLE_SYNC_DATAFLOW) return launch_flow(a, df.num_cus, st);
-  return p.large ? launch_mega<true>(a, df.num_cus, st) : launch_mega<false>(a, df.num_cus, st);
+  return p.big ? launch_mega<2>(a, df.num_cus, st) : p.large ? launch_mega<1>(a, df.num_cus, st) : launch_mega<0>(a, df.num_cus, st);
 }
 
-template <bool LARGE>
+template <int MODE>
 static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
-  constexpr int GEMM_LDS = LARGE ? TileLarge::LDS_BYTES : kSmallGemmLds;
+  constexpr bool LARGE = MODE != 0;
+  constexpr int GEMM_LDS = LARGE ? lds_bytes(true) : kSmallGemmLds;
   constexpr int BN = LARGE ? 128 : 64;
   constexpr int BM_QKV = LARGE ? 128 : OsFull::kBM, BM_OUT = LARGE ? 128 : OsFull::kBM, BM_FC2 = LARGE ? 128 : OsFc2::kBM;
   static bool attr_done = false;
   if (!attr_done) {
-    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_qkv<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
-    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_partial<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
-    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_fc1<LARGE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_qkv<MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
+    if constexpr (MODE == 2) SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_presum_big, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
+    else SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_partial<MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_fc1<MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_attn, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLdsBytes));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_attn_small, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLdsBytes));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_outproj_small, hipFuncAttributeMaxDynamicSharedMemorySize, kSmallGemmLds));
@@ -1310,18 +1468,26 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
   for (int l = 0; l < nl; ++l) {
     const LayerW &w = a.layers[l];
     half_t *yout = (l == nl - 1) ? a.y : a.yl;
-    hipLaunchKernelGGL(k_qkv<LARGE>, dim3(grid_for((a.M / BM_QKV) * (3 * H / BN))), dim3(256), GEMM_LDS, st, a, l, xin);
+    hipLaunchKernelGGL(k_qkv<MODE>, dim3(grid_for((a.M / BM_QKV) * (3 * H / BN))), dim3(256), GEMM_LDS, st, a, l, xin);
     if (LARGE) hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), 2 * a.S * 128 + 64 * 128, st, a);
     else hipLaunchKernelGGL(k_attn_small, dim3(grid_for((a.B * NH + 7) / 8 * 8 * (a.S / 16))), dim3(256), attn_small_lds_bytes(a.S), st, a);
-    if (LARGE) {
-      hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, 1);
+    if constexpr (MODE == 2) {
+      hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * (H / BigOut::kBN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, w.b_o, xin);
+      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, w.ln1_g, w.ln1_b, a.y1);
+    } else if constexpr (LARGE) {
+      hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, 1);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, 1, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
     } else {   // small M: LN1 is applied by the FC1 kernel on its LDS-resident rows
       hipLaunchKernelGGL(k_outproj_small, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, l, xin);
     }
-    hipLaunchKernelGGL(k_fc1<LARGE>, dim3(grid_for((a.M / BM_QKV) * (F / BN))), dim3(256), GEMM_LDS, st, a, l);
-    hipLaunchKernelGGL(k_partial<LARGE>, dim3(grid_for((a.M / BM_FC2) * (H / BN) * a.splitk_f)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, a.splitk_f);
-    hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout);
+    hipLaunchKernelGGL(k_fc1<MODE>, dim3(grid_for((a.M / BM_QKV) * (F / BN))), dim3(256), GEMM_LDS, st, a, l);
+    if constexpr (MODE == 2) {
+      hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * (H / BigOut::kBN))), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, w.b_fc2, a.y1);
+      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, w.ln2_g, w.ln2_b, yout);
+    } else {
+      hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_FC2) * (H / BN) * a.splitk_f)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, a.splitk_f);
+      hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout);
+    }
     xin = yout;
   }
   SOUFFLE_HIP_TRY(hipGetLastError());
@@ -1338,7 +1504,7 @@ static int run_unfused(const souffle_bert_cfg *c, const souffle_bert_layer_w *la
   static thread_local Args a;
   if (int rc = fill_args(a, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return p.large ? run_unfused_t<true>(a, nl, df.num_cus, st) : run_unfused_t<false>(a, nl, df.num_cus, st);
+  return p.big ? run_unfused_t<2>(a, nl, df.num_cus, st) : p.large ? run_unfused_t<1>(a, nl, df.num_cus, st) : run_unfused_t<0>(a, nl, df.num_cus, st);
 }
 
 }  // namespace bert

@@ -18,6 +18,16 @@ typedef unsigned u4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
 
+// The thread id as a value the optimiser cannot see through.  Inside a persistent kernel that
+// loops over layers and stages, every address computed from the plain thread id is loop-invariant
+// and gets hoisted to the top of the kernel, where dozens of such values stay live across the
+// register-hungry GEMM loops and are spilled there.  Stages take their thread id from here.
+__device__ __forceinline__ int opaque_thread_id() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
+
 // ---------------------------------------------------------------- MFMA ----
 // v_mfma_f32_16x16x32_f16: D[i][j] += sum_k A[i][k] B[k][j]
 //   A: lane l holds row i = l%16, k = 8*(l/16) .. +7
@@ -25,6 +35,25 @@ constexpr int kWave = 64;
 //   D: lane l holds col j = l%16, rows i = 4*(l/16) + v, v = 0..3
 __device__ __forceinline__ f4 mfma_16x16x32(h8 a, h8 b, f4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+// The same instruction with the accumulator tied to AGPRs and updated in place.  With many live
+// accumulators the register allocator otherwise gives the three-address form different
+// source and destination registers and copies dozens of accumulators per loop iteration.
+// The compiler does not see inside, so the wait states that its hazard recognizer would insert
+// between a VALU write of an accumulator and the first MFMA, and between the last MFMA and a
+// VALU read, are supplied by hand: mfma_pin() after the accumulators are initialised and again
+// before they are read.  All of these are volatile, so they keep their program order.
+__device__ __forceinline__ void mfma_16x16x32_inplace(f4 &c, h8 a, h8 b) {
+  asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+// `n` accumulators exist in AGPRs here (not rematerialised later, not read earlier), with
+// 32 wait states in between.
+template <int N>
+__device__ __forceinline__ void mfma_pin(f4 (&acc)[N], bool before) {
+  if (!before) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+a"(acc[i]));
+  if (before) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 }
 // v_mfma_f32_16x16x16_f16: same layouts with k = 4*(l/16) .. +3
 __device__ __forceinline__ f4 mfma_16x16x16(h4 a, h4 b, f4 c) {
@@ -40,6 +69,16 @@ __device__ __forceinline__ h4 lds_read_tr16(const half_t *p) {
   typedef __attribute__((address_space(3))) s4 lds_s4;
   const s4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4 *)(__attribute__((address_space(3))) void *)const_cast<half_t *>(p));
   return __builtin_bit_cast(h4, r);
+}
+
+// LDS accesses through an explicit address-space cast: they stay DS instructions also where the
+// compiler cannot infer that a generic pointer points into LDS (inside functions that are not
+// inlined), instead of becoming flat accesses that count on both memory counters.
+__device__ __forceinline__ u4 lds_load16(const unsigned char *p) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) u4 *>((const __attribute__((address_space(3))) unsigned char *)p);
+}
+__device__ __forceinline__ void lds_store8(unsigned char *p, u2 v) {
+  *reinterpret_cast<__attribute__((address_space(3))) u2 *>((__attribute__((address_space(3))) unsigned char *)p) = v;
 }
 
 // ------------------------------------------- agent-coherent global access ----

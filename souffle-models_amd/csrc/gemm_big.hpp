@@ -1,0 +1,238 @@
+// fp16 MFMA GEMM tile for many rows (the MFMA-bound shapes) on gfx950.
+//
+// A workgroup of 256 threads computes a 256 x BN tile of Y = X.W, wave w owning rows
+// [64w, 64w+64) and all BN columns (4 x BN/16 accumulator tiles).  K advances in steps of 32
+// through a ring of NSTAGE LDS stages that are filled by direct global->LDS loads (no register
+// staging) NSTAGE-1 steps ahead, with ONE workgroup barrier per step: with a single wave per
+// SIMD nothing else hides the latency of the operand stream.
+//
+// LDS layouts (16-byte slots; a direct load writes 64 consecutive slots, which global 16 bytes
+// each lane fetches is free, so swizzles cost nothing):
+//   X stage [256 rows][32 k]: slot(r, s) = 4r + (s ^ ((r >> 1) & 3)); an operand read of 16 rows is
+//            one contiguous KB and its 8-lane groups cover all 32 banks;
+//   W stage [32 k][BN]:       slot(k, c) = k*BN/8 + (c ^ swz(k)); the four rows a 16-lane group of
+//            the transposing read touches must fall into different banks: their distance is
+//            BN/2 banks, i.e. 8 (BN = 144), 24 (BN = 48) - fine as they are - or 0 (BN = 192),
+//            where swz(k) = 2(k & 3) moves them apart.
+// W is row-major [K][N] as the reference stores it (cpp/bert/kernels/gemm_three_stages.h:95-131);
+// the MFMA takes W as operand A and X as operand B, so a lane ends up with 4 consecutive output
+// columns of one row.
+#pragma once
+#include <type_traits>
+#include "common.hpp"
+
+namespace souffle {
+
+// f(std::integral_constant<int, I>{}) for I = B .. E-1, in order: a loop whose index is a constant
+// expression in the body.
+template <int B, int E, class Fn>
+__device__ __forceinline__ void static_for(Fn f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
+template <int BN, int NSTAGE>
+struct GemmBig {
+  static_assert(BN % 16 == 0 && (BN * 64) % 1024 == 0, "whole MFMA tiles and whole wave-wide loads");
+  static constexpr int kBM = 256, kBN = BN, kBK = 32;
+  static constexpr int NT = BN / 16;                        // accumulator tiles per row block
+  static constexpr int WSLOTS = BN / 8;                     // 16-byte slots per W row
+  static constexpr int X_STAGE = 256 * 32 * 2, W_STAGE = 32 * BN * 2, STAGE = X_STAGE + W_STAGE;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE;
+  static constexpr int EPITCH = BN * 2 + 16;                // bytes per row of a wave's epilogue slice
+  static_assert(4 * 64 * EPITCH <= LDS_BYTES, "the epilogue slices fit in the ring");
+  static constexpr int XI = X_STAGE / 1024, WI = W_STAGE / 1024;   // wave-wide loads per stage
+  // Every wave issues LPW loads per stage: 4 of X and WPW of W.  Where WI is not a multiple of 4
+  // some waves fetch a chunk a second time (same bytes to the same place): the loop stays free of
+  // wave-dependent branches and every wave can use the same vmcnt.
+  static constexpr int WPW = (WI + 3) / 4, LPW = XI / 4 + WPW;
+  static_assert(XI == 16, "256 rows x 32 k");
+  static_assert(NSTAGE >= 4 && NSTAGE <= 6, "ring depth");
+  static_assert((NSTAGE - 2) * LPW < 64, "vmcnt is a 6-bit counter");
+
+  typedef __attribute__((address_space(1))) const void *gptr_t;
+  typedef __attribute__((address_space(3))) void *lptr_t;
+
+  __device__ static __forceinline__ int wswz(int k) { return BN == 192 ? ((k & 3) << 1) : 0; }
+
+  // One wave-wide direct load: lane L's 16 bytes at `src` land at LDS byte address lds_addr + 16 L.
+  // Issued through inline assembly on purpose: for the builtin the compiler tracks the LDS write
+  // and makes every later LDS read wait for ALL outstanding loads (vmcnt 0), which would
+  // serialise the ring; here the waits are the explicit ones in run().
+  __device__ static __forceinline__ void load_lds16(const void *src, unsigned lds_addr) {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src) : "memory", "m0");
+#pragma clang diagnostic pop
+  }
+  __device__ static __forceinline__ unsigned lds_address(const unsigned char *p) {
+    return (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char *)p;
+  }
+
+  // Load number L (0 .. LPW-1) of this wave for the stage at LDS address `stage`, K offset kk.
+  // wptr(k, col) -> address of W[k][col] (col relative to the tile's first column, multiple of 8)
+  template <int L, class WPtr>
+  __device__ static __forceinline__ void issue_one(int tid, unsigned stage, const half_t *X, int ldx, int m0, int kk, WPtr wptr) {
+    const int lane = tid & 63, wave = tid >> 6;
+    if constexpr (L < 4) {
+      const int q = wave + 4 * L, r = q * 16 + (lane >> 2), sl = (lane & 3) ^ ((r >> 1) & 3);
+      load_lds16(X + (size_t)(m0 + r) * ldx + kk + sl * 8, stage + q * 1024);
+    } else {
+      const int q = (wave + 4 * (L - 4)) % WI, sl = q * 64 + lane, k = sl / WSLOTS, c = (sl % WSLOTS) ^ wswz(k);
+      load_lds16(wptr(kk + k, c * 8), stage + X_STAGE + q * 1024);
+    }
+  }
+  template <int L0, int L1, class WPtr>
+  __device__ static __forceinline__ void issue_range(int tid, unsigned stage, const half_t *X, int ldx, int m0, int kk, WPtr wptr) {
+    if constexpr (L0 < L1) {
+      issue_one<L0>(tid, stage, X, ldx, m0, kk, wptr);
+      issue_range<L0 + 1, L1>(tid, stage, X, ldx, m0, kk, wptr);
+    }
+  }
+
+  // All but the loads of the A most recent stages of this wave have landed.
+  template <int A>
+  __device__ static __forceinline__ void wait_ahead() {
+    static_assert(A >= 0 && A * LPW < 64, "vmcnt is a 6-bit counter");
+    wait_vmcnt<A * LPW>();
+  }
+
+  // LDS read look-ahead, in column tiles: the transposing reads of tile f + D are issued before the
+  // MFMAs of tile f (f counts tiles across steps).  D + 1 divides NT, so the rotating operand
+  // registers are used identically in every step.
+  static constexpr int D = NT % 4 == 0 ? 3 : 2;
+  static_assert(NT % (D + 1) == 0, "operand register rotation");
+  static constexpr int JB = NT / 2 < NT - D ? NT / 2 : NT - D;   // tile before which the step's barrier sits
+
+  // Y[m0 .. m0+256)[tile columns] over nkt K steps starting at column k0 of X;
+  // cvt(m, n, v) -> u2: the four fp16 results for v[i] = (X.W)[m][n + i] (bias, activation, residual
+  // are the caller's); store16(m, n, u4): 8 consecutive results of row m from column n on; n is
+  // relative to the tile's first column.
+  //
+  // Step kt multiplies stage kt tile by tile.  Before tile JB it waits for stage kt+1 and passes
+  // the workgroup barrier (everybody is then done with stage kt-1); the reads that run ahead into
+  // stage kt+1 (its X operand and first D weight tiles) come after the barrier.  The loads that
+  // refill the freed buffer with stage kt+NSTAGE-1 are spread over the NT tiles that follow the
+  // barrier (into the next step), a load or two per tile: a load takes the vector memory
+  // pipeline of the CU 30 cycles or more and stalls the wave meanwhile, which the four MFMAs
+  // issued just before it cover.  (Issued as one burst after the barrier, the loads of the four
+  // waves queue up behind each other and every SIMD idles: measured 2x the time per step.)
+  template <class WPtr, class Cvt, class Store16>
+  __device__ static __forceinline__ void run(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, int nkt, WPtr wptr, Cvt cvt, Store16 store16) {
+    const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+    f4 acc[4][NT];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) mfma_pin(acc[i], true);
+
+    __syncthreads();                                        // the previous user of the ring is done
+    const unsigned ring = lds_address(lds);
+#pragma unroll
+    for (int s = 0; s < NSTAGE - 1; ++s) issue_range<0, LPW>(tid, ring + s * STAGE, X, ldx, m0, k0 + s * 32, wptr);
+
+    // byte offsets of this lane's operand reads inside a stage
+    int xoff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = wave * 64 + i * 16 + l16;
+      xoff[i] = r * 64 + ((g ^ ((r >> 1) & 3)) << 4);
+    }
+    const int kr = g * 8 + (l16 >> 2);                       // first of this lane's two k rows (kr, kr + 4)
+    const int wrow = X_STAGE + kr * (BN * 2) + (l16 & 1) * 8, wsw = wswz(kr), wc = (l16 & 3) >> 1;
+
+    auto read_w = [&](const unsigned char *st, int j) {
+      const half_t *p = reinterpret_cast<const half_t *>(st + wrow + (((j * 2 + wc) ^ wsw) << 4));
+      const h4 lo = lds_read_tr16(p), hh = lds_read_tr16(p + 4 * BN);
+      return h8{lo[0], lo[1], lo[2], lo[3], hh[0], hh[1], hh[2], hh[3]};
+    };
+
+    h8 x[4], xn[4], w[D + 1];
+    wait_ahead<NSTAGE - 2>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 4; ++i) x[i] = as_h8(lds_load16(lds + xoff[i]));
+#pragma unroll
+    for (int j = 0; j < D; ++j) w[j] = read_w(lds, j);
+
+    // One K step.  LOAD_A: the tiles before the barrier issue the rest of stage kt+NSTAGE-2;
+    // LOAD_B: the tiles from the barrier on issue the first part of stage kt+NSTAGE-1;
+    // AHEAD: stages requested after stage kt+1 at the time of the wait.  All compile-time so that
+    // the body has no branches.
+    auto step = [&](int kt, auto load_a, auto load_b, auto ahead_c) {
+      constexpr bool LOAD_A = decltype(load_a)::value, LOAD_B = decltype(load_b)::value;
+      constexpr int AHEAD = decltype(ahead_c)::value;
+      const unsigned char *st = lds + (kt % NSTAGE) * STAGE, *stn = lds + ((kt + 1) % NSTAGE) * STAGE;
+      const unsigned ring_a = ring + ((kt + NSTAGE - 2) % NSTAGE) * STAGE, ring_b = ring + ((kt + NSTAGE - 1) % NSTAGE) * STAGE;
+      const int kk_a = k0 + (kt + NSTAGE - 2) * 32, kk_b = kk_a + 32;
+      static_for<0, NT>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        if constexpr (j == JB) {
+          // stage kt+1 has landed for everybody and everybody has left stage kt-1 (a plain s_barrier:
+          // no fence, the loads in flight must stay in flight)
+          wait_ahead<AHEAD>();
+          __builtin_amdgcn_s_barrier();
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int i = 0; i < 4; ++i) xn[i] = as_h8(lds_load16(stn + xoff[i]));
+        }
+        // (in the last step these read a stale buffer; the values are never used)
+        w[(j + D) % (D + 1)] = j + D < NT ? read_w(st, j + D) : read_w(stn, j + D - NT);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          mfma_16x16x32_inplace(acc[i][j], w[j % (D + 1)], x[i]);
+        }
+        // this tile's share of the refill: slot t counts tiles from the barrier
+        constexpr int t = (j - JB + NT) % NT, L0 = t * LPW / NT, L1 = (t + 1) * LPW / NT;
+        if constexpr (j >= JB) {
+          if constexpr (LOAD_B) issue_range<L0, L1>(tid, ring_b, X, ldx, m0, kk_b, wptr);
+        } else {
+          if constexpr (LOAD_A) issue_range<L0, L1>(tid, ring_a, X, ldx, m0, kk_a, wptr);
+        }
+      });
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = xn[i];
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    // nkt >= NSTAGE (the callers' shapes: K >= 192).  Stages 0 .. NSTAGE-2 were requested above.
+    const int main_end = nkt - (NSTAGE - 1);               // steps 1 .. main_end-1 request on both sides of the barrier
+    step(0, F{}, T{}, std::integral_constant<int, NSTAGE - 3>{});
+    for (int kt = 1; kt < main_end; ++kt) step(kt, T{}, T{}, std::integral_constant<int, NSTAGE - 3>{});
+    // the last NSTAGE-1 steps: the first still completes stage nkt-1; after stage kt+1 there are
+    // NSTAGE-3, ..., 1, 0, 0 stages in flight
+    step(main_end + 0, T{}, F{}, std::integral_constant<int, (NSTAGE - 3 > 0 ? NSTAGE - 3 : 0)>{});
+    step(main_end + 1, F{}, F{}, std::integral_constant<int, (NSTAGE - 4 > 0 ? NSTAGE - 4 : 0)>{});
+    step(main_end + 2, F{}, F{}, std::integral_constant<int, (NSTAGE - 5 > 0 ? NSTAGE - 5 : 0)>{});
+    if constexpr (NSTAGE >= 5) step(main_end + 3, F{}, F{}, std::integral_constant<int, (NSTAGE - 6 > 0 ? NSTAGE - 6 : 0)>{});
+    if constexpr (NSTAGE >= 6) step(main_end + 4, F{}, F{}, std::integral_constant<int, 0>{});
+#pragma unroll
+    for (int i = 0; i < 4; ++i) mfma_pin(acc[i], false);
+
+    // Epilogue.  A lane holds 4 consecutive columns of 16 rows per accumulator tile; stored
+    // directly that would be 8-byte pieces of 32-byte row segments.  The converted tile instead
+    // goes through the wave's own slice of the (now idle) ring, and leaves as 16 bytes per lane
+    // along whole rows.
+    __syncthreads();                                        // every wave has left the ring
+    unsigned char *mine = lds + wave * (64 * EPITCH);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        lds_store8(mine + (i * 16 + l16) * EPITCH + (j * 16 + g * 4) * 2, cvt(m0 + wave * 64 + i * 16 + l16, j * 16 + g * 4, acc[i][j]));
+    constexpr int CPR = BN / 8;                              // 16-byte chunks per row
+#pragma unroll
+    for (int t = 0; t < CPR; ++t) {                          // 64 rows x CPR chunks = CPR per lane
+      const int c = t * 64 + lane, row = c / CPR, col8 = c % CPR;
+      const u4 v = lds_load16(mine + row * EPITCH + col8 * 16);
+      store16(m0 + wave * 64 + row, col8 * 8, v);
+    }
+  }
+};
+
+}  // namespace souffle
