@@ -81,6 +81,21 @@ __device__ __forceinline__ void lds_store8(unsigned char *p, u2 v) {
   *reinterpret_cast<__attribute__((address_space(3))) u2 *>((__attribute__((address_space(3))) unsigned char *)p) = v;
 }
 
+// One wave-wide direct global->LDS load: lane L's 16 bytes at `src` land at LDS byte address
+// lds_addr + 16 L.  Issued through inline assembly on purpose: for the builtin the compiler
+// tracks the LDS write and makes every later LDS read wait for ALL outstanding loads (vmcnt 0),
+// which serialises any scheme that keeps loads in flight across LDS reads; with this form the
+// waits are the explicit wait_vmcnt<N>() of the caller.
+__device__ __forceinline__ void load_lds16(const void *src, unsigned lds_addr) {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src) : "memory", "m0");
+#pragma clang diagnostic pop
+}
+__device__ __forceinline__ unsigned lds_address(const unsigned char *p) {
+  return (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char *)p;
+}
+
 // ------------------------------------------- agent-coherent global access ----
 // Data handed from one workgroup to another inside a persistent kernel is written
 // through (sc1) and read with sc1 so that it is coherent across the eight XCD L2s
@@ -160,9 +175,9 @@ __device__ __forceinline__ float wave_max(float v) {
 // 0.5 x (1 + tanh(0.79788456 (x + 0.044715 x^3)))  (cpp/bert/bert_base_impl.cu:722-734)
 __device__ __forceinline__ float gelu_tanh(float x) {
   const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  // tanh(u) = 1 - 2 / (exp(2u) + 1); exp overflow gives the correct limit 1.
-  const float t = 1.0f - 2.0f / (__expf(2.0f * u) + 1.0f);
-  return 0.5f * x * (1.0f + t);
+  // 0.5 (1 + tanh(u)) = 1 - 1 / (exp(2u) + 1); exp overflow gives the correct limit 1.  The
+  // hardware reciprocal (1 ulp) replaces the IEEE division, which costs some 10 instructions.
+  return x * (1.0f - __builtin_amdgcn_rcpf(__expf(2.0f * u) + 1.0f));
 }
 
 // -------------------------------------------------------- grid barrier ----

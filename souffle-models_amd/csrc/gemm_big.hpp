@@ -57,20 +57,6 @@ struct GemmBig {
 
   __device__ static __forceinline__ int wswz(int k) { return BN == 192 ? ((k & 3) << 1) : 0; }
 
-  // One wave-wide direct load: lane L's 16 bytes at `src` land at LDS byte address lds_addr + 16 L.
-  // Issued through inline assembly on purpose: for the builtin the compiler tracks the LDS write
-  // and makes every later LDS read wait for ALL outstanding loads (vmcnt 0), which would
-  // serialise the ring; here the waits are the explicit ones in run().
-  __device__ static __forceinline__ void load_lds16(const void *src, unsigned lds_addr) {
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src) : "memory", "m0");
-#pragma clang diagnostic pop
-  }
-  __device__ static __forceinline__ unsigned lds_address(const unsigned char *p) {
-    return (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char *)p;
-  }
-
   // Load number L (0 .. LPW-1) of this wave for the stage at LDS address `stage`, K offset kk.
   // wptr(k, col) -> address of W[k][col] (col relative to the tile's first column, multiple of 8)
   template <int L, class WPtr>

@@ -32,65 +32,186 @@ struct Args {
   const half_t *x;
   half_t *mid, *y;
   unsigned *ctl;
+  unsigned long long *trace;   // optional phase stamps: trace[block * 32 + phase] (development aid)
   BlockW w[2];
 };
 
+// Weights reach the CU as a stream of 24 chunks per block, each W[128 k][64 n] (16 KB): 6 of
+// QKV, 2 of proj, 8 of FC1, 8 of FC2 (2 column blocks x 4 K blocks).  The stream does not
+// depend on any activation, so it runs two chunks ahead of the MFMAs through a ring of three
+// LDS buffers filled by direct global->LDS loads, across the LayerNorm / attention phases and
+// across the hand-over to the next block: the GEMM phases never wait for a weight load that was
+// issued less than a chunk's worth of work earlier.
+constexpr int CHUNK_K = 128, CHUNK_N = 64, CHUNK_BYTES = CHUNK_K * CHUNK_N * 2, RING = 3, CHUNKS = 24;
+constexpr int CHUNK_LOADS = CHUNK_BYTES / 1024 / 4;      // wave-wide loads per wave per chunk
+
 // LDS carve-up (bytes)
-constexpr int OFF_GEMM = 0;
-constexpr int OFF_ZS = OFF_GEMM + Tile::LDS_BYTES;
+constexpr int OFF_RING = 0;
+constexpr int OFF_ZS = OFF_RING + RING * CHUNK_BYTES;
 constexpr int OFF_BIG = OFF_ZS + NP * ZLD * 2;
 constexpr int OFF_X1 = OFF_BIG + NP * BLD * 2;
 constexpr int OFF_TAB = OFF_X1 + NP * ZLD * 2;
 constexpr int OFF_TOK = OFF_TAB + TAB * NH * 4;
 constexpr int OFF_REG = OFF_TOK + NP * 4;
-constexpr int LDS_BYTES = OFF_REG + NP * 4;
+// biases and LayerNorm vectors of the block, copied once per call (halves): reading them from
+// global memory inside the GEMM phases would make the compiler wait for ALL outstanding vector
+// memory operations - the prefetched weight chunks included - at every use
+constexpr int P_BQKV = 0, P_BPROJ = P_BQKV + 3 * C, P_BFC1 = P_BPROJ + C, P_BFC2 = P_BFC1 + F, P_G1 = P_BFC2 + C,
+              P_B1 = P_G1 + C, P_G2 = P_B1 + C, P_B2 = P_G2 + C, P_HALVES = P_B2 + C;
+constexpr int OFF_PAR = OFF_REG + NP * 4;
+constexpr int LDS_BYTES = OFF_PAR + P_HALVES * 2;
+static_assert(LDS_BYTES <= 160 * 1024, "one workgroup per CU");
+
+struct Chunk {
+  const half_t *W;
+  int ldw, k0, n0;
+};
+__device__ __forceinline__ Chunk chunk_of(const BlockW &w, int c) {
+  if (c < 6) return Chunk{w.w_qkv, 3 * C, 0, c * CHUNK_N};
+  if (c < 8) return Chunk{w.w_proj, C, 0, (c - 6) * CHUNK_N};
+  if (c < 16) return Chunk{w.w_fc1, F, 0, (c - 8) * CHUNK_N};
+  return Chunk{w.w_fc2, C, ((c - 16) & 3) * CHUNK_K, ((c - 16) >> 2) * CHUNK_N};
+}
+
+// The weight stream of one workgroup.  `issued` / `used` count chunks over the whole launch.
+struct WeightRing {
+  unsigned char *lds;
+  unsigned lds_addr;
+  int issued, used;
+};
+// Queue chunk c of block weights w into the next ring buffer.  Layout as GemmOneShot's W slice:
+// slot(k, c8) = 8 k + (c8 ^ (k & 2)), for the transposing operand read.
+__device__ __forceinline__ void ring_issue(WeightRing &r, const BlockW &w, int c) {
+  const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6;
+  const Chunk ch = chunk_of(w, c);
+  const unsigned base = r.lds_addr + (r.issued % RING) * CHUNK_BYTES;
+#pragma unroll
+  for (int q = 0; q < CHUNK_LOADS; ++q) {
+    const int inst = q * 4 + wave, sl = inst * 64 + lane, k = sl >> 3, c8 = (sl & 7) ^ (k & 2);
+    load_lds16(ch.W + (size_t)(ch.k0 + k) * ch.ldw + ch.n0 + c8 * 8, base + inst * 1024);
+  }
+  r.issued++;
+}
+// Wait for the oldest unused chunk and hand out its buffer.  `more`: chunks issued after it
+// (0..2).  After the barrier everybody has finished with the chunk before it, whose buffer the
+// caller may refill.  Other vector memory operations issued in between only make the wait stricter.
+__device__ __forceinline__ const unsigned char *ring_take(WeightRing &r) {
+  const int more = r.issued - r.used - 1;
+  if (more >= 2) wait_vmcnt<2 * CHUNK_LOADS>();
+  else if (more == 1) wait_vmcnt<CHUNK_LOADS>();
+  else wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  const unsigned char *buf = r.lds + (r.used % RING) * CHUNK_BYTES;
+  r.used++;
+  return buf;
+}
+// acc[j] (rows 16 wave .. +15, columns 16 j .. +15 of the chunk) += A[rows][ka .. ka+128) . chunk.
+// All 36 operand reads are issued before the first MFMA: with a read-then-multiply order the
+// compiler waits for each pair of reads in turn and the chunk costs 16 LDS latencies.
+__device__ __forceinline__ void chunk_mma(const unsigned char *buf, const half_t *A, int lda, int ka, f4 (&acc)[4]) {
+  const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+  const half_t *ws = reinterpret_cast<const half_t *>(buf);
+  h8 xop[CHUNK_K / 32], wop[CHUNK_K / 32][4];
+#pragma unroll
+  for (int ks = 0; ks < CHUNK_K / 32; ++ks) {
+    xop[ks] = *reinterpret_cast<const h8 *>(A + (wave * 16 + l16) * lda + ka + ks * 32 + g * 8);
+    const int k = ks * 32 + g * 8 + (l16 >> 2);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c8 = j * 2 + ((l16 & 3) >> 1);
+      const half_t *p = ws + (k * 8 + (c8 ^ (k & 2))) * 8 + (l16 & 1) * 4;
+      const h4 lo = lds_read_tr16(p), hi = lds_read_tr16(p + 4 * CHUNK_N);
+      wop[ks][j] = h8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+  }
+#pragma unroll
+  for (int ks = 0; ks < CHUNK_K / 32; ++ks)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = mfma_16x16x32(wop[ks][j], xop[ks], acc[j]);
+}
 
 __device__ __forceinline__ int region_of(int i, int n, int shift) {   // slices [0,n-7), [n-7,n-shift), [n-shift,n)
   return i < n - WS ? 0 : (i < n - shift ? 1 : 2);
 }
 
-// rows [16*wave, 16*wave+16) of a [64][C] fp16 source -> LayerNorm -> dst (LDS, ld ZLD)
-template <class RowLoad>
-__device__ __forceinline__ void layernorm_rows(RowLoad load2, half_t *dst, const half_t *gam, const half_t *bet, float eps) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float g0 = 1.f, g1 = 1.f, b0 = 0.f, b1 = 0.f;
-  if (gam) { const h2 t = *reinterpret_cast<const h2 *>(gam + 2 * lane); g0 = (float)t[0]; g1 = (float)t[1]; }
-  if (bet) { const h2 t = *reinterpret_cast<const h2 *>(bet + 2 * lane); b0 = (float)t[0]; b1 = (float)t[1]; }
-  for (int r = wave * 16; r < wave * 16 + 16; ++r) {
-    h2 o = {(half_t)0.f, (half_t)0.f};
+// LayerNorm of the 64 rows of a [64][C] fp16 source into dst (LDS, ld ZLD): four lanes share a row
+// (32 columns each), so all rows are normalised at once; rows >= N become zero.
+// load8(r, c) -> the 8 halves [r][c .. c+7]; gam and bet are in LDS.
+template <class Load8>
+__device__ __forceinline__ void layernorm_rows(Load8 load8, half_t *dst, const half_t *gam, const half_t *bet, float eps) {
+  const int tid = opaque_thread_id(), r = tid >> 2, c0 = (tid & 3) * 32;
+  h8 x[4];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    x[i] = r < N ? as_h8(load8(r, c0 + 8 * i)) : h8{};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum += (float)x[i][e];
+  }
+  sum += wave_xor(sum, 1);
+  sum += wave_xor(sum, 2);
+  const float mean = sum * (1.0f / C);
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { const float d = (float)x[i][e] - mean; sq += d * d; }
+  sq += wave_xor(sq, 1);
+  sq += wave_xor(sq, 2);
+  const float rstd = rsqrtf(sq * (1.0f / C) + eps);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    h8 o = {};
     if (r < N) {
-      const h2 v = load2(r, 2 * lane);
-      const float a = (float)v[0], b = (float)v[1];
-      const float mean = wave_sum(a + b) * (1.0f / C);
-      const float da = a - mean, db = b - mean;
-      const float rstd = rsqrtf(wave_sum(da * da + db * db) * (1.0f / C) + eps);
-      o = h2{(half_t)(da * rstd * g0 + b0), (half_t)(db * rstd * g1 + b1)};
+      const h8 g8 = *reinterpret_cast<const h8 *>(gam + c0 + 8 * i), b8 = *reinterpret_cast<const h8 *>(bet + c0 + 8 * i);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (half_t)(((float)x[i][e] - mean) * rstd * (float)g8[e] + (float)b8[e]);
     }
-    *reinterpret_cast<h2 *>(dst + r * ZLD + 2 * lane) = o;
+    *reinterpret_cast<h8 *>(dst + r * ZLD + c0 + 8 * i) = o;
   }
 }
 
-__device__ __forceinline__ f4 add_bias4(f4 v, const half_t *bias, int n) {
-  if (bias) {
-    const h4 bb = *reinterpret_cast<const h4 *>(bias + n);
-    v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
-  }
-  return v;
+__device__ __forceinline__ f4 add_bias4(f4 v, const half_t *bias_lds, int n) {
+  const h4 bb = *reinterpret_cast<const h4 *>(bias_lds + n);
+  return v + f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
 }
 
-__device__ void block_for_window(unsigned char *lds, const Args &a, const BlockW &w, int shift, const half_t *xin,
-                                 half_t *xout, int win) {
-  half_t *gemm_lds = reinterpret_cast<half_t *>(lds + OFF_GEMM);
+// One block for one window.  `next`: the weights whose first chunks are queued before this call
+// returns (the next call of this workgroup), or NULL.
+__device__ void block_for_window(unsigned char *lds, WeightRing &ring, const Args &a, const BlockW &w, const BlockW *next,
+                                 int shift, const half_t *xin, half_t *xout, int win) {
   half_t *zs = reinterpret_cast<half_t *>(lds + OFF_ZS);
   half_t *big = reinterpret_cast<half_t *>(lds + OFF_BIG);
   half_t *x1s = reinterpret_cast<half_t *>(lds + OFF_X1);
   float *tab = reinterpret_cast<float *>(lds + OFF_TAB);
   int *tok = reinterpret_cast<int *>(lds + OFF_TOK);
   int *reg = reinterpret_cast<int *>(lds + OFF_REG);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+  half_t *par = reinterpret_cast<half_t *>(lds + OFF_PAR);
+  const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
   const int nww = a.Ww / WS;
+  const int first_chunk = ring.used;                        // chunk c of this call is ring chunk first_chunk + c
+  // keep the stream two chunks ahead: chunk c+2 of this call, or the first chunks of the next
+  auto top_up = [&]() {
+    const int c = ring.issued - first_chunk;
+    if (c < CHUNKS) ring_issue(ring, w, c);
+    else if (next && c < CHUNKS + 2) ring_issue(ring, *next, c - CHUNKS);
+  };
+  // one output column block of a GEMM whose K is one chunk: acc = A[64][128] . chunk
+  auto gemm_chunk = [&](const half_t *A, int lda, f4 (&acc)[4]) {
+    const unsigned char *buf = ring_take(ring);
+    top_up();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = f4{0.f, 0.f, 0.f, 0.f};
+    chunk_mma(buf, A, lda, 0, acc);
+  };
+  const int row = wave * 16 + l16;                          // the row this lane holds results of
+  int mark_id = shift > 0 ? 16 : 0;
+  auto mark = [&]() { if (a.trace && tid == 0 && win == (int)blockIdx.x) a.trace[blockIdx.x * 32 + mark_id] = wall_clock64(); ++mark_id; };
+  mark();
 
   __syncthreads();
+  while (ring.issued < first_chunk + 2) top_up();           // (already there when the previous call queued them)
   if (tid < NP) {
     int t = -1, rg = 0;
     if (tid < N) {
@@ -104,26 +225,42 @@ __device__ void block_for_window(unsigned char *lds, const Args &a, const BlockW
     reg[tid] = rg;
   }
   for (int i = tid; i < TAB * NH; i += 256) tab[i] = w.rel_table ? (float)w.rel_table[i] : 0.f;
-  __syncthreads();
-
-  // LN1 of the gathered rows
-  layernorm_rows([&](int r, int c) { return __builtin_bit_cast(h2, ld4<true>(xin, (tok[r] * C + c) * 2)); }, zs,
-                 w.ln1_g, w.ln1_b, a.eps);
-  __syncthreads();
-
-  // QKV = Z.Wqkv + b, q pre-scaled by hd^-0.5; kept in LDS as [64][3C]
-  const float qscale = rsqrtf((float)HD);
-  for (int nt = 0; nt < 3 * C / 64; ++nt) {
-    Tile::run(gemm_lds, w.w_qkv, 3 * C, 0, nt * 64, 0, C / 64,
-              [&](int m, int k) { return *reinterpret_cast<const u4 *>(zs + m * ZLD + k); },
-              [&](int m, int n, f4 v) {
-                v = add_bias4(v, w.b_qkv, n);
-                if (n < C) v *= qscale;
-                *reinterpret_cast<u2 *>(big + m * BLD + n) = pack_h4(v);
-              });
+  {
+    auto copy = [&](int off, const half_t *src, int n, float dflt) {
+      for (int i = tid; i < n; i += 256) par[off + i] = src ? src[i] : (half_t)dflt;
+    };
+    copy(P_BQKV, w.b_qkv, 3 * C, 0.f); copy(P_BPROJ, w.b_proj, C, 0.f); copy(P_BFC1, w.b_fc1, F, 0.f); copy(P_BFC2, w.b_fc2, C, 0.f);
+    copy(P_G1, w.ln1_g, C, 1.f); copy(P_B1, w.ln1_b, C, 0.f); copy(P_G2, w.ln2_g, C, 1.f); copy(P_B2, w.ln2_b, C, 0.f);
   }
   __syncthreads();
 
+  mark();
+  // LN1 of the gathered rows
+  // (the gathered rows are also kept, in x1s, as the shortcut of the projection)
+  layernorm_rows([&](int r, int c) {
+    const u4 v = ld16<true>(xin, (tok[r] * C + c) * 2);
+    *reinterpret_cast<u4 *>(x1s + r * ZLD + c) = v;
+    return v;
+  }, zs, par + P_G1, par + P_B1, a.eps);
+  __syncthreads();
+
+  mark();
+  // QKV = Z.Wqkv + b, q pre-scaled by hd^-0.5; kept in LDS as [64][3C]
+  const float qscale = rsqrtf((float)HD);
+  for (int nt = 0; nt < 3 * C / CHUNK_N; ++nt) {
+    f4 acc[4];
+    gemm_chunk(zs, ZLD, acc);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = nt * CHUNK_N + j * 16 + g * 4;
+      f4 v = add_bias4(acc[j], par + P_BQKV, n);
+      if (n < C) v *= qscale;
+      *reinterpret_cast<u2 *>(big + row * BLD + n) = pack_h4(v);
+    }
+  }
+  __syncthreads();
+
+  mark();
   // attention: wave = head
   {
     const int h = wave;
@@ -179,62 +316,97 @@ __device__ void block_for_window(unsigned char *lds, const Args &a, const BlockW
   }
   __syncthreads();
 
+  mark();
   // x1 = x + ctx.Wproj + b  (kept in LDS)
-  for (int nt = 0; nt < C / 64; ++nt) {
-    Tile::run(gemm_lds, w.w_proj, C, 0, nt * 64, 0, C / 64,
-              [&](int m, int k) { return *reinterpret_cast<const u4 *>(zs + m * ZLD + k); },
-              [&](int m, int n, f4 v) {
-                v = add_bias4(v, w.b_proj, n);
-                if (m < N) {
-                  const h4 sh = as_h4(ld8<true>(xin, (tok[m] * C + n) * 2));
-                  v += f4{(float)sh[0], (float)sh[1], (float)sh[2], (float)sh[3]};
-                } else {
-                  v = f4{0.f, 0.f, 0.f, 0.f};
-                }
-                *reinterpret_cast<u2 *>(x1s + m * ZLD + n) = pack_h4(v);
-              });
+  for (int nt = 0; nt < C / CHUNK_N; ++nt) {
+    f4 acc[4];
+    gemm_chunk(zs, ZLD, acc);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = nt * CHUNK_N + j * 16 + g * 4;
+      f4 v = f4{0.f, 0.f, 0.f, 0.f};
+      if (row < N) {
+        const h4 sh = *reinterpret_cast<const h4 *>(x1s + row * ZLD + n);
+        v = add_bias4(acc[j], par + P_BPROJ, n) + f4{(float)sh[0], (float)sh[1], (float)sh[2], (float)sh[3]};
+      }
+      *reinterpret_cast<u2 *>(x1s + row * ZLD + n) = pack_h4(v);
+    }
   }
   __syncthreads();
 
-  layernorm_rows([&](int r, int c) { return *reinterpret_cast<const h2 *>(x1s + r * ZLD + c); }, zs, w.ln2_g, w.ln2_b, a.eps);
+  mark();
+  layernorm_rows([&](int r, int c) { return *reinterpret_cast<const u4 *>(x1s + r * ZLD + c); }, zs, par + P_G2, par + P_B2, a.eps);
   __syncthreads();
+  mark();
 
   // H = gelu(Z2.W1 + b1) in LDS
-  for (int nt = 0; nt < F / 64; ++nt) {
-    Tile::run(gemm_lds, w.w_fc1, F, 0, nt * 64, 0, C / 64,
-              [&](int m, int k) { return *reinterpret_cast<const u4 *>(zs + m * ZLD + k); },
-              [&](int m, int n, f4 v) {
-                v = add_bias4(v, w.b_fc1, n);
+  for (int nt = 0; nt < F / CHUNK_N; ++nt) {
+    f4 acc[4];
+    gemm_chunk(zs, ZLD, acc);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v[i] = gelu_tanh(v[i]);
-                *reinterpret_cast<u2 *>(big + m * BLD + n) = pack_h4(v);
-              });
+    for (int j = 0; j < 4; ++j) {
+      const int n = nt * CHUNK_N + j * 16 + g * 4;
+      f4 v = add_bias4(acc[j], par + P_BFC1, n);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = gelu_tanh(v[i]);
+      *reinterpret_cast<u2 *>(big + row * BLD + n) = pack_h4(v);
+    }
   }
   __syncthreads();
 
-  // out = x1 + H.W2 + b2, scattered back to the token rows
-  for (int nt = 0; nt < C / 64; ++nt) {
-    Tile::run(gemm_lds, w.w_fc2, C, 0, nt * 64, 0, F / 64,
-              [&](int m, int k) { return *reinterpret_cast<const u4 *>(big + m * BLD + k); },
-              [&](int m, int n, f4 v) {
-                if (m < N) {
-                  v = add_bias4(v, w.b_fc2, n);
-                  const h4 r = *reinterpret_cast<const h4 *>(x1s + m * ZLD + n);
-                  v += f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
-                  st8<true>(xout, (tok[m] * C + n) * 2, pack_h4(v));
-                }
-              });
+  mark();
+  // out = x1 + H.W2 + b2, scattered back to the token rows; K = 512 is four chunks per column block
+  for (int nt = 0; nt < C / CHUNK_N; ++nt) {
+    f4 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = f4{0.f, 0.f, 0.f, 0.f};
+    for (int kc = 0; kc < F / CHUNK_K; ++kc) {
+      const unsigned char *buf = ring_take(ring);
+      top_up();
+      chunk_mma(buf, big, BLD, kc * CHUNK_K, acc);
+    }
+    if (row < N) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = nt * CHUNK_N + j * 16 + g * 4;
+        const h4 r = *reinterpret_cast<const h4 *>(x1s + row * ZLD + n);
+        const f4 v = add_bias4(acc[j], par + P_BFC2, n) + f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+        st8<true>(xout, (tok[row] * C + n) * 2, pack_h4(v));
+      }
+    }
   }
+  mark();
 }
 
 __global__ void __launch_bounds__(256) k_block_pair(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   GridBarrier bar;
   grid_barrier_begin(bar, a.ctl);
-  const int nwin = (a.Hh / WS) * (a.Ww / WS);
-  for (int win = blockIdx.x; win < nwin; win += gridDim.x) block_for_window(lds, a, a.w[0], 0, a.x, a.mid, win);
-  grid_sync(bar);
-  for (int win = blockIdx.x; win < nwin; win += gridDim.x) block_for_window(lds, a, a.w[1], a.shift, a.mid, a.y, win);
+  WeightRing ring{lds + OFF_RING, lds_address(lds + OFF_RING), 0, 0};
+  const int nwin = (a.Hh / WS) * (a.Ww / WS), step = gridDim.x;
+  if ((int)blockIdx.x >= nwin) {
+    // Fewer windows than CUs: the spare workgroups pull the weights of both blocks into the L2 of
+    // their XCD (workgroup b runs on XCD b % 8), so that the weight stream of the working
+    // workgroups hits there instead of paying the memory latency for every chunk.
+    const int xcd_slots = (step - nwin + 7) / 8, slot = ((int)blockIdx.x - nwin) / 8;
+    float sink = 0.f;
+    for (int b = 0; b < 2; ++b) {
+      const half_t *mats[4] = {a.w[b].w_qkv, a.w[b].w_proj, a.w[b].w_fc1, a.w[b].w_fc2};
+      const int halves[4] = {C * 3 * C, C * C, C * F, F * C};
+      for (int m = 0; m < 4; ++m)
+        for (int i = (slot * 256 + (int)threadIdx.x) * 8; i < halves[m]; i += xcd_slots * 256 * 8)
+          sink += __builtin_bit_cast(f4, *reinterpret_cast<const u4 *>(mats[m] + i))[0];
+    }
+    asm volatile("" ::"v"(sink));
+    grid_sync(bar);
+    grid_barrier_end(bar);
+    return;
+  }
+  for (int win = blockIdx.x; win < nwin; win += step)
+    block_for_window(lds, ring, a, a.w[0], win + step < nwin ? &a.w[0] : &a.w[1], 0, a.x, a.mid, win);
+  grid_sync(bar);                                           // (the first weight chunks of the second block are already on their way)
+  for (int win = blockIdx.x; win < nwin; win += step)
+    block_for_window(lds, ring, a, a.w[1], win + step < nwin ? &a.w[1] : nullptr, a.shift, a.mid, a.y, win);
   grid_barrier_end(bar);
 }
 
@@ -315,6 +487,11 @@ extern "C" int souffle_swin_block_pair_fused(const souffle_swin_cfg *cfg, const 
   a.x = static_cast<const half_t *>(x); a.y = static_cast<half_t *>(y);
   a.ctl = static_cast<unsigned *>(ws);
   a.mid = reinterpret_cast<half_t *>(static_cast<char *>(ws) + round_up(kCtlWords * 4, 256));
+  {
+    int cap = 0;
+    stage_trace(&a.trace, &cap, 256);
+    if (cap < 1) a.trace = nullptr;
+  }
   for (int b = 0; b < 2; ++b) {
     const souffle_swin_block_w &s = w[b];
     if (!s.w_qkv || !s.w_proj || !s.w_fc1 || !s.w_fc2) return fail(SOUFFLE_ERR_NULL, "block %d: a weight matrix is NULL", b);
@@ -334,7 +511,7 @@ extern "C" int souffle_swin_block_pair_fused(const souffle_swin_cfg *cfg, const 
   }
   const int nwin = (cfg->height / swin::WS) * (cfg->width / swin::WS);
   void *args[] = {&a};
-  return launch_persistent((const void *)swin::k_block_pair, std::min(nwin, df.num_cus), 256, args, swin::LDS_BYTES,
+  return launch_persistent((const void *)swin::k_block_pair, df.num_cus, 256, args, swin::LDS_BYTES,
                            static_cast<hipStream_t>(stream));
 }
 
