@@ -158,6 +158,22 @@ int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert
                                  const void *x, const void *mask, void *y,
                                  void *workspace, size_t workspace_bytes, souffle_stream_t stream);
 
+/* The stage in front of the encoder: out[b*S+s] = LayerNorm(word_emb[token_ids[b*S+s]] +
+ * pos_emb[s] + type_emb[segment_ids[b*S+s]]) in fp16, statistics in fp32.  Replaces the
+ * HuggingFace embedding module the reference feeds its layer with
+ * (cpp/bert/test_souffle_bert_layer.py:186-189; python/models/bert/relay_bert.py:12-13 starts
+ * from its [1,384,768] output).  token_ids / segment_ids: int32 device arrays [B*S]
+ * (segment_ids and type_emb may be NULL); tables fp16 [rows][768]; ids are not range-checked. */
+int souffle_bert_embed(const int32_t *token_ids, const int32_t *segment_ids,
+                       const void *word_emb, const void *pos_emb, const void *type_emb,
+                       const void *ln_g, const void *ln_b, float ln_eps,
+                       int batch, int seq_len, int hidden, void *out, souffle_stream_t stream);
+/* The stage behind the encoder: out[b] = tanh(x[b*S + 0] . W + bias), W fp16 [768][768] stored
+ * [K][N] like every weight here (transposition rule: cpp/bert/test_souffle_bert_layer.py:139-143);
+ * out fp16 [B][768].  The reference stops at the last encoder layer. */
+int souffle_bert_pooler(const void *x, const void *w, const void *bias,
+                        int batch, int seq_len, int hidden, void *out, souffle_stream_t stream);
+
 /* ------------------------------------------------------------------ LSTM ---- */
 enum { SOUFFLE_GATES_IFGO = 0, SOUFFLE_GATES_IGFO = 1 };
 typedef struct {

@@ -178,3 +178,32 @@ int oracle_bert_encoder_f32(const oracle_bert_cfg *c, const oracle_bert_weights 
   free(a); free(b);
   return rc;
 }
+
+/* Embedding stage in front of the encoder: word + position + token-type rows, then LayerNorm.
+ * The reference takes this from the HuggingFace module (cpp/bert/test_souffle_bert_layer.py:186-189);
+ * positions are 0..S-1 per sequence, token types default to 0. */
+int oracle_bert_embed_f32(const int32_t *token_ids, const int32_t *segment_ids, const float *word_emb,
+                          const float *pos_emb, const float *type_emb, const float *ln_g, const float *ln_b,
+                          float eps, int batch, int seq_len, int hidden, float *out) {
+  if (!token_ids || !word_emb || !pos_emb || !out || batch <= 0 || seq_len <= 0 || hidden <= 0) return -1;
+  float *row = (float *)malloc(sizeof(float) * (size_t)hidden);
+  if (!row) return -2;
+  for (int m = 0; m < batch * seq_len; ++m) {
+    const float *w = word_emb + (size_t)token_ids[m] * hidden, *p = pos_emb + (size_t)(m % seq_len) * hidden;
+    const float *t = type_emb ? type_emb + (size_t)(segment_ids ? segment_ids[m] : 0) * hidden : NULL;
+    for (int i = 0; i < hidden; ++i) row[i] = w[i] + p[i] + (t ? t[i] : 0.0f);
+    oracle_layernorm_f32(row, ln_g, ln_b, out + (size_t)m * hidden, 1, hidden, eps);
+  }
+  free(row);
+  return 0;
+}
+
+/* BERT pooler: tanh(x[b, 0, :] . W + bias), W stored [K][N]. */
+int oracle_bert_pooler_f32(const float *x, const float *w, const float *bias, int batch, int seq_len, int hidden, float *out) {
+  if (!x || !w || !out || batch <= 0 || seq_len <= 0 || hidden <= 0) return -1;
+  for (int b = 0; b < batch; ++b) {
+    oracle_gemm_f32(x + (size_t)b * seq_len * hidden, w, bias, out + (size_t)b * hidden, 1, hidden, hidden, 1);
+    for (int n = 0; n < hidden; ++n) out[(size_t)b * hidden + n] = tanhf(out[(size_t)b * hidden + n]);
+  }
+  return 0;
+}

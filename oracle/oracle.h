@@ -16,6 +16,9 @@
  *                              brute force on tiny grids, permutation laws
  *   oracle_swin_block_pair_f32 torch CPU library restatement of a Swin block
  *   oracle_se_module_f32       torch avg_pool2d / conv2d / sigmoid composition
+ *   oracle_bert_embed_f32      torch.nn.functional.embedding + layer_norm (float64)
+ *   oracle_bert_pooler_f32     torch matmul + tanh (float64), transposition rule of the
+ *                              reference (cpp/bert/test_souffle_bert_layer.py:139-143)
  * No function here is "parity unpinned".
  *
  * Layout rule used everywhere: a weight matrix is stored [K][N] with N
@@ -72,6 +75,13 @@ int oracle_bert_encoder_f32(const oracle_bert_cfg *cfg, const oracle_bert_weight
                             int num_threads);
 
 /* Single ops exposed for unit pinning. */
+/* Front / back of the encoder (cpp/bert/test_souffle_bert_layer.py:186-189; standard BERT pooler). */
+int oracle_bert_embed_f32(const int32_t *token_ids, const int32_t *segment_ids, const float *word_emb,
+                          const float *pos_emb, const float *type_emb, const float *ln_g, const float *ln_b,
+                          float eps, int batch, int seq_len, int hidden, float *out);
+int oracle_bert_pooler_f32(const float *x, const float *w, const float *bias, int batch, int seq_len, int hidden,
+                           float *out);
+
 void oracle_gemm_f32(const float *x, const float *w, const float *bias, float *y,
                      int M, int N, int K, int num_threads);
 void oracle_layernorm_f32(const float *z, const float *g, const float *b, float *y,

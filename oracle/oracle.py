@@ -143,6 +143,41 @@ def bert_encoder(x, layers, batch, seq_len, hidden=768, heads=12, ffn=3072, act=
     return y
 
 
+def bert_embed(token_ids, word_emb, pos_emb, type_emb=None, segment_ids=None, ln_g=None, ln_b=None, eps=1e-12):
+    """LayerNorm(word[token] + pos[position] + type[segment]); token_ids [B, S] -> [B*S, hidden] fp32."""
+    tok = np.ascontiguousarray(token_ids, dtype=np.int32)
+    B, S = tok.shape
+    seg = None if segment_ids is None else np.ascontiguousarray(segment_ids, dtype=np.int32)
+    w, p = _f32(word_emb), _f32(pos_emb)
+    t = None if type_emb is None else _f32(type_emb)
+    g = None if ln_g is None else _f32(ln_g)
+    b = None if ln_b is None else _f32(ln_b)
+    hidden = w.shape[1]
+    out = np.empty((B * S, hidden), np.float32)
+    ip = lambda a: None if a is None else a.ctypes.data_as(C.c_void_p)
+    fn = lib().oracle_bert_embed_f32
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_void_p] * 7 + [C.c_float, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    rc = fn(ip(tok), ip(seg), ip(w), ip(p), ip(t), ip(g), ip(b), float(eps), B, S, hidden, ip(out))
+    assert rc == 0, rc
+    return out
+
+
+def bert_pooler(x, w, bias, batch, seq_len):
+    """tanh(x[b, 0, :] . W + bias), W [K][N]; x [B*S, hidden] -> [B, hidden] fp32."""
+    xx, ww = _f32(x), _f32(w)
+    bb = None if bias is None else _f32(bias)
+    hidden = ww.shape[1]
+    out = np.empty((batch, hidden), np.float32)
+    ip = lambda a: None if a is None else a.ctypes.data_as(C.c_void_p)
+    fn = lib().oracle_bert_pooler_f32
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_void_p] * 3 + [C.c_int, C.c_int, C.c_int, C.c_void_p]
+    rc = fn(ip(xx), ip(ww), ip(bb), batch, seq_len, hidden, ip(out))
+    assert rc == 0, rc
+    return out
+
+
 def lstm(x, w_ih, w_hh, bias=None, gate_order="ifgo", forget_bias=0.0):
     """x [T,H] or [B,T,H]; w_* [L*4,H,H]; returns y with x's shape."""
     x = _f32(x)

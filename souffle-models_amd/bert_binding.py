@@ -142,3 +142,82 @@ class Encoder:
         sh.check(fn(C.byref(self.cfg), self.warr, x.data_ptr(), sh.ptr(mask), out.data_ptr(), self.ws.ptr,
                     self.ws.nbytes, sh.current_stream()))
         return out
+
+
+def embed(token_ids, word_emb, pos_emb, type_emb=None, segment_ids=None, ln_gamma=None, ln_beta=None, ln_eps=1e-12):
+    """The stage in front of the encoder: LayerNorm(word[token] + pos[position] + type[segment]).
+    Stands in for the HuggingFace embedding module the reference feeds its layer with
+    (cpp/bert/test_souffle_bert_layer.py:186-189).  token_ids: int32 CUDA tensor [B, S];
+    returns fp16 [B*S, 768]."""
+    if not isinstance(token_ids, torch.Tensor) or not token_ids.is_cuda or token_ids.dtype != torch.int32 or token_ids.dim() != 2:
+        raise TypeError("token_ids must be an int32 CUDA tensor [B, S]")
+    B, S = token_ids.shape
+    if segment_ids is not None and (segment_ids.dtype != torch.int32 or tuple(segment_ids.shape) != (B, S) or not segment_ids.is_cuda):
+        raise TypeError("segment_ids must be an int32 CUDA tensor [B, S]")
+    for name, t in (("word_emb", word_emb), ("pos_emb", pos_emb), ("type_emb", type_emb), ("ln_gamma", ln_gamma), ("ln_beta", ln_beta)):
+        if t is not None:
+            _check_f16_cuda(name, t)
+            if t.shape[-1] != HIDDEN:
+                raise ValueError("%s last dimension must be %d" % (name, HIDDEN))
+    if pos_emb.shape[0] < S:
+        raise ValueError("pos_emb has %d rows, sequence length is %d" % (pos_emb.shape[0], S))
+    tok = token_ids.contiguous()
+    seg = None if segment_ids is None else segment_ids.contiguous()
+    out = torch.empty((B * S, HIDDEN), dtype=torch.float16, device=token_ids.device)
+    sh.check(sh.lib().souffle_bert_embed(tok.data_ptr(), sh.ptr(seg), word_emb.data_ptr(), pos_emb.data_ptr(), sh.ptr(type_emb),
+                                         sh.ptr(ln_gamma), sh.ptr(ln_beta), float(ln_eps), B, S, HIDDEN, out.data_ptr(),
+                                         sh.current_stream()))
+    return out
+
+
+def pooler(x, weight, bias, batch, seq_len):
+    """tanh(x[b, 0, :] . weight + bias): the standard BERT pooler behind the encoder.
+    weight is [K][N] like every weight here; x fp16 [B*S, 768]; returns fp16 [B, 768]."""
+    _check_f16_cuda("x", x)
+    _check_f16_cuda("weight", weight, (HIDDEN, HIDDEN))
+    if bias is not None:
+        _check_f16_cuda("bias", bias)
+    if x.numel() != batch * seq_len * HIDDEN:
+        raise ValueError("x must have %d elements" % (batch * seq_len * HIDDEN))
+    out = torch.empty((batch, HIDDEN), dtype=torch.float16, device=x.device)
+    sh.check(sh.lib().souffle_bert_pooler(x.data_ptr(), weight.data_ptr(), sh.ptr(bias), batch, seq_len, HIDDEN, out.data_ptr(),
+                                          sh.current_stream()))
+    return out
+
+
+def load_hf_bert(path, num_layers=None, prefix=""):
+    """Read a local BERT checkpoint in safetensors format (HuggingFace tensor names) into the
+    layouts used here: every nn.Linear weight [out, in] is transposed to [K][N], q/k/v are stacked
+    to [3][768][768] (the reference's rule: cpp/bert/test_souffle_bert_layer.py:131-143).
+    Returns {"layers": [per-layer dicts of fp16 CPU tensors for Encoder(...)], "embeddings": {...},
+    "pooler": {...}}.  Nothing is fetched: `path` must be a file on disk."""
+    from safetensors.torch import load_file
+    raw = load_file(path)
+    t = lambda name: raw[prefix + name]
+    kn = lambda name: t(name).t().contiguous().to(torch.float16)          # [out, in] -> [K][N]
+    vec = lambda name: t(name).contiguous().to(torch.float16)
+    n = 0
+    while (prefix + "encoder.layer.%d.attention.self.query.weight" % n) in raw:
+        n += 1
+    if num_layers is not None:
+        n = min(n, num_layers)
+    layers = []
+    for i in range(n):
+        p = "encoder.layer.%d." % i
+        layers.append({
+            "qkv_weight": torch.stack([kn(p + "attention.self.%s.weight" % q) for q in ("query", "key", "value")]).contiguous(),
+            "qkv_bias": torch.stack([vec(p + "attention.self.%s.bias" % q) for q in ("query", "key", "value")]).contiguous(),
+            "attn_fc_weight": kn(p + "attention.output.dense.weight"), "attn_fc_bias": vec(p + "attention.output.dense.bias"),
+            "ln1_gamma": vec(p + "attention.output.LayerNorm.weight"), "ln1_beta": vec(p + "attention.output.LayerNorm.bias"),
+            "fc1_weight": kn(p + "intermediate.dense.weight"), "fc1_bias": vec(p + "intermediate.dense.bias"),
+            "fc2_weight": kn(p + "output.dense.weight"), "fc2_bias": vec(p + "output.dense.bias"),
+            "ln2_gamma": vec(p + "output.LayerNorm.weight"), "ln2_beta": vec(p + "output.LayerNorm.bias"),
+        })
+    out = {"layers": layers, "embeddings": None, "pooler": None}
+    if prefix + "embeddings.word_embeddings.weight" in raw:
+        out["embeddings"] = {"word_emb": vec("embeddings.word_embeddings.weight"), "pos_emb": vec("embeddings.position_embeddings.weight"),
+                             "type_emb": vec("embeddings.token_type_embeddings.weight"),
+                             "ln_gamma": vec("embeddings.LayerNorm.weight"), "ln_beta": vec("embeddings.LayerNorm.bias")}
+    if prefix + "pooler.dense.weight" in raw:
+        out["pooler"] = {"weight": kn("pooler.dense.weight"), "bias": vec("pooler.dense.bias")}
+    return out
