@@ -308,12 +308,16 @@ __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, 
 
 // ---- many rows (M a multiple of 256): 256 x BN tiles, see gemm_big.hpp ----
 // BN is chosen per GEMM so that M = 4096 gives exactly 256 tiles, one per CU: 144 for the
-// 2304 QKV columns, 192 for FC1's 3072, 48 for the 768 of the out-projection and FC2.
+// 2304 QKV columns, 192 for FC1's 3072, 48 for the 768 of the out-projection; FC2 (K = 3072)
+// uses 96 columns and two halves of K, which asks the L2 for 0.6x the operand bytes of 48-column
+// tiles over the whole K (a CU takes in operands no faster than it multiplies them): 41 -> 31 us.
+// (The same split for the out-projection, K = 768, gains nothing: its tiles are too short.)
 using BigQkv = GemmBig<144, 5>;
 using BigFc1 = GemmBig<192, 5>;
 using BigOut = GemmBig<48, 5>;
+using BigFc2 = GemmBig<96, 5>;                 // FC2: 8 column tiles x 2 halves of K = 256 tiles at M = 4096
 constexpr int kBigLds = BigFc1::LDS_BYTES;
-static_assert(BigQkv::LDS_BYTES <= kBigLds && BigOut::LDS_BYTES <= kBigLds, "FC1 has the largest ring");
+static_assert(BigQkv::LDS_BYTES <= kBigLds && BigOut::LDS_BYTES <= kBigLds && BigFc2::LDS_BYTES <= kBigLds, "FC1 has the largest ring");
 
 // Workgroup b runs on XCD b % 8.  An XCD gets a quarter of the row tiles and half of the
 // column tiles, so that its L2 fetches each operand tile it needs once.
@@ -391,20 +395,51 @@ __device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, 
     BigOut::run(lds, X, K, tm * 256, 0, K / 32, wptr, cvt, store16);
   }
 }
-// out[m] = LN(z1[m]) * g + b; one wave per row, two-pass statistics in fp32 registers
+// A pre-LayerNorm sum in two halves of K: z1 = X[:, :K/2].W[:K/2] + bias + resid and
+// z2 (in the otherwise unused partials area) = X[:, K/2:].W[K/2:], both fp16; big_ln adds them.
 template <bool COH>
-__device__ __forceinline__ void big_ln(const Params &a, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
+__device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a, const half_t *X, int K, const half_t *W,
+                                            const half_t *bias, const half_t *resid, int first, int stride) {
+  const int m_tiles = a.M / 256, n_tiles = H / BigFc2::kBN;
+  half_t *z2 = reinterpret_cast<half_t *>(a.part);
+  for (int it = first; it < m_tiles * n_tiles * 2; it += stride) {
+    int tm, tn2;
+    big_tile(it, m_tiles, n_tiles * 2, &tm, &tn2);
+    const int ks = tn2 & 1, n0 = (tn2 >> 1) * BigFc2::kBN, k0 = ks * (K / 2);
+    auto wptr = [&](int k, int col) { return W + (size_t)k * H + n0 + col; };
+    auto cvt = [&](int m, int nr, f4 v) {
+      if (ks == 0) {
+        const int n = n0 + nr;
+        const h4 r = as_h4(ld8<false>(resid, (m * H + n) * 2));
+        v = add_bias4(v, bias, n) + f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+      }
+      return pack_h4(v);
+    };
+    auto store16 = [&](int m, int nr, u4 v) { st16<COH>(ks == 0 ? a.z1 : z2, (m * H + n0 + nr) * 2, v); };
+    BigFc2::run(lds, X, K, tm * 256, k0, (K / 2) / 32, wptr, cvt, store16);
+  }
+}
+// out[m] = LN(z1[m] (+ z2[m])) * g + b; one wave per row, two-pass statistics in fp32 registers
+template <bool COH>
+__device__ __forceinline__ void big_ln(const Params &a, const half_t *z2, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
   const int lane = opaque_thread_id() & 63;
   for (int m = first_row; m < a.M; m += row_stride) {
-    u2 raw[3];
+    u2 raw[3], raw2[3];
 #pragma unroll
-    for (int c = 0; c < 3; ++c) raw[c] = ld8<false>(a.z1, (m * H + c * 256 + lane * 4) * 2);
+    for (int c = 0; c < 3; ++c) {
+      raw[c] = ld8<false>(a.z1, (m * H + c * 256 + lane * 4) * 2);
+      if (z2) raw2[c] = ld8<false>(z2, (m * H + c * 256 + lane * 4) * 2);
+    }
     f4 v[3];
     float sum = 0.f;
 #pragma unroll
     for (int c = 0; c < 3; ++c) {
       const h4 r = as_h4(raw[c]);
       v[c] = f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+      if (z2) {
+        const h4 r2 = as_h4(raw2[c]);
+        v[c] += f4{(float)r2[0], (float)r2[1], (float)r2[2], (float)r2[3]};
+      }
       sum += v[c][0] + v[c][1] + v[c][2] + v[c][3];
     }
     const float mean = wave_sum(sum) * (1.0f / H);
@@ -1060,16 +1095,16 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       if constexpr (BIG) big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, xin, first, stride);
       else stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
       grid_sync(bar);
-      if constexpr (BIG) big_ln<true>(a, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
+      if constexpr (BIG) big_ln<true>(a, nullptr, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
       else stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
       grid_sync(bar);
       if constexpr (BIG) big_fc1<true>(lds_raw, a, w, first, stride);
       else stage_fc1<true, Tile>(lds, a, w, first, stride);
       grid_sync(bar);
-      if constexpr (BIG) big_presum<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, a.y1, first, stride);
+      if constexpr (BIG) big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, a.y1, first, stride);
       else stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
       grid_sync(bar);
-      if constexpr (BIG) big_ln<true>(a, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
+      if constexpr (BIG) big_ln<true>(a, reinterpret_cast<const half_t *>(a.part), w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
       else stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
     } else {
       // Weight slices are queued one stage ahead, from inside the grid barrier that precedes
@@ -1263,8 +1298,12 @@ __global__ void __launch_bounds__(256) k_presum_big(Args a, const half_t *X, int
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   big_presum<false>(lds_raw, a, X, K, W, bias, resid, blockIdx.x, gridDim.x);
 }
-__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *gam, const half_t *bet, half_t *out) {
-  big_ln<false>(a, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
+__global__ void __launch_bounds__(256) k_presum2_big(Args a, const half_t *X, int K, const half_t *W, const half_t *bias, const half_t *resid) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  big_presum2<false>(lds_raw, a, X, K, W, bias, resid, blockIdx.x, gridDim.x);
+}
+__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *z2, const half_t *gam, const half_t *bet, half_t *out) {
+  big_ln<false>(a, z2, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
 }
 template <int MODE>
 __global__ void __launch_bounds__(256) k_fc1(Args a, int l) {
@@ -1454,7 +1493,10 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
   static bool attr_done = false;
   if (!attr_done) {
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_qkv<MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
-    if constexpr (MODE == 2) SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_presum_big, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
+    if constexpr (MODE == 2) {
+      SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_presum_big, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
+      SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_presum2_big, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
+    }
     else SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_partial<MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_fc1<MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS));
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)k_attn, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLdsBytes));
@@ -1473,7 +1515,7 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     else hipLaunchKernelGGL(k_attn_small, dim3(grid_for((a.B * NH + 7) / 8 * 8 * (a.S / 16))), dim3(256), attn_small_lds_bytes(a.S), st, a);
     if constexpr (MODE == 2) {
       hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * (H / BigOut::kBN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, w.b_o, xin);
-      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, w.ln1_g, w.ln1_b, a.y1);
+      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)nullptr, w.ln1_g, w.ln1_b, a.y1);
     } else if constexpr (LARGE) {
       hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, 1);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, 1, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
@@ -1482,8 +1524,8 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     }
     hipLaunchKernelGGL(k_fc1<MODE>, dim3(grid_for((a.M / BM_QKV) * (F / BN))), dim3(256), GEMM_LDS, st, a, l);
     if constexpr (MODE == 2) {
-      hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * (H / BigOut::kBN))), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, w.b_fc2, a.y1);
-      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, w.ln2_g, w.ln2_b, yout);
+      hipLaunchKernelGGL(k_presum2_big, dim3(grid_for((a.M / 256) * (H / BigFc2::kBN) * 2)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, w.b_fc2, a.y1);
+      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, reinterpret_cast<const half_t *>(a.part), w.ln2_g, w.ln2_b, yout);
     } else {
       hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_FC2) * (H / BN) * a.splitk_f)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, a.splitk_f);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout);

@@ -13,7 +13,7 @@
 //   W stage [32 k][BN]:       slot(k, c) = k*BN/8 + (c ^ swz(k)); the four rows a 16-lane group of
 //            the transposing read touches must fall into different banks: their distance is
 //            BN/2 banks, i.e. 8 (BN = 144), 24 (BN = 48) - fine as they are - or 0 (BN = 192),
-//            where swz(k) = 2(k & 3) moves them apart.
+//            where swz(k) = 2(k & 3) moves them apart, or 16 (BN = 96), where swz(k) = k & 2 does.
 // W is row-major [K][N] as the reference stores it (cpp/bert/kernels/gemm_three_stages.h:95-131);
 // the MFMA takes W as operand A and X as operand B, so a lane ends up with 4 consecutive output
 // columns of one row.
@@ -36,6 +36,7 @@ __device__ __forceinline__ void static_for(Fn f) {
 template <int BN, int NSTAGE>
 struct GemmBig {
   static_assert(BN % 16 == 0 && (BN * 64) % 1024 == 0, "whole MFMA tiles and whole wave-wide loads");
+  static_assert(BN == 48 || BN == 96 || BN == 144 || BN == 192, "the W swizzle is worked out for these widths");
   static constexpr int kBM = 256, kBN = BN, kBK = 32;
   static constexpr int NT = BN / 16;                        // accumulator tiles per row block
   static constexpr int WSLOTS = BN / 8;                     // 16-byte slots per W row
@@ -55,7 +56,7 @@ struct GemmBig {
   typedef __attribute__((address_space(1))) const void *gptr_t;
   typedef __attribute__((address_space(3))) void *lptr_t;
 
-  __device__ static __forceinline__ int wswz(int k) { return BN == 192 ? ((k & 3) << 1) : 0; }
+  __device__ static __forceinline__ int wswz(int k) { return BN == 192 ? ((k & 3) << 1) : (BN == 96 ? (k & 2) : 0); }
 
   // Load number L (0 .. LPW-1) of this wave for the stage at LDS address `stage`, K offset kk.
   // wptr(k, col) -> address of W[k][col] (col relative to the tile's first column, multiple of 8)
