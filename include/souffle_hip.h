@@ -240,6 +240,49 @@ int souffle_se_module_fused(const float *x, const float *w_reduce, const float *
                             float *y, float *pooled, int C, int HW, int R, int combine,
                             void *workspace, size_t workspace_bytes, souffle_stream_t stream);
 
+/* ------------------------------------------------- EfficientNet MBConv ---- */
+/* NHWC fp16 activations (batch 1), fp16 convolution weights, fp32 folded batch-norm vectors
+ * (y = conv * scale + shift) and squeeze-excite biases.  Channel counts are multiples of 8. */
+enum { SOUFFLE_MB_NONE = 0, SOUFFLE_MB_SWISH = 1 };
+typedef struct {
+  int in_h, in_w, in_c, expand_c, out_c;   /* expand_c == in_c and expand_w == NULL: no expansion convolution */
+  int kernel, stride;                      /* depthwise: 3 or 5; 1 or 2; padding kernel/2 on every side */
+  int se_c;                                /* squeezed channels; 0 = no squeeze-excite module */
+  int has_shortcut;                        /* y += x; needs stride 1 and in_c == out_c */
+  const void *expand_w;                    /* fp16 [expand_c][in_c] */
+  const float *expand_scale, *expand_shift;
+  const void *dw_w;                        /* fp16 [kernel][kernel][expand_c] */
+  const float *dw_scale, *dw_shift;
+  const void *se_reduce_w;                 /* fp16 [se_c][expand_c] */
+  const float *se_reduce_b;                /* [se_c], nullable */
+  const void *se_expand_w;                 /* fp16 [expand_c][se_c] */
+  const float *se_expand_b;                /* [expand_c], nullable */
+  const void *project_w;                   /* fp16 [out_c][expand_c] */
+  const float *project_scale, *project_shift;
+} souffle_mbconv_block;
+/* 0 (and an error text) when the block list is not valid. */
+size_t souffle_mbconv_workspace_bytes(const souffle_mbconv_block *blocks, int num_blocks);
+/* A chain of MBConv blocks, x [in_h*in_w][in_c] of block 0 -> y [oh*ow][out_c] of the last block.
+ * Replaces the per-block operator sequence of TVMMBConvBlock.forward
+ * (python/models/efficientnet/tvm_efficientnet.py:62-118; operators
+ * python/models/efficientnet/efficientnet.py:41-57,83-101,131-141,173-195,252-282,502-518).
+ * fused != 0: one persistent launch per 16 blocks; fused == 0: one launch per operator group
+ * (expansion | depthwise | squeeze-excite + projection), the same arithmetic. */
+int souffle_mbconv_stack(const souffle_mbconv_block *blocks, int num_blocks, const void *x, void *y, int fused,
+                         void *workspace, size_t workspace_bytes, souffle_stream_t stream);
+/* y[p][o] = act((sum_k x[p][k] * gate[k] * w[o][k]) * scale[o] + shift[o]) + shortcut[p][o];
+ * scale, shift, gate (fp32 [in_c]) and shortcut (fp16 [pixels][out_c]) nullable.
+ * Replaces pointwise_conv2d_bn, pointwise_conv2d_bn_short_cut_add and head_conv1x1_bn_swish
+ * (python/models/efficientnet/efficientnet.py:41-57,83-101,502-518). */
+int souffle_pointwise_conv2d_bn(const void *x, const void *w, const float *scale, const float *shift,
+                                const float *gate, const void *shortcut, void *y,
+                                int pixels, int in_c, int out_c, int act, souffle_stream_t stream);
+/* x [in_h][in_w][C], w [kernel][kernel][C] -> y [oh][ow][C], o = (in - 1) / stride + 1.
+ * Replaces fused_depthwise_conv2d_bn_swish (python/models/efficientnet/efficientnet.py:173-195). */
+int souffle_depthwise_conv2d_bn_swish(const void *x, const void *w, const float *scale, const float *shift,
+                                      void *y, int in_h, int in_w, int channels, int kernel, int stride,
+                                      souffle_stream_t stream);
+
 /* ------------------------------------------------------------- timing ---- */
 /* Replaces benchmarkCudaFunc (cpp/souffle_utils/cuda_utils.h:102-136): after `warmup`
  * launches, min over `rounds` of the mean of `repeat` event-timed launches, in us.

@@ -16,6 +16,9 @@
  *                              brute force on tiny grids, permutation laws
  *   oracle_swin_block_pair_f32 torch CPU library restatement of a Swin block
  *   oracle_se_module_f32       torch avg_pool2d / conv2d / sigmoid composition
+ *   oracle_pointwise_conv_f32, oracle_depthwise_conv_f32, oracle_se_gate_f32,
+ *   oracle_mbconv_block_f32    torch conv2d (groups / stride / explicit padding), adaptive
+ *                              average pooling, sigmoid in float64; brute force on tiny inputs
  *   oracle_bert_embed_f32      torch.nn.functional.embedding + layer_norm (float64)
  *   oracle_bert_pooler_f32     torch matmul + tanh (float64), transposition rule of the
  *                              reference (cpp/bert/test_souffle_bert_layer.py:139-143)
@@ -140,6 +143,29 @@ enum { ORACLE_SE_MUL = 0, ORACLE_SE_ADD = 1 };
 int oracle_se_module_f32(const float *x, const float *w_reduce, const float *b_reduce,
                          const float *w_expand, const float *b_expand, float *y, float *pooled,
                          int C, int HW, int R, int combine);
+
+/* ---- EfficientNet MBConv operators (NHWC, batch 1) ---- */
+enum { ORACLE_MB_NONE = 0, ORACLE_MB_SWISH = 1 };
+typedef struct {
+  int in_h, in_w, in_c, expand_c, out_c, kernel, stride, se_c, has_shortcut;
+  const float *expand_w, *expand_scale, *expand_shift;   /* [expand_c][in_c]; NULL = no expansion conv */
+  const float *dw_w, *dw_scale, *dw_shift;               /* [kernel][kernel][expand_c] */
+  const float *se_reduce_w, *se_reduce_b;                /* [se_c][expand_c], [se_c] */
+  const float *se_expand_w, *se_expand_b;                /* [expand_c][se_c], [expand_c] */
+  const float *project_w, *project_scale, *project_shift;/* [out_c][expand_c] */
+} oracle_mbconv_block;
+/* x [pixels][in_c], w [out_c][in_c]; scale/shift/gate/shortcut nullable. */
+int oracle_pointwise_conv_f32(const float *x, const float *w, const float *scale, const float *shift,
+                              const float *gate, const float *shortcut, float *y,
+                              int pixels, int in_c, int out_c, int act, int num_threads);
+int oracle_depthwise_out_extent(int in, int kernel, int stride);
+/* x [in_h][in_w][C], w [kernel][kernel][C] -> y [oh][ow][C]. */
+int oracle_depthwise_conv_f32(const float *x, const float *w, const float *scale, const float *shift, float *y,
+                              int in_h, int in_w, int channels, int kernel, int stride, int act, int num_threads);
+int oracle_se_gate_f32(const float *x, const float *w_reduce, const float *b_reduce, const float *w_expand,
+                       const float *b_expand, float *gate, int pixels, int channels, int squeezed);
+int oracle_mbconv_block_f32(const oracle_mbconv_block *b, const float *x, float *y, float *dump_e, float *dump_d,
+                            int round_fp16, int num_threads);
 #ifdef __cplusplus
 }
 #endif

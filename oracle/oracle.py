@@ -257,3 +257,84 @@ def se_module(x, w_reduce, w_expand, b_reduce=None, b_expand=None, combine="mul"
     if rc:
         raise RuntimeError("oracle_se_module_f32 failed: %d" % rc)
     return y, pooled
+
+
+# ---- EfficientNet MBConv operators (NHWC, batch 1) ----
+_MB_INT = ["in_h", "in_w", "in_c", "expand_c", "out_c", "kernel", "stride", "se_c", "has_shortcut"]
+_MB_PTR = ["expand_w", "expand_scale", "expand_shift", "dw_w", "dw_scale", "dw_shift", "se_reduce_w", "se_reduce_b",
+           "se_expand_w", "se_expand_b", "project_w", "project_scale", "project_shift"]
+
+
+class _MbBlock(C.Structure):
+    _fields_ = [(n, C.c_int) for n in _MB_INT] + [(n, C.c_void_p) for n in _MB_PTR]
+
+
+def depthwise_out_extent(n, kernel, stride):
+    return lib().oracle_depthwise_out_extent(n, kernel, stride)
+
+
+def pointwise_conv(x, w, scale=None, shift=None, gate=None, shortcut=None, act="none", threads=0):
+    """x [pixels, in_c], w [out_c, in_c] -> [pixels, out_c]."""
+    x, w, scale, shift, gate, shortcut = _f32(x), _f32(w), _f32(scale), _f32(shift), _f32(gate), _f32(shortcut)
+    P, K = x.shape
+    N = w.shape[0]
+    y = np.empty((P, N), np.float32)
+    rc = lib().oracle_pointwise_conv_f32(_p(x), _p(w), _p(scale), _p(shift), _p(gate), _p(shortcut), _p(y), P, K, N,
+                                         {"none": 0, "swish": 1}[act], threads)
+    if rc:
+        raise RuntimeError("oracle_pointwise_conv_f32 failed: %d" % rc)
+    return y
+
+
+def depthwise_conv(x, w, scale=None, shift=None, stride=1, act="swish", threads=0):
+    """x [H, W, C], w [k, k, C] -> [oh, ow, C]."""
+    x, w, scale, shift = _f32(x), _f32(w), _f32(scale), _f32(shift)
+    H, W, Cc = x.shape
+    k = w.shape[0]
+    oh, ow = depthwise_out_extent(H, k, stride), depthwise_out_extent(W, k, stride)
+    y = np.empty((oh, ow, Cc), np.float32)
+    rc = lib().oracle_depthwise_conv_f32(_p(x), _p(w), _p(scale), _p(shift), _p(y), H, W, Cc, k, stride,
+                                         {"none": 0, "swish": 1}[act], threads)
+    if rc:
+        raise RuntimeError("oracle_depthwise_conv_f32 failed: %d" % rc)
+    return y
+
+
+def se_gate(x, w_reduce, b_reduce, w_expand, b_expand):
+    """x [pixels, C] -> gate [C]."""
+    x, w_reduce, b_reduce, w_expand, b_expand = _f32(x), _f32(w_reduce), _f32(b_reduce), _f32(w_expand), _f32(b_expand)
+    P, Cc = x.shape
+    g = np.empty(Cc, np.float32)
+    rc = lib().oracle_se_gate_f32(_p(x), _p(w_reduce), _p(b_reduce), _p(w_expand), _p(b_expand), _p(g), P, Cc,
+                                  w_reduce.shape[0])
+    if rc:
+        raise RuntimeError("oracle_se_gate_f32 failed: %d" % rc)
+    return g
+
+
+def mbconv_block(x, blk, round_fp16=False, dump=False, threads=0):
+    """blk: dict with the integer fields and weight arrays of one block (synth.mbconv_block_weights).
+    x [in_h*in_w, in_c] -> y [oh*ow, out_c] (and the expanded / depthwise tensors when dump)."""
+    keep, b = [], _MbBlock()
+    for n in _MB_INT:
+        setattr(b, n, int(blk[n]))
+    for n in _MB_PTR:
+        a = _f32(blk.get(n))
+        keep.append(a)
+        setattr(b, n, _p(a))
+    x = _f32(x).reshape(blk["in_h"] * blk["in_w"], blk["in_c"])
+    oh = depthwise_out_extent(blk["in_h"], blk["kernel"], blk["stride"])
+    ow = depthwise_out_extent(blk["in_w"], blk["kernel"], blk["stride"])
+    y = np.empty((oh * ow, blk["out_c"]), np.float32)
+    e = np.empty((x.shape[0], blk["expand_c"]), np.float32) if dump and blk.get("expand_w") is not None else None
+    d = np.empty((oh * ow, blk["expand_c"]), np.float32) if dump else None
+    rc = lib().oracle_mbconv_block_f32(C.byref(b), _p(x), _p(y), _p(e), _p(d), int(round_fp16), threads)
+    if rc:
+        raise RuntimeError("oracle_mbconv_block_f32 failed: %d" % rc)
+    return (e, d, y) if dump else y
+
+
+def mbconv_stack(x, blocks, round_fp16=False, threads=0):
+    for blk in blocks:
+        x = mbconv_block(x, blk, round_fp16=round_fp16, threads=threads)
+    return x

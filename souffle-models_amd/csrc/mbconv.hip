@@ -1,0 +1,465 @@
+// EfficientNet MBConv stack (NHWC, fp16, batch 1) as one persistent kernel on gfx950.
+//
+// Replaces the operator sequence that the reference times block by block
+// (python/models/efficientnet/tvm_efficientnet.py:62-118): head_conv1x1_bn_swish (expansion,
+// python/models/efficientnet/efficientnet.py:502-518), fused_depthwise_conv2d_bn_swish
+// (:173-195), the squeeze-excite operators (reduce_mean :131-141, se_module_pointwise_conv
+// :270-282, fused_pointwise_conv_bias_add_sigmoid_mul :252-267) and pointwise_conv2d_bn
+// (:41-57) / pointwise_conv2d_bn_short_cut_add (:83-101).  The reference launches 7 to 9
+// kernels per block; here a block is three stages of one launch, separated by grid barriers:
+//
+//   expand   : E = swish(bn(X . We^T))                      one 16x16 MFMA tile per wave
+//   depthwise: D = swish(bn(dwconv(E))), and per workgroup the contribution of its pixels to
+//              the squeeze layer W_r . sum_p D[p]  (R numbers instead of C channel sums)
+//   project  : every workgroup finishes the squeeze-excite gate from those partials (R and C
+//              are tiny), then Y = bn((D * gate) . Wp^T) (+ X), the gate applied to the
+//              activation operand on its way into the MFMA
+//
+// The whole network moves 0.4 GFLOP over ~7 MB of weights and ~12 MB of activations: every
+// stage is latency bound, so the design goal is few, short stages, not MFMA utilisation.  The
+// GEMMs therefore take both operands straight from global memory/L2 in MFMA operand layout
+// (weights are [out][in], as pointwise_conv2d_bn stores them, so a lane's 8 consecutive
+// k-values are one 16-byte load): no LDS staging, no workgroup barrier inside a stage.
+//
+// Activations written by one stage and read by the next are stored write-through and read
+// with agent-coherent loads: tiles of 16 output channels of neighbouring pixels share cache
+// lines, and those lines are written from several XCDs.
+#include "common.hpp"
+#include "host_util.hpp"
+
+namespace souffle {
+namespace mbconv {
+
+constexpr int MAX_BLOCKS = 16;   // per launch (the descriptors travel as kernel arguments)
+constexpr int MAX_C = 2048, MAX_R = 64, PART_LD = 64;
+
+struct Block {
+  int H, W, Ho, Wo, Cin, Cexp, Cout, k, stride, R, has_expand, has_shortcut;
+  const half_t *w_exp, *w_dw, *w_red, *w_se, *w_proj;
+  const float *s_exp, *b_exp, *s_dw, *b_dw, *b_red, *b_se, *s_proj, *b_proj;
+  const half_t *in;
+  half_t *e, *d, *out;
+  float *part;                   // [workgroup][PART_LD] partial sums of the squeeze layer
+};
+
+struct Args {
+  int nblk, stage_begin, stage_end, pad;
+  unsigned *ctl;
+  Block blk[MAX_BLOCKS];
+};
+static_assert(sizeof(Args) <= 4096, "kernel argument segment");
+
+__device__ __forceinline__ float swish(float v) { return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
+__device__ __forceinline__ float sigmoid(float v) { return __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
+
+// Partial dot products of one 16 x 16 tile: MFMA k-steps first, first + stride, ... (32 k-values
+// each) of rows xbase/wbase.  UNROLL steps are loaded together before their MFMAs are issued, so
+// that many 16-byte loads per operand are in flight per wave; steps past K load nothing and
+// multiply zeros.  The trip count is wave-uniform.
+template <bool GATE, bool COH, int UNROLL>
+__device__ __forceinline__ f4 tile_dot(const half_t *X, int xbase, const half_t *__restrict__ Wt, int wbase, bool wok, int K,
+                                       int first, int stride, const float *gate, int g) {
+  f4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s0 = first; s0 * 32 < K; s0 += UNROLL * stride) {
+    u4 xv[UNROLL], wv[UNROLL];
+#pragma unroll
+    for (int i = 0; i < UNROLL; ++i) {
+      const int kk = (s0 + i * stride) * 32 + g * 8;
+      const bool ok = kk < K;
+      const int ks = ok ? kk : 0;
+      xv[i] = ld16<COH>(X, (xbase + ks) * 2);
+      wv[i] = *reinterpret_cast<const u4 *>(Wt + wbase + ks);
+      if (!ok) xv[i] = u4{0u, 0u, 0u, 0u};
+      if (!ok || !wok) wv[i] = u4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int i = 0; i < UNROLL; ++i) {
+      if constexpr (GATE) {
+        const int kk = (s0 + i * stride) * 32 + g * 8, ks = kk < K ? kk : 0;
+        const f4 g0 = *reinterpret_cast<const f4 *>(gate + ks), g1 = *reinterpret_cast<const f4 *>(gate + ks + 4);
+        const h8 x = as_h8(xv[i]);
+        xv[i] = as_u4(h8{(half_t)((float)x[0] * g0[0]), (half_t)((float)x[1] * g0[1]), (half_t)((float)x[2] * g0[2]),
+                         (half_t)((float)x[3] * g0[3]), (half_t)((float)x[4] * g1[0]), (half_t)((float)x[5] * g1[1]),
+                         (half_t)((float)x[6] * g1[2]), (half_t)((float)x[7] * g1[3])});
+      }
+      acc = mfma_16x16x32(as_h8(wv[i]), as_h8(xv[i]), acc);
+    }
+  }
+  return acc;
+}
+
+// Y[M][N] = act((X[M][K] * gate[K]) . Wt[N][K]^T * scale[N] + shift[N]) (+ shortcut[M][N]) in
+// 16 x 16 output tiles.  K and N are multiples of 8, so 16-byte operand granules and 8-byte
+// result granules are all-or-nothing at the edges.  With more tiles than workgroups a wave owns
+// a tile; otherwise (few pixels, many input channels: the late blocks) a workgroup owns a tile,
+// its four waves take every fourth k-step and the partial tiles are summed through `red`.
+// COH: X and shortcut were written earlier in this launch by other workgroups.
+template <bool GATE, bool COH>
+__device__ __forceinline__ void pointwise(const half_t *X, int M, int K, int N, const half_t *__restrict__ Wt,
+                                          const float *__restrict__ scale, const float *__restrict__ shift, bool act,
+                                          const float *gate, const half_t *shortcut, half_t *Y, float *red) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+  const int nt_n = (N + 15) >> 4, units = ((M + 15) >> 4) * nt_n;
+  const bool split = units <= (int)gridDim.x;
+  auto epilogue = [&](int mt, int nt, f4 acc) {
+    const int row = mt * 16 + l16, col = nt * 16 + g * 4;
+    if (row < M && col < N) {
+      f4 sc = {1.f, 1.f, 1.f, 1.f}, sh = {0.f, 0.f, 0.f, 0.f};
+      if (scale) sc = *reinterpret_cast<const f4 *>(scale + col);
+      if (shift) sh = *reinterpret_cast<const f4 *>(shift + col);
+      f4 v = acc * sc + sh;
+      if (act) v = f4{swish(v[0]), swish(v[1]), swish(v[2]), swish(v[3])};
+      if (shortcut) {
+        const h4 s = as_h4(ld8<COH>(shortcut, (row * N + col) * 2));
+        v += f4{(float)s[0], (float)s[1], (float)s[2], (float)s[3]};
+      }
+      st8<COH>(Y, (row * N + col) * 2, pack_h4(v));
+    }
+  };
+  if (split) {
+    const int u = blockIdx.x;
+    if (u < units) {
+      const int mt = u / nt_n, nt = u - mt * nt_n, wrow = nt * 16 + l16;
+      const bool wok = wrow < N;
+      const f4 part = tile_dot<GATE, COH, 12>(X, min(mt * 16 + l16, M - 1) * K, Wt, (wok ? wrow : N - 1) * K, wok, K, wave, 4, gate, g);
+      *reinterpret_cast<f4 *>(red + tid * 4) = part;
+      __syncthreads();
+      if (wave == 0) {
+        f4 acc = part;
+#pragma unroll
+        for (int w = 1; w < 4; ++w) acc += *reinterpret_cast<const f4 *>(red + (w * 64 + lane) * 4);
+        epilogue(mt, nt, acc);
+      }
+    }
+  } else {
+    for (int u = blockIdx.x * 4 + wave; u < units; u += gridDim.x * 4) {
+      const int mt = u / nt_n, nt = u - mt * nt_n, wrow = nt * 16 + l16;
+      const bool wok = wrow < N;
+      const f4 acc = tile_dot<GATE, COH, 6>(X, min(mt * 16 + l16, M - 1) * K, Wt, (wok ? wrow : N - 1) * K, wok, K, 0, 1, gate, g);
+      epilogue(mt, nt, acc);
+    }
+  }
+}
+
+// D[ho][wo][c] = swish(bn(sum_ij X[ho*s - pad + i][wo*s - pad + j][c] * W[i][j][c])), pad = KS/2.
+// A thread owns 8 channels of one output pixel; G = C/8 neighbouring threads cover a pixel, so a
+// wave reads and writes whole contiguous runs of the NHWC tensors.  When the block has a
+// squeeze-excite module (R > 0) the thread also sums its outputs over its pixels; the workgroup
+// reduces those sums in a fixed order and writes W_r . sums, its share of the squeeze layer.
+template <int KS, bool COH>
+__device__ __forceinline__ void depthwise(const Block &b, float *red, float *sums) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int C = b.Cexp, G = C >> 3, P = 256 / G;
+  const int slot = tid / G, cg = tid - slot * G;
+  const bool active = slot < P;
+  const int npix = b.Ho * b.Wo, groups = (npix + P - 1) / P;
+  const half_t *src = b.has_expand ? b.e : b.in;
+  constexpr int pad = KS / 2;
+  float sc[8], sh[8], sum[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    sc[q] = (active && b.s_dw) ? b.s_dw[cg * 8 + q] : 1.f;
+    sh[q] = (active && b.b_dw) ? b.b_dw[cg * 8 + q] : 0.f;
+    sum[q] = 0.f;
+  }
+  for (int grp = blockIdx.x; grp < groups; grp += gridDim.x) {
+    const int pix = grp * P + slot;
+    if (active && pix < npix) {
+      const int ho = pix / b.Wo, wo = pix - ho * b.Wo;
+      float acc[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) acc[q] = 0.f;
+#pragma unroll
+      for (int i = 0; i < KS; ++i) {
+        const int hi = ho * b.stride - pad + i;
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+          const int wi = wo * b.stride - pad + j;
+          if (hi >= 0 && hi < b.H && wi >= 0 && wi < b.W) {
+            const h8 x = as_h8(ld16<COH>(src, ((hi * b.W + wi) * C + cg * 8) * 2));
+            const h8 w = as_h8(*reinterpret_cast<const u4 *>(b.w_dw + (i * KS + j) * C + cg * 8));
+#pragma unroll
+            for (int q = 0; q < 8; ++q) acc[q] += (float)x[q] * (float)w[q];
+          }
+        }
+      }
+      h8 o;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float v = swish(acc[q] * sc[q] + sh[q]);
+        sum[q] += v;
+        o[q] = (half_t)v;
+      }
+      st16<COH>(b.d, (pix * C + cg * 8) * 2, as_u4(o));
+    }
+  }
+  if (b.R <= 0) return;
+  if (active) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) red[slot * C + cg * 8 + q] = sum[q];      // slot*C + ... < P*8G <= 2048
+  }
+  __syncthreads();
+  for (int c = tid; c < C; c += 256) {
+    float s = 0.f;
+    for (int sl = 0; sl < P; ++sl) s += red[sl * C + c];
+    sums[c] = s;
+  }
+  __syncthreads();
+  if ((int)blockIdx.x < groups) {
+    for (int j = wave; j < b.R; j += 4) {
+      float s = 0.f;
+      for (int c = lane; c < C; c += 64) s += (float)b.w_red[j * C + c] * sums[c];
+      s = wave_sum(s);
+      if (lane == 0) st4<COH>(b.part, ((int)blockIdx.x * PART_LD + j) * 4, __float_as_uint(s));
+    }
+  }
+  __syncthreads();                 // red / sums are reused by the next stage
+}
+
+// gate[c] = sigmoid(b_e[c] + sum_j W_e[c][j] * swish(b_r[j] + (sum over workgroups of part[.][j]) / pixels)),
+// evaluated by every workgroup for itself, then the projection with the gate folded into its operand.
+template <bool COH>
+__device__ __forceinline__ void project(const Block &b, float *gate_s, float *r_s, float *red) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int npix = b.Ho * b.Wo, C = b.Cexp;
+  const half_t *shortcut = b.has_shortcut ? b.in : nullptr;
+  if (b.R <= 0) {
+    pointwise<false, COH>(b.d, npix, C, b.Cout, b.w_proj, b.s_proj, b.b_proj, false, nullptr, shortcut, b.out, red);
+    return;
+  }
+  const int P = 256 / (C >> 3), groups = (npix + P - 1) / P, nact = min(groups, (int)gridDim.x);
+  for (int j = wave; j < b.R; j += 4) {
+    float s = 0.f;
+    for (int wg = lane; wg < nact; wg += 64) s += __uint_as_float(ld4<COH>(b.part, (wg * PART_LD + j) * 4));
+    s = wave_sum(s);
+    if (lane == 0) r_s[j] = swish(s / (float)npix + (b.b_red ? b.b_red[j] : 0.f));
+  }
+  __syncthreads();
+  for (int c = tid; c < C; c += 256) {
+    float s = b.b_se ? b.b_se[c] : 0.f;
+    for (int j = 0; j < b.R; ++j) s += (float)b.w_se[c * b.R + j] * r_s[j];
+    gate_s[c] = sigmoid(s);
+  }
+  __syncthreads();
+  pointwise<true, COH>(b.d, npix, C, b.Cout, b.w_proj, b.s_proj, b.b_proj, false, gate_s, shortcut, b.out, red);
+}
+
+// Stage s of the launch is phase s % 3 (expand, depthwise, project) of block s / 3.
+__global__ void __launch_bounds__(256) k_mbconv(const Args a) {
+  __shared__ __attribute__((aligned(16))) float red[2048];
+  __shared__ __attribute__((aligned(16))) float vec[MAX_C];
+  __shared__ float r_s[MAX_R];
+  GridBarrier bar;
+  grid_barrier_begin(bar, a.ctl);
+  for (int st = a.stage_begin; st < a.stage_end; ++st) {
+    const int bi = st / 3, ph = st - bi * 3;
+    const Block &b = a.blk[bi];
+    bool ran = true;
+    if (ph == 0) {
+      if (b.has_expand)
+        pointwise<false, true>(b.in, b.H * b.W, b.Cin, b.Cexp, b.w_exp, b.s_exp, b.b_exp, true, nullptr, nullptr, b.e, red);
+      else
+        ran = false;
+    } else if (ph == 1) {
+      if (b.k == 3) depthwise<3, true>(b, red, vec);
+      else depthwise<5, true>(b, red, vec);
+    } else {
+      project<true>(b, vec, r_s, red);
+    }
+    if (ran && st + 1 < a.stage_end) grid_sync(bar);
+  }
+  grid_barrier_end(bar);
+}
+
+// ---- single operators (the reference's operator list as entry points of their own) ----
+struct PwArgs {
+  const half_t *x, *w, *shortcut;
+  const float *scale, *shift, *gate;
+  half_t *y;
+  int M, K, N, act;
+};
+__global__ void __launch_bounds__(256) k_pointwise(const PwArgs a) {
+  __shared__ __attribute__((aligned(16))) float gate_s[MAX_C];
+  __shared__ __attribute__((aligned(16))) float red[1024];
+  if (a.gate) {
+    for (int c = threadIdx.x; c < a.K; c += 256) gate_s[c] = a.gate[c];
+    __syncthreads();
+    pointwise<true, false>(a.x, a.M, a.K, a.N, a.w, a.scale, a.shift, a.act != 0, gate_s, a.shortcut, a.y, red);
+  } else {
+    pointwise<false, false>(a.x, a.M, a.K, a.N, a.w, a.scale, a.shift, a.act != 0, nullptr, a.shortcut, a.y, red);
+  }
+}
+__global__ void __launch_bounds__(256) k_depthwise(const Block b) {
+  __shared__ float red[2048];
+  __shared__ float vec[MAX_C];
+  if (b.k == 3) depthwise<3, false>(b, red, vec);
+  else depthwise<5, false>(b, red, vec);
+}
+
+static int out_extent(int in, int kernel, int stride) { return (in + (kernel - 1) - kernel) / stride + 1; }
+
+static int check_block(const souffle_mbconv_block *s, int i) {
+  if (s->in_h <= 0 || s->in_w <= 0) return fail(SOUFFLE_ERR_SHAPE, "block %d: in_h and in_w must be positive", i);
+  if (s->in_c <= 0 || s->expand_c <= 0 || s->out_c <= 0 || s->in_c % 8 || s->expand_c % 8 || s->out_c % 8)
+    return fail(SOUFFLE_ERR_SHAPE, "block %d: channel counts must be positive multiples of 8 (got %d, %d, %d)", i, s->in_c,
+                s->expand_c, s->out_c);
+  if (s->expand_c > MAX_C) return fail(SOUFFLE_ERR_SHAPE, "block %d: expand_c <= %d required (got %d)", i, MAX_C, s->expand_c);
+  if (s->se_c < 0 || s->se_c > MAX_R) return fail(SOUFFLE_ERR_SHAPE, "block %d: 0 <= se_c <= %d required (got %d)", i, MAX_R, s->se_c);
+  if (s->kernel != 3 && s->kernel != 5) return fail(SOUFFLE_ERR_SHAPE, "block %d: kernel must be 3 or 5 (got %d)", i, s->kernel);
+  if (s->stride != 1 && s->stride != 2) return fail(SOUFFLE_ERR_SHAPE, "block %d: stride must be 1 or 2 (got %d)", i, s->stride);
+  if (!s->expand_w && s->expand_c != s->in_c)
+    return fail(SOUFFLE_ERR_SHAPE, "block %d: without an expansion convolution expand_c must equal in_c", i);
+  if (s->has_shortcut && (s->stride != 1 || s->in_c != s->out_c))
+    return fail(SOUFFLE_ERR_SHAPE, "block %d: the shortcut needs stride 1 and in_c == out_c", i);
+  if ((long long)s->in_h * s->in_w * s->expand_c >= (1ll << 29))
+    return fail(SOUFFLE_ERR_SHAPE, "block %d: activation of %d x %d x %d elements exceeds the 2^29 limit", i, s->in_h, s->in_w, s->expand_c);
+  if (!s->dw_w || !s->project_w) return fail(SOUFFLE_ERR_NULL, "block %d: dw_w and project_w must not be NULL", i);
+  if (s->se_c > 0 && (!s->se_reduce_w || !s->se_expand_w))
+    return fail(SOUFFLE_ERR_NULL, "block %d: se_reduce_w and se_expand_w must not be NULL when se_c > 0", i);
+  if (!aligned16(s->expand_w) || !aligned16(s->dw_w) || !aligned16(s->project_w) || !aligned16(s->expand_scale) ||
+      !aligned16(s->expand_shift) || !aligned16(s->project_scale) || !aligned16(s->project_shift))
+    return fail(SOUFFLE_ERR_ALIGN, "block %d: weights and folded batch-norm vectors must be 16-byte aligned", i);
+  return SOUFFLE_OK;
+}
+
+// Workspace: control block, then per block E (if expanded), D, the block output (all blocks but
+// the last) and the squeeze partials, each at an address of its own (see the file comment).
+struct Plan {
+  size_t e[1024], d[1024], out[1024], part[1024], total;
+};
+static int make_plan(const souffle_mbconv_block *blocks, int n, Plan *p) {
+  if (!blocks || n <= 0 || n > 1024) return fail(SOUFFLE_ERR_SHAPE, "need 1..1024 blocks");
+  size_t off = round_up(kCtlWords * 4, 256);
+  for (int i = 0; i < n; ++i) {
+    const souffle_mbconv_block *s = blocks + i;
+    if (int rc = check_block(s, i)) return rc;
+    const int oh = out_extent(s->in_h, s->kernel, s->stride), ow = out_extent(s->in_w, s->kernel, s->stride);
+    if (i + 1 < n && (blocks[i + 1].in_h != oh || blocks[i + 1].in_w != ow || blocks[i + 1].in_c != s->out_c))
+      return fail(SOUFFLE_ERR_SHAPE, "block %d does not take what block %d produces (%d x %d x %d)", i + 1, i, oh, ow, s->out_c);
+    p->e[i] = off;
+    if (s->expand_w) off += round_up((size_t)s->in_h * s->in_w * s->expand_c * 2, 256);
+    p->d[i] = off;
+    off += round_up((size_t)oh * ow * s->expand_c * 2, 256);
+    p->out[i] = off;
+    if (i + 1 < n) off += round_up((size_t)oh * ow * s->out_c * 2, 256);
+    p->part[i] = off;
+    off += round_up((size_t)1024 * PART_LD * 4, 256);          // up to 1024 workgroups
+  }
+  p->total = off;
+  return SOUFFLE_OK;
+}
+
+static void fill_block(Block *b, const souffle_mbconv_block *s) {
+  b->H = s->in_h; b->W = s->in_w;
+  b->Ho = out_extent(s->in_h, s->kernel, s->stride); b->Wo = out_extent(s->in_w, s->kernel, s->stride);
+  b->Cin = s->in_c; b->Cexp = s->expand_c; b->Cout = s->out_c; b->k = s->kernel; b->stride = s->stride; b->R = s->se_c;
+  b->has_expand = s->expand_w != nullptr; b->has_shortcut = s->has_shortcut != 0;
+  b->w_exp = static_cast<const half_t *>(s->expand_w); b->w_dw = static_cast<const half_t *>(s->dw_w);
+  b->w_red = static_cast<const half_t *>(s->se_reduce_w); b->w_se = static_cast<const half_t *>(s->se_expand_w);
+  b->w_proj = static_cast<const half_t *>(s->project_w);
+  b->s_exp = s->expand_scale; b->b_exp = s->expand_shift; b->s_dw = s->dw_scale; b->b_dw = s->dw_shift;
+  b->b_red = s->se_reduce_b; b->b_se = s->se_expand_b; b->s_proj = s->project_scale; b->b_proj = s->project_shift;
+}
+
+}  // namespace mbconv
+}  // namespace souffle
+
+using namespace souffle;
+
+extern "C" size_t souffle_mbconv_workspace_bytes(const souffle_mbconv_block *blocks, int num_blocks) {
+  static thread_local mbconv::Plan p;
+  if (mbconv::make_plan(blocks, num_blocks, &p)) return 0;
+  return p.total;
+}
+
+extern "C" int souffle_mbconv_stack(const souffle_mbconv_block *blocks, int num_blocks, const void *x, void *y, int fused,
+                                    void *ws, size_t ws_bytes, souffle_stream_t stream) {
+  static thread_local mbconv::Plan p;
+  if (int rc = mbconv::make_plan(blocks, num_blocks, &p)) return rc;
+  if (!x || !y) return fail(SOUFFLE_ERR_NULL, "x and y must not be NULL");
+  if (!aligned16(x) || !aligned16(y)) return fail(SOUFFLE_ERR_ALIGN, "x and y must be 16-byte aligned");
+  if (!ws || ws_bytes < p.total) return fail(SOUFFLE_ERR_WORKSPACE, "workspace missing or too small: need %zu bytes", p.total);
+  if (!aligned16(ws)) return fail(SOUFFLE_ERR_ALIGN, "workspace must be 16-byte aligned");
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  if (df.num_cus > 1024) return fail(SOUFFLE_ERR_DEVICE, "more than 1024 compute units");
+  char *base = static_cast<char *>(ws);
+  const hipStream_t st = static_cast<hipStream_t>(stream);
+  for (int first = 0; first < num_blocks; first += mbconv::MAX_BLOCKS) {
+    const int n = num_blocks - first < mbconv::MAX_BLOCKS ? num_blocks - first : mbconv::MAX_BLOCKS;
+    mbconv::Args a;
+    a.nblk = n; a.pad = 0;
+    a.ctl = static_cast<unsigned *>(ws);
+    for (int i = 0; i < n; ++i) {
+      const int gi = first + i;
+      mbconv::Block *b = a.blk + i;
+      mbconv::fill_block(b, blocks + gi);
+      b->in = gi == 0 ? static_cast<const half_t *>(x) : reinterpret_cast<const half_t *>(base + p.out[gi - 1]);
+      b->e = reinterpret_cast<half_t *>(base + p.e[gi]);
+      b->d = reinterpret_cast<half_t *>(base + p.d[gi]);
+      b->out = gi + 1 == num_blocks ? static_cast<half_t *>(y) : reinterpret_cast<half_t *>(base + p.out[gi]);
+      b->part = reinterpret_cast<float *>(base + p.part[gi]);
+    }
+    void *args[] = {&a};
+    if (fused) {
+      a.stage_begin = 0; a.stage_end = 3 * n;
+      if (int rc = launch_persistent((const void *)mbconv::k_mbconv, df.num_cus, 256, args, 0, st)) return rc;
+    } else {
+      for (int s = 0; s < 3 * n; ++s) {
+        if (s % 3 == 0 && !a.blk[s / 3].has_expand) continue;
+        a.stage_begin = s; a.stage_end = s + 1;
+        if (int rc = launch_persistent((const void *)mbconv::k_mbconv, df.num_cus, 256, args, 0, st)) return rc;
+      }
+    }
+  }
+  return SOUFFLE_OK;
+}
+
+extern "C" int souffle_pointwise_conv2d_bn(const void *x, const void *w, const float *scale, const float *shift, const float *gate,
+                                           const void *shortcut, void *y, int pixels, int in_c, int out_c, int act,
+                                           souffle_stream_t stream) {
+  if (!x || !w || !y) return fail(SOUFFLE_ERR_NULL, "x, w and y must not be NULL");
+  if (pixels <= 0 || in_c <= 0 || out_c <= 0 || in_c % 8 || out_c % 8)
+    return fail(SOUFFLE_ERR_SHAPE, "pixels must be positive, in_c and out_c positive multiples of 8 (got %d, %d, %d)", pixels, in_c, out_c);
+  if (gate && in_c > mbconv::MAX_C) return fail(SOUFFLE_ERR_SHAPE, "a gated operand needs in_c <= %d (got %d)", mbconv::MAX_C, in_c);
+  if ((long long)pixels * in_c >= (1ll << 29) || (long long)pixels * out_c >= (1ll << 29))
+    return fail(SOUFFLE_ERR_SHAPE, "tensors of 2^29 elements or more are not supported");
+  if (act != SOUFFLE_MB_NONE && act != SOUFFLE_MB_SWISH) return fail(SOUFFLE_ERR_SHAPE, "unknown activation %d", act);
+  if (!aligned16(x) || !aligned16(w) || !aligned16(y) || !aligned16(scale) || !aligned16(shift) || !aligned16(shortcut))
+    return fail(SOUFFLE_ERR_ALIGN, "tensors must be 16-byte aligned");
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  mbconv::PwArgs a{static_cast<const half_t *>(x), static_cast<const half_t *>(w), static_cast<const half_t *>(shortcut), scale, shift,
+                   gate, static_cast<half_t *>(y), pixels, in_c, out_c, act};
+  // few tiles: a workgroup per tile (its waves split K); many: a wave per tile
+  const long long units = (long long)((pixels + 15) / 16) * ((out_c + 15) / 16);
+  const int grid = units <= df.num_cus ? (int)units : (int)(units / 4 + 1 < df.num_cus * 4 ? units / 4 + 1 : df.num_cus * 4);
+  hipLaunchKernelGGL(mbconv::k_pointwise, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+  SOUFFLE_HIP_TRY(hipGetLastError());
+  return SOUFFLE_OK;
+}
+
+extern "C" int souffle_depthwise_conv2d_bn_swish(const void *x, const void *w, const float *scale, const float *shift, void *y,
+                                                 int in_h, int in_w, int channels, int kernel, int stride,
+                                                 souffle_stream_t stream) {
+  if (!x || !w || !y) return fail(SOUFFLE_ERR_NULL, "x, w and y must not be NULL");
+  if (in_h <= 0 || in_w <= 0 || channels <= 0 || channels % 8 || channels > mbconv::MAX_C)
+    return fail(SOUFFLE_ERR_SHAPE, "in_h, in_w positive and channels a positive multiple of 8, at most %d (got %d, %d, %d)",
+                mbconv::MAX_C, in_h, in_w, channels);
+  if (kernel != 3 && kernel != 5) return fail(SOUFFLE_ERR_SHAPE, "kernel must be 3 or 5 (got %d)", kernel);
+  if (stride != 1 && stride != 2) return fail(SOUFFLE_ERR_SHAPE, "stride must be 1 or 2 (got %d)", stride);
+  if ((long long)in_h * in_w * channels >= (1ll << 29)) return fail(SOUFFLE_ERR_SHAPE, "tensors of 2^29 elements or more are not supported");
+  if (!aligned16(x) || !aligned16(w) || !aligned16(y)) return fail(SOUFFLE_ERR_ALIGN, "tensors must be 16-byte aligned");
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  mbconv::Block b{};
+  b.H = in_h; b.W = in_w; b.Ho = mbconv::out_extent(in_h, kernel, stride); b.Wo = mbconv::out_extent(in_w, kernel, stride);
+  b.Cin = b.Cexp = channels; b.k = kernel; b.stride = stride; b.R = 0; b.has_expand = 0;
+  b.w_dw = static_cast<const half_t *>(w); b.s_dw = scale; b.b_dw = shift;
+  b.in = static_cast<const half_t *>(x); b.d = static_cast<half_t *>(y);
+  const int P = 256 / (channels / 8), groups = (b.Ho * b.Wo + P - 1) / P;
+  const int grid = groups < df.num_cus * 4 ? groups : df.num_cus * 4;
+  hipLaunchKernelGGL(mbconv::k_depthwise, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), b);
+  SOUFFLE_HIP_TRY(hipGetLastError());
+  return SOUFFLE_OK;
+}

@@ -1,7 +1,7 @@
 """ctypes view of libsouffle_hip.so (the C ABI declared in include/souffle_hip.h).
 
 The binding modules in this directory (bert_binding, lstm_binding,
-swin_transformer_binding, swin_trans_fc2, efficientnet_se_module_binding) are thin
+swin_transformer_binding, swin_trans_fc2, efficientnet_se_module_binding, efficientnet_binding) are thin
 wrappers over this module; torch is used for device memory and streams only.
 There is no CPU or eager fallback: if the library is missing, loading fails.
 """
@@ -53,6 +53,16 @@ class SwinBlockW(C.Structure):
     _fields_ = [(n, C.c_void_p) for n in SWIN_W_FIELDS]
 
 
+MB_INT_FIELDS = ["in_h", "in_w", "in_c", "expand_c", "out_c", "kernel", "stride", "se_c", "has_shortcut"]
+MB_PTR_FIELDS = ["expand_w", "expand_scale", "expand_shift", "dw_w", "dw_scale", "dw_shift", "se_reduce_w", "se_reduce_b",
+                 "se_expand_w", "se_expand_b", "project_w", "project_scale", "project_shift"]
+MB_NONE, MB_SWISH = 0, 1
+
+
+class MbconvBlock(C.Structure):
+    _fields_ = [(n, C.c_int) for n in MB_INT_FIELDS] + [(n, C.c_void_p) for n in MB_PTR_FIELDS]
+
+
 class DevInfo(C.Structure):
     _fields_ = [("num_cus", C.c_int), ("lds_bytes_per_cu", C.c_int), ("clock_khz", C.c_int),
                 ("mem_clock_khz", C.c_int), ("mem_bus_bits", C.c_int), ("l2_bytes", C.c_int),
@@ -98,6 +108,13 @@ SIGNATURES = {
     "souffle_se_module_fused": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                           C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t,
                                           C.c_void_p]),
+    "souffle_mbconv_workspace_bytes": (C.c_size_t, [C.POINTER(MbconvBlock), C.c_int]),
+    "souffle_mbconv_stack": (C.c_int, [C.POINTER(MbconvBlock), C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
+                                       C.c_size_t, C.c_void_p]),
+    "souffle_pointwise_conv2d_bn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                              C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+    "souffle_depthwise_conv2d_bn_swish": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                                    C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]),
     "souffle_bench_us": (C.c_int, [BENCH_FN, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
                                    C.POINTER(C.c_double), C.POINTER(C.c_double)]),
 }

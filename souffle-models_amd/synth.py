@@ -117,3 +117,66 @@ def swin_block_weights(config_id=3, block=0, C=128, heads=4, window=7, mlp_ratio
 
 def swin_input(config_id=3, tokens=56 * 56, C=128):
     return f16(normal(seed_of(config_id, 0), (tokens, C), 1.0))
+
+
+# --------------------------------------------------------- EfficientNet ----
+# (kernel, stride, in_c, out_c, expand_ratio, repeats) of EfficientNet-B0's seven stages; the
+# reference builds the same list from efficientnet_pytorch's block arguments
+# (python/models/efficientnet/tvm_efficientnet.py:138-158).  SE ratio 0.25 of the block input.
+EFFICIENTNET_B0_STAGES = [(3, 1, 32, 16, 1, 1), (3, 2, 16, 24, 6, 2), (5, 2, 24, 40, 6, 2), (3, 2, 40, 80, 6, 3),
+                          (5, 1, 80, 112, 6, 3), (5, 2, 112, 192, 6, 4), (3, 1, 192, 320, 6, 1)]
+
+
+def mbconv_block_shapes(stages=EFFICIENTNET_B0_STAGES, image=112):
+    """The integer fields of every MBConv block of the stack, in order (the stem has already
+    halved a 224x224 image to `image`)."""
+    out, h = [], image
+    for kernel, stride, cin, cout, ratio, repeats in stages:
+        for r in range(repeats):
+            s, ci = (stride, cin) if r == 0 else (1, cout)
+            out.append({"in_h": h, "in_w": h, "in_c": ci, "expand_c": ci * ratio, "out_c": cout, "kernel": kernel,
+                        "stride": s, "se_c": max(1, int(ci * 0.25)), "has_shortcut": int(s == 1 and ci == cout),
+                        "has_expand": ratio != 1})
+            h = (h - 1) // s + 1
+    return out
+
+
+def mbconv_block_weights(shape, config_id=4, block=0, in_rms=1.0):
+    """fp16 N(0,0.02) convolution weights and fp32 folded batch-norm scale/shift of one block.
+    The folded scales are about those a batch norm would have on this data (they undo the 0.02
+    of the weights, the fan-in and the expected magnitude `in_rms` of the block input), so
+    activations stay of order one through the stack."""
+    t, b = block * 16, dict(shape)
+    ci, ce, co, k, r = b["in_c"], b["expand_c"], b["out_c"], b["kernel"], b["se_c"]
+
+    def fold(idx, n, fan_in, rms_in):
+        u = uniform(seed_of(config_id, t + idx), (n,), 0.75, 1.25)
+        return (u / (0.02 * np.sqrt(fan_in) * rms_in)).astype(np.float32), \
+            normal(seed_of(config_id, t + idx + 1), (n,), 0.1).astype(np.float32)
+
+    if b.pop("has_expand"):
+        b["expand_w"] = f16(normal(seed_of(config_id, t + 1), (ce, ci), 0.02))
+        b["expand_scale"], b["expand_shift"] = fold(2, ce, ci, in_rms)
+    else:
+        b["expand_w"] = b["expand_scale"] = b["expand_shift"] = None
+    b["dw_w"] = f16(normal(seed_of(config_id, t + 4), (k, k, ce), 0.02))
+    b["dw_scale"], b["dw_shift"] = fold(5, ce, k * k, 0.6)
+    b["se_reduce_w"] = f16(normal(seed_of(config_id, t + 7), (r, ce), 0.02))
+    b["se_reduce_b"] = normal(seed_of(config_id, t + 8), (r,), 0.1).astype(np.float32)
+    b["se_expand_w"] = f16(normal(seed_of(config_id, t + 9), (ce, r), 0.02))
+    b["se_expand_b"] = normal(seed_of(config_id, t + 10), (ce,), 0.5).astype(np.float32)
+    b["project_w"] = f16(normal(seed_of(config_id, t + 11), (co, ce), 0.02))
+    b["project_scale"], b["project_shift"] = fold(12, co, ce, 0.52)
+    return b
+
+
+def mbconv_stack_weights(config_id=4, stages=EFFICIENTNET_B0_STAGES, image=112):
+    out, rms = [], 1.0
+    for i, s in enumerate(mbconv_block_shapes(stages, image)):
+        out.append(mbconv_block_weights(s, config_id, i, rms))
+        rms = float(np.sqrt(1.0 + rms * rms)) if s["has_shortcut"] else 1.0   # the shortcut adds the input back
+    return out
+
+
+def mbconv_input(config_id=4, pixels=112 * 112, channels=32):
+    return f16(normal(seed_of(config_id, 0), (pixels, channels), 1.0))
