@@ -1,4 +1,4 @@
-"""Secondary bench workloads selected with bench.py --workload {lstm,swin,se,layer_stages}.
+"""Secondary bench workloads selected with bench.py --workload {lstm,swin,se,mbconv}.
 Each prints the same JSON shape as the default workload."""
 import os
 import sys
@@ -128,7 +128,60 @@ def bench_se(args):
                  roof, {"per_shape": rows, "reference_a100_sum_us": sum(a100)})
 
 
+def bench_mbconv(args):
+    import numpy as np
+    import torch
+    import efficientnet_binding as eb
+    import synth
+    from bench import time_steps
+    blocks = synth.mbconv_stack_weights()
+    x = synth.mbconv_input()
+
+    def up(v):
+        return torch.from_numpy(v).cuda() if isinstance(v, np.ndarray) else v
+    stack = eb.MBConvStack([{k: up(v) for k, v in b.items()} for b in blocks])
+    dx = torch.from_numpy(x).cuda()
+    y = stack(dx).float().cpu().numpy()
+    res_cpu = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle
+        thr = _threads()
+        ref = oracle.mbconv_stack(x, blocks, threads=thr)
+        dd = np.abs(y - ref)
+        if not (dd.max() <= 2e-2 and dd.mean() <= 2e-3):
+            print("PARITY FAILURE (mbconv): %g %g" % (dd.max(), dd.mean()), file=sys.stderr)
+            sys.exit(1)
+        us, n = _cpu_time(lambda: oracle.mbconv_stack(x, blocks, threads=thr), min(args.cpu_seconds, 8.0))
+        res_cpu = {"value": us, "unit": "us", "cores": thr, "kind": "port",
+                   "sample": "%d passes of the 16-block stack through oracle/mbconv_oracle.c (OpenMP fp32)" % n}
+    wall_u, ev_u = time_steps(lambda i: stack(dx, fused=False), max(10, args.steps // 4), args.warmup)
+    wall, ev = time_steps(lambda i: stack(dx), args.steps, args.warmup)
+    # algorithmic bytes: every weight tensor once, the input image and the result
+    wbytes = sum(v.nbytes for b in blocks for v in b.values() if isinstance(v, np.ndarray))
+    bytes_alg = wbytes + x.nbytes + y.size * 2
+    flops = 0.0
+    for b in blocks:
+        hw, oh = b["in_h"] * b["in_w"], ((b["in_h"] - 1) // b["stride"] + 1) ** 2
+        flops += 2.0 * hw * b["in_c"] * b["expand_c"] * (b["expand_w"] is not None) + 2.0 * oh * b["kernel"] ** 2 * b["expand_c"] + \
+            2.0 * oh * b["expand_c"] * b["out_c"]
+    ach = bytes_alg / (ev * 1e-3) / 1e9
+    stages = sum(3 if b["expand_w"] is not None else 2 for b in blocks)
+    roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
+            "kernel": "k_mbconv", "algorithmic_bytes_per_launch": bytes_alg, "algorithmic_flops_per_launch": flops,
+            "avg_launch_us": ev * 1e3,
+            "note": "%d dependent stages bound the latency, not the %.1f MB of weights and activations" % (stages, bytes_alg / 1e6)}
+    res = _base("mbconv_stack_latency_us", wall * 1e3, args,
+                "EfficientNet-B0 MBConv stack (16 blocks), 112x112x32 -> 7x7x320, batch 1, fp16 (BASELINE configs[4])", "f16", roof,
+                {"unfused_per_op_us": ev_u * 1e3, "stages": stages, "us_per_stage": ev * 1e3 / stages})
+    if res_cpu:
+        res["cpu_baseline"] = res_cpu
+    return res
+
+
 def run(args):
+    if args.workload == "mbconv":
+        return bench_mbconv(args)
     if args.workload == "lstm":
         return bench_lstm(args)
     if args.workload == "swin":

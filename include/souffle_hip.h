@@ -255,7 +255,7 @@ typedef struct {
   const float *dw_scale, *dw_shift;
   const void *se_reduce_w;                 /* fp16 [se_c][expand_c] */
   const float *se_reduce_b;                /* [se_c], nullable */
-  const void *se_expand_w;                 /* fp16 [expand_c][se_c] */
+  const void *se_expand_w;                 /* fp16 [se_c][expand_c]: input-major, as se_module_pointwise_conv declares it */
   const float *se_expand_b;                /* [expand_c], nullable */
   const void *project_w;                   /* fp16 [out_c][expand_c] */
   const float *project_scale, *project_shift;

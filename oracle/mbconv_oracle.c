@@ -75,7 +75,9 @@ int oracle_depthwise_conv_f32(const float *x, const float *w, const float *scale
   return 0;
 }
 
-/* gate[c] = sigmoid(b_e[c] + sum_j W_e[c][j] * swish(b_r[j] + sum_c' W_r[j][c'] * mean_p X[p][c']))
+/* w_reduce [squeezed][channels] (output-major), w_expand [squeezed][channels] (input-major, the layout
+ * se_module_pointwise_conv declares).
+ * gate[c] = sigmoid(b_e[c] + sum_j W_e[j][c] * swish(b_r[j] + sum_c' W_r[j][c'] * mean_p X[p][c']))
  * (reduce_mean efficientnet.py:131-141; se_module_pointwise_conv :270-282 twice, swish between;
  *  fused_pointwise_conv_bias_add_sigmoid :413-424 for the second layer and its sigmoid). */
 int oracle_se_gate_f32(const float *x, const float *w_reduce, const float *b_reduce, const float *w_expand,
@@ -93,7 +95,7 @@ int oracle_se_gate_f32(const float *x, const float *w_reduce, const float *b_red
   }
   for (int c = 0; c < channels; ++c) {
     float a = b_expand ? b_expand[c] : 0.f;
-    for (int j = 0; j < squeezed; ++j) a += w_expand[(size_t)c * squeezed + j] * r[j];
+    for (int j = 0; j < squeezed; ++j) a += w_expand[(size_t)j * channels + c] * r[j];
     gate[c] = 1.0f / (1.0f + expf(-a));
   }
   free(m); free(r);

@@ -151,7 +151,7 @@ typedef struct {
   const float *expand_w, *expand_scale, *expand_shift;   /* [expand_c][in_c]; NULL = no expansion conv */
   const float *dw_w, *dw_scale, *dw_shift;               /* [kernel][kernel][expand_c] */
   const float *se_reduce_w, *se_reduce_b;                /* [se_c][expand_c], [se_c] */
-  const float *se_expand_w, *se_expand_b;                /* [expand_c][se_c], [expand_c] */
+  const float *se_expand_w, *se_expand_b;                /* [se_c][expand_c] (input-major), [expand_c] */
   const float *project_w, *project_scale, *project_shift;/* [out_c][expand_c] */
 } oracle_mbconv_block;
 /* x [pixels][in_c], w [out_c][in_c]; scale/shift/gate/shortcut nullable. */

@@ -27,11 +27,21 @@
 #include "common.hpp"
 #include "host_util.hpp"
 
+#ifdef SOUFFLE_STAGE_MARKS
+#define MB_MARK(tb, id) do { if (tb) { __builtin_amdgcn_s_waitcnt(0); trace_mark(*(tb), (id)); } } while (0)
+#else
+#define MB_MARK(tb, id) do { } while (0)
+#endif
+
 namespace souffle {
 namespace mbconv {
 
 constexpr int MAX_BLOCKS = 16;   // per launch (the descriptors travel as kernel arguments)
 constexpr int MAX_C = 2048, MAX_R = 64, PART_LD = 64;
+#ifndef MBCONV_COH_LOADS
+#define MBCONV_COH_LOADS 1
+#endif
+constexpr bool kCohLoads = MBCONV_COH_LOADS != 0;
 
 struct Block {
   int H, W, Ho, Wo, Cin, Cexp, Cout, k, stride, R, has_expand, has_shortcut;
@@ -43,8 +53,9 @@ struct Block {
 };
 
 struct Args {
-  int nblk, stage_begin, stage_end, pad;
+  int nblk, stage_begin, stage_end, trace_cap;
   unsigned *ctl;
+  unsigned long long *trace;     // optional stage stamps (souffle_set_stage_trace)
   Block blk[MAX_BLOCKS];
 };
 static_assert(sizeof(Args) <= 4096, "kernel argument segment");
@@ -52,38 +63,51 @@ static_assert(sizeof(Args) <= 4096, "kernel argument segment");
 __device__ __forceinline__ float swish(float v) { return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
 __device__ __forceinline__ float sigmoid(float v) { return __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
 
-// Partial dot products of one 16 x 16 tile: MFMA k-steps first, first + stride, ... (32 k-values
-// each) of rows xbase/wbase.  UNROLL steps are loaded together before their MFMAs are issued, so
-// that many 16-byte loads per operand are in flight per wave; steps past K load nothing and
-// multiply zeros.  The trip count is wave-uniform.
-template <bool GATE, bool COH, int UNROLL>
-__device__ __forceinline__ f4 tile_dot(const half_t *X, int xbase, const half_t *__restrict__ Wt, int wbase, bool wok, int K,
-                                       int first, int stride, const float *gate, int g) {
-  f4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int s0 = first; s0 * 32 < K; s0 += UNROLL * stride) {
-    u4 xv[UNROLL], wv[UNROLL];
+// Operands of NS MFMA k-steps (32 k-values each) of one 16 x 16 tile: steps first, first + stride, ...
+// of rows xbase / wbase, requested together so that 2*NS 16-byte loads are in flight per wave.
+// Steps past K request element 0 and are zeroed.
+template <bool COH, int NS>
+__device__ __forceinline__ void tile_load(u4 (&xv)[NS], u4 (&wv)[NS], const half_t *X, int xbase, const half_t *__restrict__ Wt,
+                                          int wbase, bool wok, int K, int first, int stride, int g) {
 #pragma unroll
-    for (int i = 0; i < UNROLL; ++i) {
-      const int kk = (s0 + i * stride) * 32 + g * 8;
-      const bool ok = kk < K;
-      const int ks = ok ? kk : 0;
-      xv[i] = ld16<COH>(X, (xbase + ks) * 2);
+  for (int i = 0; i < NS; ++i) {
+    const int k0 = (first + i * stride) * 32, kk = k0 + g * 8;
+    const bool ok = kk < K;
+    const int ks = ok ? kk : 0;
+    xv[i] = wv[i] = u4{0u, 0u, 0u, 0u};
+    if (k0 < K) {                        // wave-uniform: whole steps past K cost nothing
+      xv[i] = ld16<COH && kCohLoads>(X, (xbase + ks) * 2);
       wv[i] = *reinterpret_cast<const u4 *>(Wt + wbase + ks);
       if (!ok) xv[i] = u4{0u, 0u, 0u, 0u};
       if (!ok || !wok) wv[i] = u4{0u, 0u, 0u, 0u};
     }
+  }
+}
+template <bool GATE, int NS>
+__device__ __forceinline__ f4 tile_mma(f4 acc, u4 (&xv)[NS], u4 (&wv)[NS], int K, int first, int stride, const float *gate, int g) {
 #pragma unroll
-    for (int i = 0; i < UNROLL; ++i) {
-      if constexpr (GATE) {
-        const int kk = (s0 + i * stride) * 32 + g * 8, ks = kk < K ? kk : 0;
-        const f4 g0 = *reinterpret_cast<const f4 *>(gate + ks), g1 = *reinterpret_cast<const f4 *>(gate + ks + 4);
-        const h8 x = as_h8(xv[i]);
-        xv[i] = as_u4(h8{(half_t)((float)x[0] * g0[0]), (half_t)((float)x[1] * g0[1]), (half_t)((float)x[2] * g0[2]),
-                         (half_t)((float)x[3] * g0[3]), (half_t)((float)x[4] * g1[0]), (half_t)((float)x[5] * g1[1]),
-                         (half_t)((float)x[6] * g1[2]), (half_t)((float)x[7] * g1[3])});
-      }
-      acc = mfma_16x16x32(as_h8(wv[i]), as_h8(xv[i]), acc);
+  for (int i = 0; i < NS; ++i) {
+    if ((first + i * stride) * 32 >= K) break;     // wave-uniform
+    if constexpr (GATE) {
+      const int kk = (first + i * stride) * 32 + g * 8, ks = kk < K ? kk : 0;
+      const f4 g0 = *reinterpret_cast<const f4 *>(gate + ks), g1 = *reinterpret_cast<const f4 *>(gate + ks + 4);
+      const h8 x = as_h8(xv[i]);
+      xv[i] = as_u4(h8{(half_t)((float)x[0] * g0[0]), (half_t)((float)x[1] * g0[1]), (half_t)((float)x[2] * g0[2]),
+                       (half_t)((float)x[3] * g0[3]), (half_t)((float)x[4] * g1[0]), (half_t)((float)x[5] * g1[1]),
+                       (half_t)((float)x[6] * g1[2]), (half_t)((float)x[7] * g1[3])});
     }
+    acc = mfma_16x16x32(as_h8(wv[i]), as_h8(xv[i]), acc);
+  }
+  return acc;
+}
+// All remaining k-steps from `first` on, NS at a time.  The trip count is wave-uniform.
+template <bool GATE, bool COH, int NS>
+__device__ __forceinline__ f4 tile_dot(f4 acc, const half_t *X, int xbase, const half_t *__restrict__ Wt, int wbase, bool wok, int K,
+                                       int first, int stride, const float *gate, int g) {
+  for (int s0 = first; s0 * 32 < K; s0 += NS * stride) {
+    u4 xv[NS], wv[NS];
+    tile_load<COH, NS>(xv, wv, X, xbase, Wt, wbase, wok, K, s0, stride, g);
+    acc = tile_mma<GATE, NS>(acc, xv, wv, K, s0, stride, gate, g);
   }
   return acc;
 }
@@ -93,14 +117,19 @@ __device__ __forceinline__ f4 tile_dot(const half_t *X, int xbase, const half_t 
 // result granules are all-or-nothing at the edges.  With more tiles than workgroups a wave owns
 // a tile; otherwise (few pixels, many input channels: the late blocks) a workgroup owns a tile,
 // its four waves take every fourth k-step and the partial tiles are summed through `red`.
+// mid() is called once by every thread of the workgroup after the operands of the first tile
+// have been requested and before they are used: whatever else the stage has to do first (the
+// squeeze-excite gate) runs while those loads travel.  It may synchronise the workgroup.
 // COH: X and shortcut were written earlier in this launch by other workgroups.
-template <bool GATE, bool COH>
+constexpr int kFirstSteps = 12;
+template <bool GATE, bool COH, class Mid>
 __device__ __forceinline__ void pointwise(const half_t *X, int M, int K, int N, const half_t *__restrict__ Wt,
                                           const float *__restrict__ scale, const float *__restrict__ shift, bool act,
-                                          const float *gate, const half_t *shortcut, half_t *Y, float *red) {
+                                          const float *gate, const half_t *shortcut, half_t *Y, float *red, Mid mid) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
   const int nt_n = (N + 15) >> 4, units = ((M + 15) >> 4) * nt_n;
   const bool split = units <= (int)gridDim.x;
+  const int stride = split ? 4 : 1, first = split ? wave : 0;
   auto epilogue = [&](int mt, int nt, f4 acc) {
     const int row = mt * 16 + l16, col = nt * 16 + g * 4;
     if (row < M && col < N) {
@@ -110,87 +139,212 @@ __device__ __forceinline__ void pointwise(const half_t *X, int M, int K, int N, 
       f4 v = acc * sc + sh;
       if (act) v = f4{swish(v[0]), swish(v[1]), swish(v[2]), swish(v[3])};
       if (shortcut) {
-        const h4 s = as_h4(ld8<COH>(shortcut, (row * N + col) * 2));
+        const h4 s = as_h4(ld8<COH && kCohLoads>(shortcut, (row * N + col) * 2));
         v += f4{(float)s[0], (float)s[1], (float)s[2], (float)s[3]};
       }
       st8<COH>(Y, (row * N + col) * 2, pack_h4(v));
     }
   };
-  if (split) {
-    const int u = blockIdx.x;
-    if (u < units) {
-      const int mt = u / nt_n, nt = u - mt * nt_n, wrow = nt * 16 + l16;
-      const bool wok = wrow < N;
-      const f4 part = tile_dot<GATE, COH, 12>(X, min(mt * 16 + l16, M - 1) * K, Wt, (wok ? wrow : N - 1) * K, wok, K, wave, 4, gate, g);
-      *reinterpret_cast<f4 *>(red + tid * 4) = part;
-      __syncthreads();
-      if (wave == 0) {
-        f4 acc = part;
+  int u = split ? (int)blockIdx.x : (int)blockIdx.x * 4 + wave;
+  {
+    const bool has = u < units;          // workgroup-uniform when split
+    const int uu = has ? u : 0, mt = uu / nt_n, nt = uu - mt * nt_n, wrow = nt * 16 + l16;
+    const bool wok = wrow < N;
+    const int xbase = min(mt * 16 + l16, M - 1) * K, wbase = (wok ? wrow : N - 1) * K;
+    u4 xv[kFirstSteps], wv[kFirstSteps];
+    if (has) tile_load<COH, kFirstSteps>(xv, wv, X, xbase, Wt, wbase, wok, K, first, stride, g);
+    mid();
+    if (has) {
+      f4 acc = tile_mma<GATE, kFirstSteps>(f4{0.f, 0.f, 0.f, 0.f}, xv, wv, K, first, stride, gate, g);
+      acc = tile_dot<GATE, COH, kFirstSteps>(acc, X, xbase, Wt, wbase, wok, K, first + kFirstSteps * stride, stride, gate, g);
+      if (split) {
+        *reinterpret_cast<f4 *>(red + tid * 4) = acc;
+        __syncthreads();
+        if (wave == 0) {
 #pragma unroll
-        for (int w = 1; w < 4; ++w) acc += *reinterpret_cast<const f4 *>(red + (w * 64 + lane) * 4);
+          for (int w = 1; w < 4; ++w) acc += *reinterpret_cast<const f4 *>(red + (w * 64 + lane) * 4);
+          epilogue(mt, nt, acc);
+        }
+      } else {
         epilogue(mt, nt, acc);
       }
     }
-  } else {
-    for (int u = blockIdx.x * 4 + wave; u < units; u += gridDim.x * 4) {
+  }
+  if (!split) {
+    for (u += gridDim.x * 4; u < units; u += gridDim.x * 4) {
       const int mt = u / nt_n, nt = u - mt * nt_n, wrow = nt * 16 + l16;
       const bool wok = wrow < N;
-      const f4 acc = tile_dot<GATE, COH, 6>(X, min(mt * 16 + l16, M - 1) * K, Wt, (wok ? wrow : N - 1) * K, wok, K, 0, 1, gate, g);
+      const f4 acc = tile_dot<GATE, COH, 6>(f4{0.f, 0.f, 0.f, 0.f}, X, min(mt * 16 + l16, M - 1) * K, Wt, (wok ? wrow : N - 1) * K, wok, K,
+                                             0, 1, gate, g);
       epilogue(mt, nt, acc);
     }
   }
 }
 
-// D[ho][wo][c] = swish(bn(sum_ij X[ho*s - pad + i][wo*s - pad + j][c] * W[i][j][c])), pad = KS/2.
-// A thread owns 8 channels of one output pixel; G = C/8 neighbouring threads cover a pixel, so a
-// wave reads and writes whole contiguous runs of the NHWC tensors.  When the block has a
-// squeeze-excite module (R > 0) the thread also sums its outputs over its pixels; the workgroup
-// reduces those sums in a fixed order and writes W_r . sums, its share of the squeeze layer.
+// D[ho][wo][c] = swish(bn(sum_ij X[ho*s - pad + i][wo*s - pad + j][c] * W[i][j][c])), pad = KS/2, for the 8
+// channels of group cg at output pixel pix; returns the 8 fp32 results and stores them as fp16.
+// All taps and their weights are requested before the first is used (addresses clamped into the
+// image, taps outside it masked afterwards): one memory latency per pixel instead of one per tap.
 template <int KS, bool COH>
-__device__ __forceinline__ void depthwise(const Block &b, float *red, float *sums) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int C = b.Cexp, G = C >> 3, P = 256 / G;
-  const int slot = tid / G, cg = tid - slot * G;
-  const bool active = slot < P;
-  const int npix = b.Ho * b.Wo, groups = (npix + P - 1) / P;
-  const half_t *src = b.has_expand ? b.e : b.in;
+__device__ __forceinline__ void dw_pixel(const Block &b, const half_t *src, int pix, int cg, float (&v)[8]) {
   constexpr int pad = KS / 2;
-  float sc[8], sh[8], sum[8];
+  const int C = b.Cexp, ho = pix / b.Wo, wo = pix - ho * b.Wo;
+  u4 xv[KS * KS], wv[KS * KS];
+  unsigned inside = 0;
+#pragma unroll
+  for (int i = 0; i < KS; ++i) {
+    const int hi = ho * b.stride - pad + i, hc = min(max(hi, 0), b.H - 1);
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+      const int wi = wo * b.stride - pad + j, wc = min(max(wi, 0), b.W - 1);
+      xv[i * KS + j] = ld16<COH && kCohLoads>(src, ((hc * b.W + wc) * C + cg * 8) * 2);
+      if (hi == hc && wi == wc) inside |= 1u << (i * KS + j);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < KS * KS; ++t) wv[t] = *reinterpret_cast<const u4 *>(b.w_dw + t * C + cg * 8);
+  f4 sc0 = {1.f, 1.f, 1.f, 1.f}, sc1 = sc0, sh0 = {0.f, 0.f, 0.f, 0.f}, sh1 = sh0;
+  if (b.s_dw) { sc0 = *reinterpret_cast<const f4 *>(b.s_dw + cg * 8); sc1 = *reinterpret_cast<const f4 *>(b.s_dw + cg * 8 + 4); }
+  if (b.b_dw) { sh0 = *reinterpret_cast<const f4 *>(b.b_dw + cg * 8); sh1 = *reinterpret_cast<const f4 *>(b.b_dw + cg * 8 + 4); }
+  float acc[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) acc[q] = 0.f;
+#pragma unroll
+  for (int t = 0; t < KS * KS; ++t) {
+    const h8 w = as_h8(wv[t]);
+    const h8 x = as_h8((inside >> t) & 1u ? xv[t] : u4{0u, 0u, 0u, 0u});
+#pragma unroll
+    for (int q = 0; q < 8; ++q) acc[q] += (float)x[q] * (float)w[q];
+  }
+  h8 o;
 #pragma unroll
   for (int q = 0; q < 8; ++q) {
-    sc[q] = (active && b.s_dw) ? b.s_dw[cg * 8 + q] : 1.f;
-    sh[q] = (active && b.b_dw) ? b.b_dw[cg * 8 + q] : 0.f;
-    sum[q] = 0.f;
+    v[q] = swish(acc[q] * (q < 4 ? sc0[q & 3] : sc1[q & 3]) + (q < 4 ? sh0[q & 3] : sh1[q & 3]));
+    o[q] = (half_t)v[q];
   }
-  for (int grp = blockIdx.x; grp < groups; grp += gridDim.x) {
-    const int pix = grp * P + slot;
-    if (active && pix < npix) {
-      const int ho = pix / b.Wo, wo = pix - ho * b.Wo;
-      float acc[8];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) acc[q] = 0.f;
-#pragma unroll
-      for (int i = 0; i < KS; ++i) {
-        const int hi = ho * b.stride - pad + i;
-#pragma unroll
-        for (int j = 0; j < KS; ++j) {
-          const int wi = wo * b.stride - pad + j;
-          if (hi >= 0 && hi < b.H && wi >= 0 && wi < b.W) {
-            const h8 x = as_h8(ld16<COH>(src, ((hi * b.W + wi) * C + cg * 8) * 2));
-            const h8 w = as_h8(*reinterpret_cast<const u4 *>(b.w_dw + (i * KS + j) * C + cg * 8));
-#pragma unroll
-            for (int q = 0; q < 8; ++q) acc[q] += (float)x[q] * (float)w[q];
-          }
-        }
-      }
-      h8 o;
+  st16<COH>(b.d, (pix * C + cg * 8) * 2, as_u4(o));
+}
+
+// How the depthwise stage is dealt to workgroups, and how many of them write a row of squeeze partials.
+// Images of at most 256 output pixels: a workgroup owns whole channel groups (all pixels of up to 8
+// groups of 8 channels), so its channel sums are complete and its share of the squeeze layer needs
+// only its own columns of W_r.  Larger images: a workgroup owns runs of pixels (all channels), so
+// that waves read and write contiguous runs of the NHWC tensors.
+struct DwPlan {
+  bool by_channel;
+  int per_wg;        // channel groups per workgroup pass (by_channel) or pixels per pass
+  int passes;        // workgroup passes in total
+};
+__host__ __device__ __forceinline__ DwPlan dw_plan(const Block &b) {
+  const int npix = b.Ho * b.Wo, G = b.Cexp >> 3;
+  DwPlan p;
+  p.by_channel = npix <= 256;
+  if (p.by_channel) {
+    p.per_wg = 256 / npix < 8 ? 256 / npix : 8;
+    p.passes = (G + p.per_wg - 1) / p.per_wg;
+  } else {
+    p.per_wg = 256 / G;
+    p.passes = (npix + p.per_wg - 1) / p.per_wg;
+  }
+  return p;
+}
+
+template <int KS, bool COH>
+__device__ __forceinline__ void depthwise(const Block &b, float *red, float *sums, const GridBarrier *tb = nullptr) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int C = b.Cexp, G = C >> 3, npix = b.Ho * b.Wo;
+  const half_t *src = b.has_expand ? b.e : b.in;
+  const DwPlan plan = dw_plan(b);
+  if ((int)blockIdx.x >= plan.passes) return;
+  if (plan.by_channel) {
+    const int CGW = plan.per_wg, slot = tid / npix, pix = tid - slot * npix;
+    float pj = 0.f;                                  // thread j < R: this workgroup's share of squeeze row j
+    for (int set = blockIdx.x; set < plan.passes; set += gridDim.x) {
+      const int cg = set * CGW + slot;
+      const bool act = slot < CGW && cg < G;
+      // thread j requests its row of W_r for the set's channels before anything else
+      u4 wr[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
-        const float v = swish(acc[q] * sc[q] + sh[q]);
-        sum[q] += v;
-        o[q] = (half_t)v;
+        const bool ok = tid < b.R && q < CGW && set * CGW + q < G;
+        wr[q] = u4{0u, 0u, 0u, 0u};
+        if (b.R > 0) {                   // without a squeeze-excite module w_red may be NULL
+          wr[q] = *reinterpret_cast<const u4 *>(b.w_red + (ok ? tid * C + (set * CGW + q) * 8 : 0));
+          if (!ok) wr[q] = u4{0u, 0u, 0u, 0u};
+        }
       }
-      st16<COH>(b.d, (pix * C + cg * 8) * 2, as_u4(o));
+      float v[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) v[q] = 0.f;
+      MB_MARK(tb, 0);
+      if (act) dw_pixel<KS, COH>(b, src, pix, cg, v);
+      if (b.R > 0) {
+        // channel sums over the pixels: channel ch = slot*8 + q, NP threads per channel take every NP-th pixel
+        if (slot < CGW) {
+#pragma unroll
+          for (int q = 0; q < 8; ++q) red[(slot * 8 + q) * npix + pix] = v[q];        // < 8*CGW*npix <= 2048
+        }
+        __syncthreads();
+        const int nch = CGW * 8, NP = 256 / nch, ch = tid % nch, part = tid / nch;
+        MB_MARK(tb, 1);
+        if (part < NP) {
+          float t = 0.f;
+          for (int x = part; x < npix; x += NP) t += red[ch * npix + x];
+          sums[part * nch + ch] = t;                                                   // < 256
+        }
+        __syncthreads();
+        if (tid < nch) {
+          float t = 0.f;
+          for (int x = 0; x < NP; ++x) t += sums[x * nch + tid];
+          sums[256 + tid] = t;
+        }
+        __syncthreads();
+        MB_MARK(tb, 2);
+        if (tid < b.R) {
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            if (q < CGW) {
+              const h8 w = as_h8(wr[q]);
+              const f4 s0 = *reinterpret_cast<const f4 *>(sums + 256 + q * 8), s1 = *reinterpret_cast<const f4 *>(sums + 256 + q * 8 + 4);
+              pj += (float)w[0] * s0[0] + (float)w[1] * s0[1] + (float)w[2] * s0[2] + (float)w[3] * s0[3] +
+                    (float)w[4] * s1[0] + (float)w[5] * s1[1] + (float)w[6] * s1[2] + (float)w[7] * s1[3];
+            }
+          }
+        }
+        __syncthreads();
+      }
+    }
+    if (tid < b.R) st4<COH>(b.part, ((int)blockIdx.x * PART_LD + tid) * 4, __float_as_uint(pj));
+    MB_MARK(tb, 3);
+    return;
+  }
+  // pixel-major: thread (slot, cg) takes pixel grp*P + slot
+  const int P = plan.per_wg, slot = tid / G, cg = tid - slot * G;
+  const bool active = slot < P;
+  float sum[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) sum[q] = 0.f;
+  // rows wave, wave+4, wave+8, wave+12 of W_r are requested now and used after the pixels
+  u4 wr[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int j = wave + 4 * a, g8 = lane + 64 * m;
+      const bool ok = j < b.R && g8 < G;
+      wr[a][m] = u4{0u, 0u, 0u, 0u};
+      if (b.R > 0) {                     // without a squeeze-excite module w_red may be NULL
+        wr[a][m] = *reinterpret_cast<const u4 *>(b.w_red + (ok ? j * C + g8 * 8 : 0));
+        if (!ok) wr[a][m] = u4{0u, 0u, 0u, 0u};
+      }
+    }
+  for (int grp = blockIdx.x; grp < plan.passes; grp += gridDim.x) {
+    const int pix = grp * P + slot;
+    if (active && pix < npix) {
+      float v[8];
+      dw_pixel<KS, COH>(b, src, pix, cg, v);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) sum[q] += v[q];
     }
   }
   if (b.R <= 0) return;
@@ -205,66 +359,159 @@ __device__ __forceinline__ void depthwise(const Block &b, float *red, float *sum
     sums[c] = s;
   }
   __syncthreads();
-  if ((int)blockIdx.x < groups) {
-    for (int j = wave; j < b.R; j += 4) {
-      float s = 0.f;
-      for (int c = lane; c < C; c += 64) s += (float)b.w_red[j * C + c] * sums[c];
-      s = wave_sum(s);
-      if (lane == 0) st4<COH>(b.part, ((int)blockIdx.x * PART_LD + j) * 4, __float_as_uint(s));
+  for (int j0 = wave; j0 < b.R; j0 += 16) {
+    if (j0 != wave) {                                // further rows (R > 16): requested here
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          const int j = j0 + 4 * a, g8 = lane + 64 * m;
+          const bool ok = j < b.R && g8 < G;
+          wr[a][m] = *reinterpret_cast<const u4 *>(b.w_red + (ok ? j * C + g8 * 8 : 0));
+          if (!ok) wr[a][m] = u4{0u, 0u, 0u, 0u};
+        }
+    }
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int g8 = lane + 64 * m;
+      if (g8 < G) {
+        const f4 s0 = *reinterpret_cast<const f4 *>(sums + g8 * 8), s1 = *reinterpret_cast<const f4 *>(sums + g8 * 8 + 4);
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          const h8 w = as_h8(wr[a][m]);
+          s[a] += (float)w[0] * s0[0] + (float)w[1] * s0[1] + (float)w[2] * s0[2] + (float)w[3] * s0[3] +
+                  (float)w[4] * s1[0] + (float)w[5] * s1[1] + (float)w[6] * s1[2] + (float)w[7] * s1[3];
+        }
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const float t = wave_sum(s[a]);
+      if (lane == 0 && j0 + 4 * a < b.R) st4<COH>(b.part, ((int)blockIdx.x * PART_LD + j0 + 4 * a) * 4, __float_as_uint(t));
     }
   }
   __syncthreads();                 // red / sums are reused by the next stage
 }
 
-// gate[c] = sigmoid(b_e[c] + sum_j W_e[c][j] * swish(b_r[j] + (sum over workgroups of part[.][j]) / pixels)),
-// evaluated by every workgroup for itself, then the projection with the gate folded into its operand.
+// gate[c] = sigmoid(b_e[c] + sum_j W_e[j][c] * swish(b_r[j] + (sum over workgroups of part[.][j]) / pixels)),
+// evaluated by every workgroup that has a tile of the projection, while the operands of that tile
+// are already on their way; then the projection with the gate folded into its activation operand.
+constexpr int kGateRows = 24;      // rows of W_e a thread requests at a time
 template <bool COH>
-__device__ __forceinline__ void project(const Block &b, float *gate_s, float *r_s, float *red) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__device__ __forceinline__ void project(const Block &b, float *gate_s, float *r_s, float *red, const GridBarrier *tb = nullptr) {
+  const int tid = threadIdx.x;
   const int npix = b.Ho * b.Wo, C = b.Cexp;
   const half_t *shortcut = b.has_shortcut ? b.in : nullptr;
   if (b.R <= 0) {
-    pointwise<false, COH>(b.d, npix, C, b.Cout, b.w_proj, b.s_proj, b.b_proj, false, nullptr, shortcut, b.out, red);
+    pointwise<false, COH>(b.d, npix, C, b.Cout, b.w_proj, b.s_proj, b.b_proj, false, nullptr, shortcut, b.out, red, []() {});
     return;
   }
-  const int P = 256 / (C >> 3), groups = (npix + P - 1) / P, nact = min(groups, (int)gridDim.x);
-  for (int j = wave; j < b.R; j += 4) {
-    float s = 0.f;
-    for (int wg = lane; wg < nact; wg += 64) s += __uint_as_float(ld4<COH>(b.part, (wg * PART_LD + j) * 4));
-    s = wave_sum(s);
-    if (lane == 0) r_s[j] = swish(s / (float)npix + (b.b_red ? b.b_red[j] : 0.f));
+  {   // workgroups without a tile of the projection have nothing to do in this stage
+    const int units = ((npix + 15) >> 4) * ((b.Cout + 15) >> 4);
+    if ((int)blockIdx.x * (units <= (int)gridDim.x ? 1 : 4) >= units) return;
   }
-  __syncthreads();
-  for (int c = tid; c < C; c += 256) {
-    float s = b.b_se ? b.b_se[c] : 0.f;
-    for (int j = 0; j < b.R; ++j) s += (float)b.w_se[c * b.R + j] * r_s[j];
-    gate_s[c] = sigmoid(s);
-  }
-  __syncthreads();
-  pointwise<true, COH>(b.d, npix, C, b.Cout, b.w_proj, b.s_proj, b.b_proj, false, gate_s, shortcut, b.out, red);
+  auto gate = [&]() {
+    const int G = C >> 3, nact = min(dw_plan(b).passes, (int)gridDim.x);
+    const int JS = 256 / G, slice = tid / G, cg = tid - slice * G;
+    // requested up front: the first chunk of partial rows and this thread's first rows of W_e
+    const int R4 = (b.R + 3) >> 2, chunk_rows = 1024 / R4;
+    u4 pv[4], w[kGateRows];
+    auto load_partials = [&](int row0) {
+      const int ngran = min(chunk_rows, nact - row0) * R4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int idx = tid + 256 * i, r = idx / R4, q = idx - r * R4;
+        pv[i] = ld16<COH && kCohLoads>(b.part, idx < ngran ? ((row0 + r) * PART_LD + q * 4) * 4 : 0);
+      }
+    };
+    auto load_rows = [&](int j0) {
+#pragma unroll
+      for (int i = 0; i < kGateRows; ++i)
+        w[i] = *reinterpret_cast<const u4 *>(b.w_se + (slice < JS ? min(j0 + i * JS, b.R - 1) * C + cg * 8 : 0));
+    };
+    MB_MARK(tb, 0);
+    load_partials(0);
+    load_rows(slice);
+    MB_MARK(tb, 1);
+    // (1) the partial rows of all workgroups go through LDS, thread (quarter, j) sums every fourth row
+    //     of column j, the quarters are added in a fixed order
+    const int j = tid & 63, quarter = tid >> 6;
+    float accj = 0.f;
+    for (int row0 = 0; row0 < nact; row0 += chunk_rows) {
+      if (row0) load_partials(row0);
+      const int rows = min(chunk_rows, nact - row0), ngran = rows * R4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (tid + 256 * i < ngran) *reinterpret_cast<u4 *>(red + (tid + 256 * i) * 4) = pv[i];
+      __syncthreads();
+      if (j < b.R)
+        for (int r = quarter; r < rows; r += 4) accj += red[r * R4 * 4 + j];
+      __syncthreads();
+    }
+    gate_s[quarter * 64 + j] = accj;
+    __syncthreads();
+    if (tid < b.R) {
+      const float s = (gate_s[tid] + gate_s[64 + tid]) + (gate_s[128 + tid] + gate_s[192 + tid]);
+      r_s[tid] = swish(s / (float)npix + (b.b_red ? b.b_red[tid] : 0.f));
+    }
+    __syncthreads();
+    MB_MARK(tb, 2);
+    // (2) W_e . r with 16-byte loads: thread (slice, cg) takes 8 channels and every JS-th squeezed row
+    float g8[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) g8[q] = 0.f;
+    if (slice < JS) {
+      for (int j0 = slice; j0 < b.R; j0 += JS * kGateRows) {
+        if (j0 != slice) load_rows(j0);
+#pragma unroll
+        for (int i = 0; i < kGateRows; ++i) {
+          const int jj = j0 + i * JS;
+          const float rj = jj < b.R ? r_s[min(jj, MAX_R - 1)] : 0.f;
+          const h8 h = as_h8(w[i]);
+#pragma unroll
+          for (int q = 0; q < 8; ++q) g8[q] += (float)h[q] * rj;
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < 8; ++q) red[slice * C + cg * 8 + q] = g8[q];          // JS * C <= 2048
+    }
+    __syncthreads();
+    for (int c = tid; c < C; c += 256) {
+      float s = b.b_se ? b.b_se[c] : 0.f;
+      for (int sl = 0; sl < JS; ++sl) s += red[sl * C + c];
+      gate_s[c] = sigmoid(s);
+    }
+    __syncthreads();
+    MB_MARK(tb, 3);
+  };
+  pointwise<true, COH>(b.d, npix, C, b.Cout, b.w_proj, b.s_proj, b.b_proj, false, gate_s, shortcut, b.out, red, gate);
+  MB_MARK(tb, 4);
 }
 
 // Stage s of the launch is phase s % 3 (expand, depthwise, project) of block s / 3.
 __global__ void __launch_bounds__(256) k_mbconv(const Args a) {
-  __shared__ __attribute__((aligned(16))) float red[2048];
+  __shared__ __attribute__((aligned(16))) float red[4096];
   __shared__ __attribute__((aligned(16))) float vec[MAX_C];
   __shared__ float r_s[MAX_R];
   GridBarrier bar;
   grid_barrier_begin(bar, a.ctl);
+  bar.trace = a.trace;
+  bar.trace_cap = a.trace_cap;
   for (int st = a.stage_begin; st < a.stage_end; ++st) {
     const int bi = st / 3, ph = st - bi * 3;
     const Block &b = a.blk[bi];
     bool ran = true;
     if (ph == 0) {
       if (b.has_expand)
-        pointwise<false, true>(b.in, b.H * b.W, b.Cin, b.Cexp, b.w_exp, b.s_exp, b.b_exp, true, nullptr, nullptr, b.e, red);
+        pointwise<false, true>(b.in, b.H * b.W, b.Cin, b.Cexp, b.w_exp, b.s_exp, b.b_exp, true, nullptr, nullptr, b.e, red, []() {});
       else
         ran = false;
     } else if (ph == 1) {
-      if (b.k == 3) depthwise<3, true>(b, red, vec);
-      else depthwise<5, true>(b, red, vec);
+      if (b.k == 3) depthwise<3, true>(b, red, vec, &bar);
+      else depthwise<5, true>(b, red, vec, &bar);
     } else {
-      project<true>(b, vec, r_s, red);
+      project<true>(b, vec, r_s, red, &bar);
     }
     if (ran && st + 1 < a.stage_end) grid_sync(bar);
   }
@@ -284,14 +531,14 @@ __global__ void __launch_bounds__(256) k_pointwise(const PwArgs a) {
   if (a.gate) {
     for (int c = threadIdx.x; c < a.K; c += 256) gate_s[c] = a.gate[c];
     __syncthreads();
-    pointwise<true, false>(a.x, a.M, a.K, a.N, a.w, a.scale, a.shift, a.act != 0, gate_s, a.shortcut, a.y, red);
+    pointwise<true, false>(a.x, a.M, a.K, a.N, a.w, a.scale, a.shift, a.act != 0, gate_s, a.shortcut, a.y, red, []() {});
   } else {
-    pointwise<false, false>(a.x, a.M, a.K, a.N, a.w, a.scale, a.shift, a.act != 0, nullptr, a.shortcut, a.y, red);
+    pointwise<false, false>(a.x, a.M, a.K, a.N, a.w, a.scale, a.shift, a.act != 0, nullptr, a.shortcut, a.y, red, []() {});
   }
 }
 __global__ void __launch_bounds__(256) k_depthwise(const Block b) {
-  __shared__ float red[2048];
-  __shared__ float vec[MAX_C];
+  __shared__ __attribute__((aligned(16))) float red[2048];
+  __shared__ __attribute__((aligned(16))) float vec[MAX_C];
   if (b.k == 3) depthwise<3, false>(b, red, vec);
   else depthwise<5, false>(b, red, vec);
 }
@@ -343,7 +590,7 @@ static int make_plan(const souffle_mbconv_block *blocks, int n, Plan *p) {
     p->out[i] = off;
     if (i + 1 < n) off += round_up((size_t)oh * ow * s->out_c * 2, 256);
     p->part[i] = off;
-    off += round_up((size_t)1024 * PART_LD * 4, 256);          // up to 1024 workgroups
+    off += round_up((size_t)256 * PART_LD * 4, 256);           // at most 256 workgroups
   }
   p->total = off;
   return SOUFFLE_OK;
@@ -382,14 +629,16 @@ extern "C" int souffle_mbconv_stack(const souffle_mbconv_block *blocks, int num_
   if (!aligned16(ws)) return fail(SOUFFLE_ERR_ALIGN, "workspace must be 16-byte aligned");
   DeviceFacts df;
   if (int rc = device_facts(&df)) return rc;
-  if (df.num_cus > 1024) return fail(SOUFFLE_ERR_DEVICE, "more than 1024 compute units");
+  const int grid = df.num_cus < 256 ? df.num_cus : 256;     // the gate stage reads one partial row per thread
   char *base = static_cast<char *>(ws);
   const hipStream_t st = static_cast<hipStream_t>(stream);
   for (int first = 0; first < num_blocks; first += mbconv::MAX_BLOCKS) {
     const int n = num_blocks - first < mbconv::MAX_BLOCKS ? num_blocks - first : mbconv::MAX_BLOCKS;
     mbconv::Args a;
-    a.nblk = n; a.pad = 0;
+    a.nblk = n;
     a.ctl = static_cast<unsigned *>(ws);
+    a.trace = nullptr; a.trace_cap = 0;
+    if (fused) stage_trace(&a.trace, &a.trace_cap, grid);
     for (int i = 0; i < n; ++i) {
       const int gi = first + i;
       mbconv::Block *b = a.blk + i;
@@ -403,12 +652,12 @@ extern "C" int souffle_mbconv_stack(const souffle_mbconv_block *blocks, int num_
     void *args[] = {&a};
     if (fused) {
       a.stage_begin = 0; a.stage_end = 3 * n;
-      if (int rc = launch_persistent((const void *)mbconv::k_mbconv, df.num_cus, 256, args, 0, st)) return rc;
+      if (int rc = launch_persistent((const void *)mbconv::k_mbconv, grid, 256, args, 0, st)) return rc;
     } else {
       for (int s = 0; s < 3 * n; ++s) {
         if (s % 3 == 0 && !a.blk[s / 3].has_expand) continue;
         a.stage_begin = s; a.stage_end = s + 1;
-        if (int rc = launch_persistent((const void *)mbconv::k_mbconv, df.num_cus, 256, args, 0, st)) return rc;
+        if (int rc = launch_persistent((const void *)mbconv::k_mbconv, grid, 256, args, 0, st)) return rc;
       }
     }
   }
@@ -457,8 +706,8 @@ extern "C" int souffle_depthwise_conv2d_bn_swish(const void *x, const void *w, c
   b.Cin = b.Cexp = channels; b.k = kernel; b.stride = stride; b.R = 0; b.has_expand = 0;
   b.w_dw = static_cast<const half_t *>(w); b.s_dw = scale; b.b_dw = shift;
   b.in = static_cast<const half_t *>(x); b.d = static_cast<half_t *>(y);
-  const int P = 256 / (channels / 8), groups = (b.Ho * b.Wo + P - 1) / P;
-  const int grid = groups < df.num_cus * 4 ? groups : df.num_cus * 4;
+  const int passes = mbconv::dw_plan(b).passes;
+  const int grid = passes < df.num_cus * 4 ? passes : df.num_cus * 4;
   hipLaunchKernelGGL(mbconv::k_depthwise, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), b);
   SOUFFLE_HIP_TRY(hipGetLastError());
   return SOUFFLE_OK;

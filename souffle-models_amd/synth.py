@@ -163,7 +163,7 @@ def mbconv_block_weights(shape, config_id=4, block=0, in_rms=1.0):
     b["dw_scale"], b["dw_shift"] = fold(5, ce, k * k, 0.6)
     b["se_reduce_w"] = f16(normal(seed_of(config_id, t + 7), (r, ce), 0.02))
     b["se_reduce_b"] = normal(seed_of(config_id, t + 8), (r,), 0.1).astype(np.float32)
-    b["se_expand_w"] = f16(normal(seed_of(config_id, t + 9), (ce, r), 0.02))
+    b["se_expand_w"] = f16(normal(seed_of(config_id, t + 9), (r, ce), 0.02))
     b["se_expand_b"] = normal(seed_of(config_id, t + 10), (ce,), 0.5).astype(np.float32)
     b["project_w"] = f16(normal(seed_of(config_id, t + 11), (co, ce), 0.02))
     b["project_scale"], b["project_shift"] = fold(12, co, ce, 0.52)

@@ -107,12 +107,12 @@ def test_oracle_depthwise_against_brute_force_loops():
 def test_oracle_se_gate_against_torch():
     P, Cc, R = 49, 24, 6
     x = rnd(13, (P, Cc))
-    wr, br, we, be = rnd(14, (R, Cc), 0.3), rnd(15, (R,)), rnd(16, (Cc, R), 0.3), rnd(17, (Cc,))
+    wr, br, we, be = rnd(14, (R, Cc), 0.3), rnd(15, (R,)), rnd(16, (R, Cc), 0.3), rnd(17, (Cc,))
     got = oracle.se_gate(x, wr, br, we, be)
     p = Fn.adaptive_avg_pool2d(t64(x).t().reshape(1, Cc, 7, 7), 1).reshape(Cc)
     r = t64(wr) @ p + t64(br)
     r = r * torch.sigmoid(r)
-    e = torch.sigmoid(t64(we) @ r + t64(be))
+    e = torch.sigmoid(t64(we).t() @ r + t64(be))
     assert np.abs(got - e.numpy()).max() < 2e-6
 
 
@@ -132,7 +132,7 @@ def torch_block(x, b):
     p = v.mean(dim=(2, 3))[0]
     r = t64(b["se_reduce_w"]) @ p + t64(b["se_reduce_b"])
     r = r * torch.sigmoid(r)
-    e = torch.sigmoid(t64(b["se_expand_w"]) @ r + t64(b["se_expand_b"]))
+    e = torch.sigmoid(t64(b["se_expand_w"]).t() @ r + t64(b["se_expand_b"]))
     v = v * e[None, :, None, None]
     v = Fn.conv2d(v, t64(b["project_w"])[:, :, None, None]) * t64(b["project_scale"])[None, :, None, None] + \
         t64(b["project_shift"])[None, :, None, None]
