@@ -9,11 +9,12 @@
 // kernels per block; here a block is three stages of one launch, separated by grid barriers:
 //
 //   expand   : E = swish(bn(X . We^T))                      one 16x16 MFMA tile per wave
-//   depthwise: D = swish(bn(dwconv(E))), and per workgroup the contribution of its pixels to
-//              the squeeze layer W_r . sum_p D[p]  (R numbers instead of C channel sums)
-//   project  : every workgroup finishes the squeeze-excite gate from those partials (R and C
-//              are tiny), then Y = bn((D * gate) . Wp^T) (+ X), the gate applied to the
-//              activation operand on its way into the MFMA
+//   depthwise: D = swish(bn(dwconv(E))), and per workgroup the contribution of its pixels or
+//              channels to the squeeze layer W_r . sum_p D[p] (R numbers instead of C channel
+//              sums); after one more grid barrier workgroup w turns the partials into the
+//              squeeze-excite gate of channel group w
+//   project  : Y = bn((D * gate) . Wp^T) (+ X), the gate applied to the activation operand on
+//              its way into the MFMA
 //
 // The whole network moves 0.4 GFLOP over ~7 MB of weights and ~12 MB of activations: every
 // stage is latency bound, so the design goal is few, short stages, not MFMA utilisation.  The
@@ -50,6 +51,7 @@ struct Block {
   const half_t *in;
   half_t *e, *d, *out;
   float *part;                   // [workgroup][PART_LD] partial sums of the squeeze layer
+  float *gate;                   // [Cexp] squeeze-excite factors
 };
 
 struct Args {
@@ -185,8 +187,11 @@ __device__ __forceinline__ void pointwise(const half_t *X, int M, int K, int N, 
 // channels of group cg at output pixel pix; returns the 8 fp32 results and stores them as fp16.
 // All taps and their weights are requested before the first is used (addresses clamped into the
 // image, taps outside it masked afterwards): one memory latency per pixel instead of one per tap.
-template <int KS, bool COH>
-__device__ __forceinline__ void dw_pixel(const Block &b, const half_t *src, int pix, int cg, float (&v)[8]) {
+// SLAB: the taps come from an LDS copy of the workgroup's channel groups, laid out
+// [input pixel][groups of the workgroup] in 16-byte granules (`slab`, `slab_ld` groups, this thread's `slot`).
+template <int KS, bool COH, bool SLAB = false>
+__device__ __forceinline__ void dw_pixel(const Block &b, const half_t *src, int pix, int cg, float (&v)[8],
+                                         const u4 *slab = nullptr, int slab_ld = 0, int slot = 0) {
   constexpr int pad = KS / 2;
   const int C = b.Cexp, ho = pix / b.Wo, wo = pix - ho * b.Wo;
   u4 xv[KS * KS], wv[KS * KS];
@@ -197,7 +202,8 @@ __device__ __forceinline__ void dw_pixel(const Block &b, const half_t *src, int 
 #pragma unroll
     for (int j = 0; j < KS; ++j) {
       const int wi = wo * b.stride - pad + j, wc = min(max(wi, 0), b.W - 1);
-      xv[i * KS + j] = ld16<COH && kCohLoads>(src, ((hc * b.W + wc) * C + cg * 8) * 2);
+      if constexpr (SLAB) xv[i * KS + j] = slab[(hc * b.W + wc) * slab_ld + slot];
+      else xv[i * KS + j] = ld16<COH && kCohLoads>(src, ((hc * b.W + wc) * C + cg * 8) * 2);
       if (hi == hc && wi == wc) inside |= 1u << (i * KS + j);
     }
   }
@@ -250,7 +256,7 @@ __host__ __device__ __forceinline__ DwPlan dw_plan(const Block &b) {
 }
 
 template <int KS, bool COH>
-__device__ __forceinline__ void depthwise(const Block &b, float *red, float *sums, const GridBarrier *tb = nullptr) {
+__device__ __forceinline__ void depthwise(const Block &b, float *red, float *sums, u4 *slab, const GridBarrier *tb = nullptr) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int C = b.Cexp, G = C >> 3, npix = b.Ho * b.Wo;
   const half_t *src = b.has_expand ? b.e : b.in;
@@ -273,11 +279,28 @@ __device__ __forceinline__ void depthwise(const Block &b, float *red, float *sum
           if (!ok) wr[q] = u4{0u, 0u, 0u, 0u};
         }
       }
+      // the set's channel groups of every input pixel go to LDS first, [input pixel][CGW] granules of
+      // 16 bytes (at most 1024: input pixels <= 4 x output pixels, CGW x output pixels <= 256): the image
+      // is fetched once per workgroup in runs of CGW*16 bytes instead of once per tap and lane
+      {
+        const int ngr = b.H * b.W * CGW;
+        u4 sv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int idx = tid + 256 * i, ip = idx / CGW, sl = idx - ip * CGW;
+          const bool ok = idx < ngr && set * CGW + sl < G;
+          sv[i] = ld16<COH && kCohLoads>(src, ok ? (ip * C + (set * CGW + sl) * 8) * 2 : 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (tid + 256 * i < ngr) slab[tid + 256 * i] = sv[i];
+        __syncthreads();
+      }
       float v[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) v[q] = 0.f;
       MB_MARK(tb, 0);
-      if (act) dw_pixel<KS, COH>(b, src, pix, cg, v);
+      if (act) dw_pixel<KS, COH, true>(b, src, pix, cg, v, slab, CGW, slot);
       if (b.R > 0) {
         // channel sums over the pixels: channel ch = slot*8 + q, NP threads per channel take every NP-th pixel
         if (slot < CGW) {
@@ -311,8 +334,8 @@ __device__ __forceinline__ void depthwise(const Block &b, float *red, float *sum
             }
           }
         }
-        __syncthreads();
       }
+      __syncthreads();               // slab, red and sums are rewritten by the next set
     }
     if (tid < b.R) st4<COH>(b.part, ((int)blockIdx.x * PART_LD + tid) * 4, __float_as_uint(pj));
     MB_MARK(tb, 3);
@@ -394,12 +417,74 @@ __device__ __forceinline__ void depthwise(const Block &b, float *red, float *sum
   __syncthreads();                 // red / sums are reused by the next stage
 }
 
-// gate[c] = sigmoid(b_e[c] + sum_j W_e[j][c] * swish(b_r[j] + (sum over workgroups of part[.][j]) / pixels)),
-// evaluated by every workgroup that has a tile of the projection, while the operands of that tile
-// are already on their way; then the projection with the gate folded into its activation operand.
-constexpr int kGateRows = 24;      // rows of W_e a thread requests at a time
+// Second half of the depthwise stage of a block with a squeeze-excite module:
+// gate[c] = sigmoid(b_e[c] + sum_j W_e[j][c] * swish(b_r[j] + (sum over workgroups of part[.][j]) / pixels)).
+// One grid barrier after the partials; then workgroup w evaluates the 8 channels of group w (and
+// w + grid, ...): every element of W_e is read once by the whole grid, requested before the barrier.
 template <bool COH>
-__device__ __forceinline__ void project(const Block &b, float *gate_s, float *r_s, float *red, const GridBarrier *tb = nullptr) {
+__device__ __forceinline__ void squeeze_gate(const Block &b, GridBarrier &bar, float *red, float *scratch, float *r_s) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int C = b.Cexp, G = C >> 3, npix = b.Ho * b.Wo;
+  const bool mine = (int)blockIdx.x < G;
+  u4 we = {0u, 0u, 0u, 0u};
+  if (mine && tid < b.R) we = *reinterpret_cast<const u4 *>(b.w_se + tid * C + blockIdx.x * 8);
+  grid_sync(bar);
+  if (!mine) return;
+  // the partial rows of all workgroups go through LDS (all loads of a chunk in flight together),
+  // thread (quarter, j) sums every fourth row of column j, the quarters are added in a fixed order
+  const int nact = min(dw_plan(b).passes, (int)gridDim.x);
+  const int R4 = (b.R + 3) >> 2, chunk_rows = 1024 / R4;
+  const int j = tid & 63, quarter = tid >> 6;
+  float accj = 0.f;
+  for (int row0 = 0; row0 < nact; row0 += chunk_rows) {
+    const int rows = min(chunk_rows, nact - row0), ngran = rows * R4;
+    u4 pv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + 256 * i, r = idx / R4, q = idx - r * R4;
+      pv[i] = ld16<COH && kCohLoads>(b.part, idx < ngran ? ((row0 + r) * PART_LD + q * 4) * 4 : 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (tid + 256 * i < ngran) *reinterpret_cast<u4 *>(red + (tid + 256 * i) * 4) = pv[i];
+    __syncthreads();
+    if (j < b.R)
+      for (int r = quarter; r < rows; r += 4) accj += red[r * R4 * 4 + j];
+    __syncthreads();
+  }
+  scratch[quarter * 64 + j] = accj;
+  __syncthreads();
+  if (tid < 64) {                    // wave 0: lane j holds r[j], then the 8 channel sums over j
+    float rj = 0.f;
+    if (tid < b.R) {
+      const float t = (scratch[tid] + scratch[64 + tid]) + (scratch[128 + tid] + scratch[192 + tid]);
+      rj = swish(t / (float)npix + (b.b_red ? b.b_red[tid] : 0.f));
+    }
+    for (int cg = blockIdx.x; cg < G; cg += gridDim.x) {
+      if (cg != (int)blockIdx.x) {
+        we = u4{0u, 0u, 0u, 0u};
+        if (tid < b.R) we = *reinterpret_cast<const u4 *>(b.w_se + tid * C + cg * 8);
+      }
+      const h8 w = as_h8(we);
+      float mine_q = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float t = wave_sum((float)w[q] * rj);
+        if (lane == q) mine_q = t;
+      }
+      if (lane < 8) {
+        const int c = cg * 8 + lane;
+        st4<COH>(b.gate, c * 4, __float_as_uint(sigmoid(mine_q + (b.b_se ? b.b_se[c] : 0.f))));
+      }
+    }
+  }
+  __syncthreads();
+}
+
+// Projection with the squeeze-excite gate folded into its activation operand; the gate vector is
+// requested together with the operands of the first tile.
+template <bool COH>
+__device__ __forceinline__ void project(const Block &b, float *gate_s, float *red, const GridBarrier *tb = nullptr) {
   const int tid = threadIdx.x;
   const int npix = b.Ho * b.Wo, C = b.Cexp;
   const half_t *shortcut = b.has_shortcut ? b.in : nullptr;
@@ -412,78 +497,16 @@ __device__ __forceinline__ void project(const Block &b, float *gate_s, float *r_
     if ((int)blockIdx.x * (units <= (int)gridDim.x ? 1 : 4) >= units) return;
   }
   auto gate = [&]() {
-    const int G = C >> 3, nact = min(dw_plan(b).passes, (int)gridDim.x);
-    const int JS = 256 / G, slice = tid / G, cg = tid - slice * G;
-    // requested up front: the first chunk of partial rows and this thread's first rows of W_e
-    const int R4 = (b.R + 3) >> 2, chunk_rows = 1024 / R4;
-    u4 pv[4], w[kGateRows];
-    auto load_partials = [&](int row0) {
-      const int ngran = min(chunk_rows, nact - row0) * R4;
+    u4 gv[MAX_C / 1024];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int idx = tid + 256 * i, r = idx / R4, q = idx - r * R4;
-        pv[i] = ld16<COH && kCohLoads>(b.part, idx < ngran ? ((row0 + r) * PART_LD + q * 4) * 4 : 0);
-      }
-    };
-    auto load_rows = [&](int j0) {
-#pragma unroll
-      for (int i = 0; i < kGateRows; ++i)
-        w[i] = *reinterpret_cast<const u4 *>(b.w_se + (slice < JS ? min(j0 + i * JS, b.R - 1) * C + cg * 8 : 0));
-    };
-    MB_MARK(tb, 0);
-    load_partials(0);
-    load_rows(slice);
-    MB_MARK(tb, 1);
-    // (1) the partial rows of all workgroups go through LDS, thread (quarter, j) sums every fourth row
-    //     of column j, the quarters are added in a fixed order
-    const int j = tid & 63, quarter = tid >> 6;
-    float accj = 0.f;
-    for (int row0 = 0; row0 < nact; row0 += chunk_rows) {
-      if (row0) load_partials(row0);
-      const int rows = min(chunk_rows, nact - row0), ngran = rows * R4;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (tid + 256 * i < ngran) *reinterpret_cast<u4 *>(red + (tid + 256 * i) * 4) = pv[i];
-      __syncthreads();
-      if (j < b.R)
-        for (int r = quarter; r < rows; r += 4) accj += red[r * R4 * 4 + j];
-      __syncthreads();
+    for (int i = 0; i < MAX_C / 1024; ++i) {
+      const int idx = tid + 256 * i;
+      gv[i] = ld16<COH && kCohLoads>(b.gate, idx * 4 < C ? idx * 16 : 0);
     }
-    gate_s[quarter * 64 + j] = accj;
-    __syncthreads();
-    if (tid < b.R) {
-      const float s = (gate_s[tid] + gate_s[64 + tid]) + (gate_s[128 + tid] + gate_s[192 + tid]);
-      r_s[tid] = swish(s / (float)npix + (b.b_red ? b.b_red[tid] : 0.f));
-    }
-    __syncthreads();
-    MB_MARK(tb, 2);
-    // (2) W_e . r with 16-byte loads: thread (slice, cg) takes 8 channels and every JS-th squeezed row
-    float g8[8];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) g8[q] = 0.f;
-    if (slice < JS) {
-      for (int j0 = slice; j0 < b.R; j0 += JS * kGateRows) {
-        if (j0 != slice) load_rows(j0);
-#pragma unroll
-        for (int i = 0; i < kGateRows; ++i) {
-          const int jj = j0 + i * JS;
-          const float rj = jj < b.R ? r_s[min(jj, MAX_R - 1)] : 0.f;
-          const h8 h = as_h8(w[i]);
-#pragma unroll
-          for (int q = 0; q < 8; ++q) g8[q] += (float)h[q] * rj;
-        }
-      }
-#pragma unroll
-      for (int q = 0; q < 8; ++q) red[slice * C + cg * 8 + q] = g8[q];          // JS * C <= 2048
-    }
+    for (int i = 0; i < MAX_C / 1024; ++i)
+      if ((tid + 256 * i) * 4 < C) *reinterpret_cast<u4 *>(gate_s + (tid + 256 * i) * 4) = gv[i];
     __syncthreads();
-    for (int c = tid; c < C; c += 256) {
-      float s = b.b_se ? b.b_se[c] : 0.f;
-      for (int sl = 0; sl < JS; ++sl) s += red[sl * C + c];
-      gate_s[c] = sigmoid(s);
-    }
-    __syncthreads();
-    MB_MARK(tb, 3);
   };
   pointwise<true, COH>(b.d, npix, C, b.Cout, b.w_proj, b.s_proj, b.b_proj, false, gate_s, shortcut, b.out, red, gate);
   MB_MARK(tb, 4);
@@ -493,6 +516,7 @@ __device__ __forceinline__ void project(const Block &b, float *gate_s, float *r_
 __global__ void __launch_bounds__(256) k_mbconv(const Args a) {
   __shared__ __attribute__((aligned(16))) float red[4096];
   __shared__ __attribute__((aligned(16))) float vec[MAX_C];
+  __shared__ u4 slab[1024];
   __shared__ float r_s[MAX_R];
   GridBarrier bar;
   grid_barrier_begin(bar, a.ctl);
@@ -508,10 +532,11 @@ __global__ void __launch_bounds__(256) k_mbconv(const Args a) {
       else
         ran = false;
     } else if (ph == 1) {
-      if (b.k == 3) depthwise<3, true>(b, red, vec, &bar);
-      else depthwise<5, true>(b, red, vec, &bar);
+      if (b.k == 3) depthwise<3, true>(b, red, vec, slab, &bar);
+      else depthwise<5, true>(b, red, vec, slab, &bar);
+      if (b.R > 0) squeeze_gate<true>(b, bar, red, vec, r_s);
     } else {
-      project<true>(b, vec, r_s, red, &bar);
+      project<true>(b, vec, red, &bar);
     }
     if (ran && st + 1 < a.stage_end) grid_sync(bar);
   }
@@ -539,8 +564,9 @@ __global__ void __launch_bounds__(256) k_pointwise(const PwArgs a) {
 __global__ void __launch_bounds__(256) k_depthwise(const Block b) {
   __shared__ __attribute__((aligned(16))) float red[2048];
   __shared__ __attribute__((aligned(16))) float vec[MAX_C];
-  if (b.k == 3) depthwise<3, false>(b, red, vec);
-  else depthwise<5, false>(b, red, vec);
+  __shared__ u4 slab[1024];
+  if (b.k == 3) depthwise<3, false>(b, red, vec, slab);
+  else depthwise<5, false>(b, red, vec, slab);
 }
 
 static int out_extent(int in, int kernel, int stride) { return (in + (kernel - 1) - kernel) / stride + 1; }
@@ -572,7 +598,7 @@ static int check_block(const souffle_mbconv_block *s, int i) {
 // Workspace: control block, then per block E (if expanded), D, the block output (all blocks but
 // the last) and the squeeze partials, each at an address of its own (see the file comment).
 struct Plan {
-  size_t e[1024], d[1024], out[1024], part[1024], total;
+  size_t e[1024], d[1024], out[1024], part[1024], gate[1024], total;
 };
 static int make_plan(const souffle_mbconv_block *blocks, int n, Plan *p) {
   if (!blocks || n <= 0 || n > 1024) return fail(SOUFFLE_ERR_SHAPE, "need 1..1024 blocks");
@@ -591,6 +617,8 @@ static int make_plan(const souffle_mbconv_block *blocks, int n, Plan *p) {
     if (i + 1 < n) off += round_up((size_t)oh * ow * s->out_c * 2, 256);
     p->part[i] = off;
     off += round_up((size_t)256 * PART_LD * 4, 256);           // at most 256 workgroups
+    p->gate[i] = off;
+    off += round_up((size_t)MAX_C * 4, 256);
   }
   p->total = off;
   return SOUFFLE_OK;
@@ -648,6 +676,7 @@ extern "C" int souffle_mbconv_stack(const souffle_mbconv_block *blocks, int num_
       b->d = reinterpret_cast<half_t *>(base + p.d[gi]);
       b->out = gi + 1 == num_blocks ? static_cast<half_t *>(y) : reinterpret_cast<half_t *>(base + p.out[gi]);
       b->part = reinterpret_cast<float *>(base + p.part[gi]);
+      b->gate = reinterpret_cast<float *>(base + p.gate[gi]);
     }
     void *args[] = {&a};
     if (fused) {
