@@ -7,7 +7,7 @@ pass over one synthetic input; the timed passes rotate through several distinct 
 sets (> 512 MB in total) so that the weight stream comes from HBM, not from the 256 MB
 Infinity Cache.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload encoder|layer|encoder_s384|encoder_b32|lstm|swin|se|mbconv]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload encoder|layer|encoder_s384|encoder_b32|lstm|swin|swin_merge|se|mbconv]
 """
 import argparse
 import json

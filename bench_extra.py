@@ -1,4 +1,4 @@
-"""Secondary bench workloads selected with bench.py --workload {lstm,swin,se,mbconv}.
+"""Secondary bench workloads selected with bench.py --workload {lstm,swin,swin_merge,se,mbconv}.
 Each prints the same JSON shape as the default workload."""
 import os
 import sys
@@ -179,7 +179,49 @@ def bench_mbconv(args):
     return res
 
 
+def bench_swin_merge(args):
+    import numpy as np
+    import torch
+    import swin_transformer_binding as sb
+    import synth
+    from bench import time_steps
+    H = W = 56
+    Cc = 128
+    x = synth.swin_input(3)
+    w = synth.f16(synth.normal(synth.seed_of(3, 200), (4 * Cc, 2 * Cc), 0.02))
+    g = synth.f16(1.0 + synth.normal(synth.seed_of(3, 201), (4 * Cc,), 0.1))
+    b = synth.f16(synth.normal(synth.seed_of(3, 202), (4 * Cc,), 0.1))
+    dx, dw, dg, db = [torch.from_numpy(a).cuda() for a in (x, w, g, b)]
+    y = sb.patch_merging(dx, H, W, dg, db, dw).float().cpu().numpy()
+    res_cpu = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle
+        thr = _threads()
+        ref = oracle.swin_patch_merge(x, H, W, g, b, w, threads=thr)
+        dd = np.abs(y - ref)
+        if not (dd.max() <= 2e-2 and dd.mean() <= 2e-3):
+            print("PARITY FAILURE (swin_merge): %g %g" % (dd.max(), dd.mean()), file=sys.stderr)
+            sys.exit(1)
+        us, n = _cpu_time(lambda: oracle.swin_patch_merge(x, H, W, g, b, w, threads=thr), min(args.cpu_seconds, 5.0))
+        res_cpu = {"value": us, "unit": "us", "cores": thr, "kind": "port",
+                   "sample": "%d passes of the 56x56x128 patch merge through oracle/swin_oracle.c (OpenMP fp32)" % n}
+    wall, ev = time_steps(lambda i: sb.patch_merging(dx, H, W, dg, db, dw), args.steps, args.warmup)
+    bytes_alg = x.nbytes + w.nbytes + g.nbytes + b.nbytes + y.size * 2
+    ach = bytes_alg / (ev * 1e-3) / 1e9
+    roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
+            "kernel": "k_patch_merge", "algorithmic_bytes_per_launch": bytes_alg,
+            "algorithmic_flops_per_launch": 2.0 * 784 * 512 * 256, "avg_launch_us": ev * 1e3,
+            "note": "one launch of 1.5 MB and 0.2 GFLOP: launch and memory latency, not bandwidth"}
+    res = _base("swin_patch_merge_latency_us", wall * 1e3, args, "Swin patch merging 56x56x128 -> 28x28x256, fp16", "f16", roof, {})
+    if res_cpu:
+        res["cpu_baseline"] = res_cpu
+    return res
+
+
 def run(args):
+    if args.workload == "swin_merge":
+        return bench_swin_merge(args)
     if args.workload == "mbconv":
         return bench_mbconv(args)
     if args.workload == "lstm":

@@ -228,6 +228,15 @@ int souffle_swin_ffn_fused(const void *x, const void *w1, const void *w2, void *
 int souffle_gemm_f16(const void *x, const void *w, void *y, int M, int N, int K,
                      souffle_stream_t stream);
 
+/* Patch merging between two Swin stages: x [H][W][C] -> y [(H/2)*(W/2)][2C],
+ * y = LN(cat(x[0::2,0::2], x[1::2,0::2], x[0::2,1::2], x[1::2,1::2]); gamma, beta, eps) . w, w fp16 [4C][2C],
+ * gamma/beta fp16 [4C] nullable.  H, W even, C a multiple of 32.
+ * Replaces fused_patch_merging_reshape_reduce_sum, layer_normalization_variance,
+ * layer_normalization_normal and the reduction product
+ * (python/models/swin_transformer/swin_patch_merge.py:3-13,49-144). */
+int souffle_swin_patch_merge(const void *x, const void *ln_g, const void *ln_b, const void *w, void *y,
+                             int height, int width, int channels, float ln_eps, souffle_stream_t stream);
+
 /* ----------------------------------------------------- EfficientNet SE ---- */
 enum { SOUFFLE_SE_MUL = 0, SOUFFLE_SE_ADD = 1 };
 size_t souffle_se_workspace_bytes(int C, int HW, int R);

@@ -15,6 +15,9 @@
  *   oracle_swin_index_maps     torch.roll / view+permute window partition,
  *                              brute force on tiny grids, permutation laws
  *   oracle_swin_block_pair_f32 torch CPU library restatement of a Swin block
+ *   oracle_swin_patch_merge_f32  the reference's own torch statement (strided slices, cat,
+ *                              layer_norm, matmul; swin_patch_merge.py:3-13) in float64 and its
+ *                              tensor-expression index formula evaluated by brute force
  *   oracle_se_module_f32       torch avg_pool2d / conv2d / sigmoid composition
  *   oracle_pointwise_conv_f32, oracle_depthwise_conv_f32, oracle_se_gate_f32,
  *   oracle_mbconv_block_f32    torch conv2d (groups / stride / explicit padding), adaptive
@@ -135,6 +138,10 @@ int oracle_swin_block_pair_f32(const oracle_swin_cfg *cfg, const oracle_swin_blo
 /* Y1 = X.W1 ; Y2 = Y1.W2 (no bias, no activation) -- the reference's fused Swin FFN. */
 int oracle_swin_ffn_f32(const float *x, const float *w1, const float *w2, float *y1, float *y2,
                         int M, int K, int F, int num_threads);
+
+/* x [H][W][C] -> y [(H/2)*(W/2)][2C]; ln_g / ln_b [4C] nullable; w [4C][2C]. */
+int oracle_swin_patch_merge_f32(const float *x, const float *ln_g, const float *ln_b, const float *w, float *y,
+                                int height, int width, int channels, float ln_eps, int num_threads);
 
 /* ---- EfficientNet SE module ---- */
 enum { ORACLE_SE_MUL = 0, ORACLE_SE_ADD = 1 };

@@ -246,6 +246,17 @@ def swin_ffn(x, w1, w2, threads=0):
     return y1, y2
 
 
+def swin_patch_merge(x, height, width, ln_g, ln_b, w, ln_eps=1e-5, threads=0):
+    """x [H*W, C] -> [(H/2)*(W/2), 2C]."""
+    x, ln_g, ln_b, w = _f32(x), _f32(ln_g), _f32(ln_b), _f32(w)
+    Cc = x.shape[-1]
+    y = np.empty(((height // 2) * (width // 2), 2 * Cc), np.float32)
+    rc = lib().oracle_swin_patch_merge_f32(_p(x), _p(ln_g), _p(ln_b), _p(w), _p(y), height, width, Cc, C.c_float(ln_eps), threads)
+    if rc:
+        raise RuntimeError("oracle_swin_patch_merge_f32 failed: %d" % rc)
+    return y
+
+
 def se_module(x, w_reduce, w_expand, b_reduce=None, b_expand=None, combine="mul"):
     """x [C,HW]; returns (y [C,HW], pooled [C])."""
     x, w_reduce, w_expand, b_reduce, b_expand = _f32(x), _f32(w_reduce), _f32(w_expand), _f32(b_reduce), _f32(b_expand)

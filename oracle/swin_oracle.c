@@ -131,3 +131,26 @@ int oracle_swin_ffn_f32(const float *x, const float *w1, const float *w2, float 
   oracle_gemm_f32(y1, w2, NULL, y2, M, K, F, num_threads);
   return 0;
 }
+
+/* Patch merging (python/models/swin_transformer/swin_patch_merge.py:3-13 and the tensor expression
+ * :49-63): merged[m][q*C + c] = x[2i + q%2][2j + q/2][c] with m = i*(W/2) + j, then LayerNorm over
+ * the 4C merged channels (:95-144; biased variance, eps inside the root) and the bias-free
+ * reduction y = LN(merged) . w, w [4C][2C]. */
+int oracle_swin_patch_merge_f32(const float *x, const float *ln_g, const float *ln_b, const float *w, float *y,
+                                int height, int width, int channels, float ln_eps, int num_threads) {
+  if (!x || !w || !y || height <= 0 || width <= 0 || (height & 1) || (width & 1) || channels <= 0) return -1;
+  const int H2 = height / 2, W2 = width / 2, M = H2 * W2, K = 4 * channels, N = 2 * channels;
+  float *merged = (float *)malloc(sizeof(float) * (size_t)M * K);
+  float *z = (float *)malloc(sizeof(float) * (size_t)M * K);
+  if (!merged || !z) { free(merged); free(z); return -3; }
+  for (int i = 0; i < H2; ++i)
+    for (int j = 0; j < W2; ++j)
+      for (int q = 0; q < 4; ++q)
+        for (int c = 0; c < channels; ++c)
+          merged[((size_t)i * W2 + j) * K + q * channels + c] =
+              x[((size_t)(2 * i + q % 2) * width + 2 * j + q / 2) * channels + c];
+  oracle_layernorm_f32(merged, ln_g, ln_b, z, M, K, ln_eps);
+  oracle_gemm_f32(z, w, NULL, y, M, N, K, num_threads);
+  free(merged); free(z);
+  return 0;
+}

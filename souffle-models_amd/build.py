@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libsouffle_hip.so")
-SOURCES = ["api_common.hip", "bert.hip", "bert_io.hip", "lstm.hip", "swin.hip", "se.hip", "mbconv.hip"]
+SOURCES = ["api_common.hip", "bert.hip", "bert_io.hip", "lstm.hip", "swin.hip", "swin_merge.hip", "se.hip", "mbconv.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -116,3 +116,19 @@ def index_maps(height, width, window, shift):
     p = lambda a: a.ctypes.data_as(C.c_void_p)
     sh.check(sh.lib().souffle_swin_index_maps(height, width, window, shift, p(g), p(s), p(r), p(reg)))
     return g, s, r.reshape(N, N), reg
+
+
+def patch_merging(x, height, width, norm_weight, norm_bias, reduction_weight, ln_eps=1e-5):
+    """Patch merging between two stages (python/models/swin_transformer/swin_patch_merge.py:3-13):
+    x [H*W, C] fp16 -> [(H/2)*(W/2), 2C]; norm_weight / norm_bias [4C] (None = 1 / 0),
+    reduction_weight [4C, 2C] (the transpose of torch's Linear weight, like every weight here)."""
+    Cc = x.shape[-1]
+    _check("x", x, (height * width, Cc))
+    _check("reduction_weight", reduction_weight, (4 * Cc, 2 * Cc))
+    for n, t in (("norm_weight", norm_weight), ("norm_bias", norm_bias)):
+        if t is not None:
+            _check(n, t, (4 * Cc,))
+    y = torch.empty(((height // 2) * (width // 2), 2 * Cc), dtype=torch.float16, device=x.device)
+    sh.check(sh.lib().souffle_swin_patch_merge(x.data_ptr(), sh.ptr(norm_weight), sh.ptr(norm_bias), reduction_weight.data_ptr(),
+                                               y.data_ptr(), height, width, Cc, float(ln_eps), sh.current_stream()))
+    return y
