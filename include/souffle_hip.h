@@ -98,7 +98,9 @@ int souffle_set_bert_sync(int mode);
 enum { SOUFFLE_ACT_GELU_TANH = 0, SOUFFLE_ACT_RELU = 1 };
 
 typedef struct {
-  int batch, seq_len;          /* runtime; batch*seq_len must be a multiple of 128, seq_len of 64, seq_len <= 512 */
+  int batch, seq_len;          /* runtime; seq_len <= 512.  Lengths other than 64/128/256/384/512 run as the next of
+                                  these with the surplus keys masked out (rows copied in and out through the
+                                  workspace; not with per-stage dump tensors) */
   int hidden, heads, ffn;      /* 768, 12, 3072 (the reference's compile-time family, cpp/bert/kernels/bert.h:8-16) */
   int act;                     /* SOUFFLE_ACT_*; reference fused path uses ReLU, its unfused path tanh-GELU */
   float scale;                 /* multiplies q.k (0.125 = 1/sqrt(64)) */

@@ -109,6 +109,22 @@ def souffle_bert_layer(src, qkv_weight, attn_fc_weight, feed_forward_fc1_weight,
         sh.check(fn(C.byref(cfg), C.byref(w), src.data_ptr(), sh.ptr(mask), out.data_ptr(), None, ws.ptr,
                     ws.nbytes, sh.current_stream()))
         return out
+    SP = next(v for v in (64, 128, 256, 384, 512) if v >= S) if S <= 512 else S
+    if SP != S:
+        # per-stage tensors of a sequence length that is not built: run the padded length with the
+        # surplus keys masked out and cut the six tensors back to S
+        xp = torch.zeros((B, SP, HIDDEN), dtype=torch.float16, device=dev)
+        xp[:, :S] = src.view(B, S, HIDDEN)
+        mp = torch.zeros((B, SP, SP), dtype=torch.float16, device=dev)
+        mp[:, :, S:] = -10000.0
+        if mask is not None:
+            mp[:, :S, :S] = mask
+        outs = souffle_bert_layer(xp, qkv_weight, attn_fc_weight, feed_forward_fc1_weight, feed_forward_fc2_weight, opt_level,
+                                  act=act, scale=scale, ln_eps=ln_eps, mask=mp, dump=True, **biases)
+        hd = HIDDEN // HEADS
+        rows = lambda t: t.view(B, SP, -1)[:, :S].reshape(B * S, -1)
+        return [outs[0].view(B * 3, HEADS, SP, hd)[:, :, :S].contiguous(), outs[1].view(B * HEADS, SP, SP)[:, :S, :S].contiguous(),
+                rows(outs[2]), rows(outs[3]), rows(outs[4]), rows(outs[5])]
     qkv = torch.empty((B * 3, HEADS, S, HIDDEN // HEADS), dtype=torch.float16, device=dev)
     probs = torch.empty((B * HEADS, S, S), dtype=torch.float16, device=dev)
     ctx = torch.empty((M, HIDDEN), dtype=torch.float16, device=dev)

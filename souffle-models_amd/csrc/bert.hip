@@ -1320,23 +1320,59 @@ __global__ void __launch_bounds__(256) k_outproj_small(Args a, int l, const half
   small_outproj<false>(lds_raw, a, a.layers[l], xin, false);
 }
 
+// ---- sequence lengths that are not built: rows copied into / out of a padded layout ----
+// xp[b][s][:] = s < S ? x[b][s][:] : 0, 16 bytes per thread.
+__global__ void __launch_bounds__(256) k_pad_rows(const half_t *x, half_t *xp, int B, int S, int SP) {
+  const int n = B * SP * (H / 8);
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
+    const int g = i % (H / 8), r = i / (H / 8), b = r / SP, sq = r - b * SP;
+    u4 v = {0u, 0u, 0u, 0u};
+    if (sq < S) v = *reinterpret_cast<const u4 *>(x + ((size_t)(b * S + sq) * H + g * 8));
+    *reinterpret_cast<u4 *>(xp + (size_t)i * 8) = v;
+  }
+}
+// y[b][s][:] = yp[b][s][:] for s < S.
+__global__ void __launch_bounds__(256) k_unpad_rows(const half_t *yp, half_t *y, int B, int S, int SP) {
+  const int n = B * S * (H / 8);
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
+    const int g = i % (H / 8), r = i / (H / 8), b = r / S, sq = r - b * S;
+    *reinterpret_cast<u4 *>(y + (size_t)i * 8) = *reinterpret_cast<const u4 *>(yp + ((size_t)(b * SP + sq) * H + g * 8));
+  }
+}
+// mp[b][q][k] = k >= S ? -10000 : (q < S and mask given ? mask[b][q][k] : 0): exp(-10000 - max) is 0 in
+// fp32, so the surplus keys take no part in any softmax.
+__global__ void __launch_bounds__(256) k_pad_mask(const half_t *mask, half_t *mp, int B, int S, int SP) {
+  const int n = B * SP * SP;
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
+    const int k = i % SP, r = i / SP, b = r / SP, q = r - b * SP;
+    half_t v = (half_t)0.0f;
+    if (k >= S) v = (half_t)-10000.0f;
+    else if (mask && q < S) v = mask[((size_t)b * S + q) * S + k];
+    mp[i] = v;
+  }
+}
+
 // ------------------------------------------------------------------- host ----
 struct Plan {
   bool large, big;
   int splitk_o, splitk_f;
   size_t off_ctl, off_qkv, off_ctx, off_z1, off_y1, off_h, off_yl, off_part, layer_stride, total;
   size_t flow_bytes;      // a layer's buffers without its output (which comes last)
+  size_t off_xpad, off_ypad, off_maskpad;
   unsigned flow_marker;
 };
+
+// The attention tiles are built for these sequence lengths; any other length up to 512 runs as the
+// next one of them with the surplus key positions masked out (rows copied in and out, see run_padded).
+static int padded_len(int s) { return s <= 64 ? 64 : s <= 128 ? 128 : s <= 256 ? 256 : s <= 384 ? 384 : 512; }
 
 static int validate(const souffle_bert_cfg *c) {
   if (!c) return fail(SOUFFLE_ERR_NULL, "cfg is NULL");
   if (c->hidden != H || c->heads != NH || c->ffn != F)
     return fail(SOUFFLE_ERR_SHAPE, "only hidden=768 heads=12 ffn=3072 is built (got %d/%d/%d)", c->hidden, c->heads, c->ffn);
   if (c->batch <= 0 || c->seq_len <= 0) return fail(SOUFFLE_ERR_SHAPE, "batch and seq_len must be positive");
-  const int s = c->seq_len;
-  if (!(s == 64 || s == 128 || s == 256 || s == 384 || s == 512))
-    return fail(SOUFFLE_ERR_SHAPE, "seq_len must be one of 64,128,256,384,512 (got %d)", s);
+  if (c->seq_len > 512) return fail(SOUFFLE_ERR_SHAPE, "seq_len must be at most 512 (got %d)", c->seq_len);
+  const int s = padded_len(c->seq_len);          // other lengths run padded to the next built one
   const long long m = (long long)c->batch * s;
   if (m >= 1024 && m % 128 != 0) return fail(SOUFFLE_ERR_SHAPE, "batch*seq_len >= 1024 must be a multiple of 128 (got %lld)", m);
   if (m > 65536) return fail(SOUFFLE_ERR_SHAPE, "batch*seq_len must be <= 65536 (got %lld)", m);
@@ -1347,7 +1383,7 @@ static int validate(const souffle_bert_cfg *c) {
 
 static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   Plan p;
-  const size_t M = (size_t)c->batch * c->seq_len;
+  const size_t M = (size_t)c->batch * padded_len(c->seq_len);
   p.large = M >= 1024;
   p.big = M >= 2048 && M % 256 == 0;
   p.splitk_o = 1;
@@ -1366,6 +1402,15 @@ static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   p.layer_stride = off - first;                       // one set of inter-stage buffers per layer
   p.flow_bytes = p.off_yl - p.off_qkv;
   p.total = first + p.layer_stride * (size_t)(num_layers < 1 ? 1 : num_layers);
+  // a sequence length that is not built: padded copies of x and y and the padded additive mask
+  p.off_xpad = p.off_ypad = p.off_maskpad = 0;
+  if (padded_len(c->seq_len) != c->seq_len) {
+    off = p.total;
+    p.off_xpad = take(M * H * 2);
+    p.off_ypad = take(M * H * 2);
+    p.off_maskpad = take(M * (size_t)padded_len(c->seq_len) * 2);
+    p.total = off;
+  }
   // names the layout (rows, layers, extent) in the control block; never 0
   p.flow_marker = (unsigned)((M * 2654435761ull) ^ ((size_t)num_layers * 40503ull) ^ (p.total >> 4)) | 0x80000000u;
   return p;
@@ -1466,14 +1511,66 @@ static int launch_flow(Args &a, int grid, hipStream_t st) {
   }
 }
 
-static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *layers, int nl, const void *x,
-                     const void *mask, void *y, const souffle_bert_dump *dump, void *ws, size_t ws_bytes,
+// A sequence length that is not built runs as the next built one: x is copied into a zero-padded
+// layout, the additive mask is extended so that the surplus keys drop out of every softmax, and the
+// first S rows of every sequence are copied back.  Returns the configuration and pointers the
+// kernels see (`before`), and copies the result out (`after`).
+struct Padded {
+  souffle_bert_cfg cfg;
+  const void *x, *mask;
+  void *y;
+  bool on;
+};
+static int pad_before(Padded &pd, const souffle_bert_cfg *c, const void *x, const void *mask, void *y, const souffle_bert_dump *dump,
+                      void *ws, size_t ws_bytes, const Plan &p, int num_cus, hipStream_t st) {
+  pd.cfg = *c; pd.x = x; pd.mask = mask; pd.y = y;
+  pd.on = padded_len(c->seq_len) != c->seq_len;
+  if (!pd.on) return SOUFFLE_OK;
+  if (dump) return fail(SOUFFLE_ERR_SHAPE, "per-stage tensors need seq_len in {64,128,256,384,512} (got %d)", c->seq_len);
+  if (!x || !y) return fail(SOUFFLE_ERR_NULL, "layers, x and y must not be NULL");
+  if (!ws) return fail(SOUFFLE_ERR_WORKSPACE, "workspace is NULL (need %zu bytes)", p.total);
+  if (ws_bytes < p.total) return fail(SOUFFLE_ERR_WORKSPACE, "workspace too small: %zu < %zu bytes", ws_bytes, p.total);
+  if (!aligned16(x) || !aligned16(y) || !aligned16(ws))
+    return fail(SOUFFLE_ERR_ALIGN, "x, y and workspace must be 16-byte aligned");
+  char *base = static_cast<char *>(ws);
+  const int SP = padded_len(c->seq_len);
+  pd.cfg.seq_len = SP;
+  pd.x = base + p.off_xpad; pd.y = base + p.off_ypad; pd.mask = base + p.off_maskpad;
+  const int cap = num_cus * 8;
+  auto grid_for = [&](long long n) { const long long g = (n + 255) / 256; return (int)(g < cap ? g : cap); };
+  hipLaunchKernelGGL(k_pad_rows, dim3(grid_for((long long)c->batch * SP * (H / 8))), dim3(256), 0, st, static_cast<const half_t *>(x),
+                     reinterpret_cast<half_t *>(base + p.off_xpad), c->batch, c->seq_len, SP);
+  hipLaunchKernelGGL(k_pad_mask, dim3(grid_for((long long)c->batch * SP * SP)), dim3(256), 0, st, static_cast<const half_t *>(mask),
+                     reinterpret_cast<half_t *>(base + p.off_maskpad), c->batch, c->seq_len, SP);
+  SOUFFLE_HIP_TRY(hipGetLastError());
+  return SOUFFLE_OK;
+}
+static int pad_after(const Padded &pd, const souffle_bert_cfg *c, void *y, int num_cus, hipStream_t st) {
+  if (!pd.on) return SOUFFLE_OK;
+  const long long n = (long long)c->batch * c->seq_len * (H / 8);
+  const long long g = (n + 255) / 256;
+  hipLaunchKernelGGL(k_unpad_rows, dim3((int)(g < num_cus * 8 ? g : num_cus * 8)), dim3(256), 0, st, static_cast<const half_t *>(pd.y),
+                     static_cast<half_t *>(y), c->batch, c->seq_len, pd.cfg.seq_len);
+  SOUFFLE_HIP_TRY(hipGetLastError());
+  return SOUFFLE_OK;
+}
+
+static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *layers, int nl, const void *x_in,
+                     const void *mask_in, void *y_out, const souffle_bert_dump *dump, void *ws, size_t ws_bytes,
                      souffle_stream_t stream) {
   if (int rc = validate(c)) return rc;
   DeviceFacts df;
   if (int rc = device_facts(&df)) return rc;
   if (!df.cooperative) return fail(SOUFFLE_ERR_DEVICE, "device does not support cooperative launch");
   const Plan p = make_plan(c, nl);
+  Padded pd;
+  if (int rc = pad_before(pd, c, x_in, mask_in, y_out, dump, ws, ws_bytes, p, df.num_cus, static_cast<hipStream_t>(stream))) return rc;
+  if (pd.on) {
+    const int rc = run_fused(&pd.cfg, layers, nl, pd.x, pd.mask, pd.y, nullptr, ws, ws_bytes, stream);
+    return rc ? rc : pad_after(pd, c, y_out, df.num_cus, static_cast<hipStream_t>(stream));
+  }
+  const void *x = x_in, *mask = mask_in;
+  void *y = y_out;
   static thread_local Args a;
   if (int rc = fill_args(a, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
   stage_trace(&a.trace, &a.trace_cap, df.num_cus);
@@ -1543,6 +1640,12 @@ static int run_unfused(const souffle_bert_cfg *c, const souffle_bert_layer_w *la
   DeviceFacts df;
   if (int rc = device_facts(&df)) return rc;
   const Plan p = make_plan(c, nl);
+  Padded pd;
+  if (int rc = pad_before(pd, c, x, mask, y, dump, ws, ws_bytes, p, df.num_cus, static_cast<hipStream_t>(stream))) return rc;
+  if (pd.on) {
+    const int rc = run_unfused(&pd.cfg, layers, nl, pd.x, pd.mask, pd.y, nullptr, ws, ws_bytes, stream);
+    return rc ? rc : pad_after(pd, c, y, df.num_cus, static_cast<hipStream_t>(stream));
+  }
   static thread_local Args a;
   if (int rc = fill_args(a, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);

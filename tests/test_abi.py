@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
 def test_bert_validation_without_gpu():
     lib = sh.lib()
     assert lib.souffle_bert_workspace_bytes(None) == 0
-    bad = sh.BertCfg(1, 100, 768, 12, 3072, 0, 0.125, 1e-12, 1, 0)
+    bad = sh.BertCfg(1, 600, 768, 12, 3072, 0, 0.125, 1e-12, 1, 0)
     assert lib.souffle_bert_workspace_bytes(C.byref(bad)) == 0 and "seq_len" in sh.last_error()
     bad = sh.BertCfg(1, 128, 1024, 16, 4096, 0, 0.125, 1e-12, 1, 0)
     assert lib.souffle_bert_workspace_bytes(C.byref(bad)) == 0 and "hidden=768" in sh.last_error()

@@ -128,6 +128,38 @@ def test_dataflow_sync_equals_barrier_sync(B, S, layers):
     assert_close("encoder dataflow", y_1, oracle.bert_encoder(synth.bert_input(2, B, S), ws, B, S))
 
 
+@pytest.mark.parametrize("B,S,layers,masked", [(1, 100, 2, False), (2, 77, 1, True), (1, 200, 1, False), (3, 5, 1, False)])
+def test_sequence_lengths_that_are_not_built(B, S, layers, masked):
+    """Any length up to 512 runs as the next built one with the surplus keys masked out; the result is
+    that of the unpadded computation (oracle at the true length)."""
+    announce("bert encoder B=%d S=%d L=%d masked=%s" % (B, S, layers, masked))
+    import bert_binding
+    ws = [synth.bert_layer_weights(2, l, with_bias=True) for l in range(layers)]
+    x = synth.bert_input(5, B, S)
+    mask = None
+    if masked:
+        keep = synth.uniform01(synth.seed_of(0, 98), B * S * S).reshape(B, S, S) < 0.9
+        keep[:, :, 0] = True
+        mask = np.where(keep, 0.0, -10000.0).astype(np.float16)
+    ref = x
+    for w in ws:
+        ref = oracle.bert_layer(ref, w, B, S, mask=mask)
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    md = None if mask is None else dev(mask)
+    y_f = enc(dev(x), fused=True, mask=md).clone()
+    y_u = enc(dev(x), fused=False, mask=md).clone()
+    torch.cuda.synchronize()
+    assert tuple(y_f.shape) == (B * S, 768)
+    assert_close("encoder fused", y_f, ref)
+    assert torch.equal(y_f, y_u)
+    if layers == 1:
+        outs = run_layer(ws[0], x, B, S, 4, mask=md)
+        full = oracle.bert_layer(x, ws[0], B, S, mask=mask, dump=True)
+        for n, g, r in zip(NAMES, outs, full):
+            assert_close(n, g, r)
+        assert torch.equal(outs[-1], y_f)
+
+
 def test_layernorm_invariants_at_full_size():
     """Size-independent property: with gamma 1 / beta 0 every output row has mean 0, variance 1."""
     announce("bert LN invariants B=32")
@@ -143,7 +175,7 @@ def test_argument_errors_are_reported_not_fatal():
     import bert_binding
     import souffle_hip as sh
     w = dev_weights(synth.bert_layer_weights(0, 0))
-    x = torch.zeros(1, 100, 768, dtype=torch.float16, device="cuda:0")
+    x = torch.zeros(1, 600, 768, dtype=torch.float16, device="cuda:0")
     with pytest.raises(sh.SouffleError) as e:
         bert_binding.souffle_bert_layer(x, w["qkv_weight"], w["attn_fc_weight"], w["fc1_weight"], w["fc2_weight"], 4)
     assert e.value.code == -2 and "seq_len" in str(e.value)
