@@ -156,6 +156,16 @@ def bench_encoder(args, B, S, L, name):
                   "min_of_means_us_warm": mn, "median_us_warm": med, "parity": parity,
                   "launches_fused": 1, "launches_unfused": (6 if M < 1024 else 7) * L},
     }
+    # empirical ceilings of this device beside the published ones: device-to-device copy and an MFMA-only loop
+    try:
+        copy_gbs, mfma_tflops = sh.measured_ceilings()
+        roof["measured_copy_GBps"] = copy_gbs
+        roof["measured_mfma_f16_TFLOPs"] = mfma_tflops
+        roof["frac_of_measured"] = ach / (mfma_tflops if mfma_bound else copy_gbs)
+        if (B, S) == (1, 384):            # mixed shape: both fractions
+            roof["mfma_frac"] = flops / (cold_ev * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS
+    except sh.SouffleError as e:
+        roof["measured_ceilings_error"] = str(e)
     if cpu:
         res["cpu_baseline"] = cpu
         res["extra"]["gpu_speedup_vs_cpu"] = cpu["value"] / (cold_ev * 1e3)

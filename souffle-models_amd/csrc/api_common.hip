@@ -9,6 +9,7 @@
 #include <type_traits>
 #include <vector>
 #include "gemm_tile.hpp"
+#include "common.hpp"
 #include "host_util.hpp"
 
 namespace souffle {
@@ -156,6 +157,41 @@ extern "C" int souffle_device_info(souffle_devinfo *out) {
   out->cooperative_launch = p.cooperativeLaunch;
   out->wavefront_size = p.warpSize;
   strncpy(out->arch, p.gcnArchName, sizeof(out->arch) - 1);
+  return SOUFFLE_OK;
+}
+
+// MFMA-only loop for the empirical matrix-core ceiling: 8 independent 16x16x32 fp16 accumulator
+// tiles per wave, no memory traffic inside the loop.
+namespace souffle {
+__global__ void __launch_bounds__(256) k_mfma_probe(float *out, int iters) {
+  const int lane = threadIdx.x & 63;
+  h8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) { a[i] = (half_t)(0.001f * (lane + i)); b[i] = (half_t)(0.002f * (lane - i)); }
+  f4 acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = f4{0.f, 0.f, 0.f, 0.f};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = mfma_16x16x32(a, b, acc[j]);
+  }
+  f4 s = acc[0];
+#pragma unroll
+  for (int j = 1; j < 8; ++j) s += acc[j];
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = s[0] + s[1] + s[2] + s[3];
+}
+}  // namespace souffle
+
+extern "C" int souffle_mfma_probe(float *out, size_t out_bytes, int iters, double *flops, souffle_stream_t stream) {
+  if (!out) return fail(SOUFFLE_ERR_NULL, "out is NULL");
+  if (iters <= 0 || iters > (1 << 20)) return fail(SOUFFLE_ERR_SHAPE, "iters must be in 1..2^20 (got %d)", iters);
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  const int grid = df.num_cus * 2;                       // 8 waves per CU
+  if (out_bytes < (size_t)grid * 256 * 4) return fail(SOUFFLE_ERR_WORKSPACE, "out needs %zu bytes", (size_t)grid * 256 * 4);
+  hipLaunchKernelGGL(souffle::k_mfma_probe, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), out, iters);
+  SOUFFLE_HIP_TRY(hipGetLastError());
+  if (flops) *flops = (double)grid * 4 * iters * 8 * (2.0 * 16 * 16 * 32);
   return SOUFFLE_OK;
 }
 

@@ -10,6 +10,8 @@
 //     trip, no flags, no atomics) and the layers run as a true wavefront;
 //   - layer 0 consumes x_t (not the reference kernel's one-step-late x_{t-1}, :324-326),
 //     state and accumulation are fp32, weights fp16.
+//   - (tried: the 16 workgroups of a layer on one XCD with L2-scope polls for the recurrent
+//     hand-over; 258 us against 223 us, the write-through stores are not seen sooner through the L2);
 // Workgroup (l, g) owns hidden units [16g, 16g+16) of layer l: 64 gate rows x 512 inputs.
 // Lane layout inside a wave: unit = lane/16, gate = (lane/4)%4, column phase = lane%4, so
 // the four gates of a unit meet through three lane shuffles.
@@ -75,7 +77,8 @@ __global__ void __launch_bounds__(256) k_lstm(Args a) {
       if (!need0) v0 = a.x[(size_t)t * HID + tid];
       const u2 *p0 = below + (size_t)t * HID + tid, *p1 = own + (size_t)(t > 0 ? t - 1 : 0) * HID + tid;
       bool ok0 = !need0, ok1 = !need1;
-      for (int spin = 0; !(ok0 && ok1); ++spin) {
+      // once a wait has given up, later steps do not wait again: the launch is flagged as failed and ends quickly
+      for (int spin = 0; !(ok0 && ok1) && !failed; ++spin) {
         if (spin >= kMaxSpin) { failed = true; break; }
         // (a slot that is already in is polled again: harmless, and the loop stays branch-free)
         const u2 q0 = ld8_atomic(p0), q1 = ld8_atomic(p1);

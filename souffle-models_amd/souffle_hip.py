@@ -76,6 +76,7 @@ SIGNATURES = {
     "souffle_last_error": (C.c_char_p, []),
     "souffle_version": (C.c_char_p, []),
     "souffle_device_info": (C.c_int, [C.POINTER(DevInfo)]),
+    "souffle_mfma_probe": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double), C.c_void_p]),
     "souffle_set_stage_trace": (C.c_int, [C.c_void_p, C.c_size_t]),
     "souffle_set_cooperative_launch": (C.c_int, [C.c_int]),
     "souffle_workspace_init": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
@@ -210,6 +211,26 @@ def device_info():
     info = DevInfo()
     check(lib().souffle_device_info(C.byref(info)))
     return {n: (getattr(info, n).decode() if n == "arch" else getattr(info, n)) for n, _ in DevInfo._fields_}
+
+
+def measured_ceilings(device="cuda:0"):
+    """Empirical ceilings of this device: (device-to-device copy GB/s counting read + written bytes,
+    MFMA-only fp16 TFLOP/s).  Synchronises."""
+    import torch
+    n = 1 << 30
+    a = torch.empty(n, dtype=torch.uint8, device=device).fill_(1)
+    b = torch.empty_like(a)
+    mn, _ = bench_us(lambda: b.copy_(a), warmup=3, rounds=3, repeat=5)
+    copy_gbs = 2.0 * n / (mn * 1e-6) / 1e9
+    del a, b
+    out = torch.empty(device_info()["num_cus"] * 512, dtype=torch.float32, device=device)
+    flops = C.c_double()
+    iters = 50000
+
+    def probe():
+        check(lib().souffle_mfma_probe(out.data_ptr(), out.numel() * 4, iters, C.byref(flops), current_stream()))
+    mn, _ = bench_us(probe, warmup=2, rounds=3, repeat=3)
+    return copy_gbs, flops.value / (mn * 1e-6) / 1e12
 
 
 def bench_us(launch, warmup=20, rounds=10, repeat=100, stream=None):

@@ -160,6 +160,14 @@ def test_sequence_lengths_that_are_not_built(B, S, layers, masked):
         assert torch.equal(outs[-1], y_f)
 
 
+def test_souffle_bert_base_module():
+    """The reference's zero-weight 12-layer driver (cpp/bert/bert_base_impl.cu:277-308): returns 0."""
+    announce("souffle_bert_base")
+    import souffle_bert_base
+    assert souffle_bert_base.souffle_bert_base() == 0
+    assert souffle_bert_base.souffle_bert_base(seq_len=128, fused=True) == 0
+
+
 def test_layernorm_invariants_at_full_size():
     """Size-independent property: with gamma 1 / beta 0 every output row has mean 0, variance 1."""
     announce("bert LN invariants B=32")
