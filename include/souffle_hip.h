@@ -51,7 +51,7 @@ typedef struct {
   char arch[64];
 } souffle_devinfo;
 int souffle_device_info(souffle_devinfo *out);
-/* Queues one MFMA-only kernel (8 waves per CU, `iters` x 8 independent fp16 16x16x32 MFMAs per wave, no
+/* Queues one MFMA-only kernel (4 waves per CU, `iters` x 16 independent fp16 16x16x32 MFMAs per wave, no
  * memory traffic) and reports the flops it performs: timed by the caller, it gives the empirical
  * matrix-core ceiling that the published peak is compared with.  `out` takes 2 KiB per CU of results. */
 int souffle_mfma_probe(float *out, size_t out_bytes, int iters, double *flops, souffle_stream_t stream);

@@ -225,7 +225,7 @@ def measured_ceilings(device="cuda:0"):
     del a, b
     out = torch.empty(device_info()["num_cus"] * 512, dtype=torch.float32, device=device)
     flops = C.c_double()
-    iters = 50000
+    iters = 25000
 
     def probe():
         check(lib().souffle_mfma_probe(out.data_ptr(), out.numel() * 4, iters, C.byref(flops), current_stream()))
