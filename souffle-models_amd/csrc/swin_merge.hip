@@ -15,7 +15,7 @@
 namespace souffle {
 namespace swin_merge {
 
-using Tile = GemmTile<64, 64, 64, 2, 2>;
+using Tile = GemmTile<64, 64, 128, 2, 2>;      // K = 4C advances in 4C/128 steps: the kernel is a chain of memory latencies
 
 struct Args {
   int H, W, C, M, K, N;
@@ -63,7 +63,7 @@ __global__ void __launch_bounds__(256) k_patch_merge(const Args a) {
       }
     }
     __syncthreads();
-    Tile::run(gl, a.w, a.N, m0, n0, 0, a.K / 64,
+    Tile::run(gl, a.w, a.N, m0, n0, 0, a.K / Tile::kBK,
               [&](int m, int k) {
                 if (m >= a.M) return u4{0u, 0u, 0u, 0u};
                 const h8 v = as_h8(*reinterpret_cast<const u4 *>(a.x + source(m, k)));
@@ -109,6 +109,11 @@ extern "C" int souffle_swin_patch_merge(const void *x, const void *ln_g, const v
   const int items = ((a.M + 63) / 64) * (a.N / 64);
   const int grid = items < df.num_cus * 2 ? items : df.num_cus * 2;
   const size_t lds = swin_merge::Tile::LDS_BYTES + 64 * 2 * sizeof(float);
+  static bool attr_done = false;
+  if (!attr_done) {
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)swin_merge::k_patch_merge, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_done = true;
+  }
   hipLaunchKernelGGL(swin_merge::k_patch_merge, dim3(grid), dim3(256), lds, static_cast<hipStream_t>(stream), a);
   SOUFFLE_HIP_TRY(hipGetLastError());
   return SOUFFLE_OK;
