@@ -164,6 +164,14 @@ def bench_encoder(args, B, S, L, name):
         roof["frac_of_measured"] = ach / (mfma_tflops if mfma_bound else copy_gbs)
         if (B, S) == (1, 384):            # mixed shape: both fractions
             roof["mfma_frac"] = flops / (cold_ev * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS
+        if M < 1024:
+            # what a chain of this many dependent grid-wide stages costs with no arithmetic at all
+            nst = 6 * L
+            bar_us, floor_us = sh.stage_floor_us(nst)
+            res["extra"]["stages_per_launch"] = nst
+            res["extra"]["barriers_only_us"] = bar_us
+            res["extra"]["stage_chain_floor_us"] = floor_us
+            res["extra"]["frac_of_stage_chain_floor"] = floor_us / (cold_ev * 1e3)
     except sh.SouffleError as e:
         roof["measured_ceilings_error"] = str(e)
     if cpu:

@@ -54,6 +54,12 @@ int souffle_device_info(souffle_devinfo *out);
 /* Queues one MFMA-only kernel (4 waves per CU, `iters` x 16 independent fp16 16x16x32 MFMAs per wave, no
  * memory traffic) and reports the flops it performs: timed by the caller, it gives the empirical
  * matrix-core ceiling that the published peak is compared with.  `out` takes 2 KiB per CU of results. */
+/* Queues a persistent kernel of `stages` dependent grid-wide stages without arithmetic on an initialised
+ * workspace (souffle_workspace_init; 16 KiB are enough).  mode 0: the grid barrier alone; mode 1: 16 bytes
+ * written through, the barrier, and a read of what a workgroup of another XCD wrote, per stage.  Timed by
+ * the caller it gives the latency floor of a chain of dependent stages on this device, which bounds the
+ * skinny shapes (B*S < 1024) rather than the HBM or MFMA roofline. */
+int souffle_stage_floor_probe(void *workspace, size_t workspace_bytes, int stages, int mode, souffle_stream_t stream);
 int souffle_mfma_probe(float *out, size_t out_bytes, int iters, double *flops, souffle_stream_t stream);
 
 /* Zero the control block at the head of a workspace (stream-ordered, no allocation).

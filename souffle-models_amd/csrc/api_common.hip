@@ -198,6 +198,46 @@ extern "C" int souffle_mfma_probe(float *out, size_t out_bytes, int iters, doubl
   return SOUFFLE_OK;
 }
 
+// The floor of a chain of dependent grid-wide stages on this device: `n` stages that do nothing but
+// hand a value on.  mode 0: the grid barrier alone.  mode 1: every workgroup writes 16 bytes through,
+// passes the barrier, and reads the 16 bytes another workgroup (on another XCD) wrote; what it reads
+// goes into what it writes next, so each stage costs a store acknowledgement, a barrier and one
+// memory round trip, like a real stage with no arithmetic.
+namespace souffle {
+__global__ void __launch_bounds__(256) k_stage_floor(unsigned *ctl, u4 *buf, int n, int mode, unsigned *out) {
+  GridBarrier bar;
+  grid_barrier_begin(bar, ctl);
+  const int grid = gridDim.x, peer = (blockIdx.x + 37) % grid;
+  u4 v = {blockIdx.x, 1u, 2u, 3u};
+  for (int i = 0; i < n; ++i) {
+    if (mode && threadIdx.x == 0) st16<true>(buf, ((i & 1) * grid + (int)blockIdx.x) * 16, v);
+    grid_sync(bar);
+    if (mode) {
+      const u4 r = ld16<true>(buf, ((i & 1) * grid + peer) * 16);
+      v = u4{v[0] + r[0], v[1] ^ r[1], v[2] + 1u, r[3]};
+    }
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = v[0] + v[1] + v[2] + v[3];
+  grid_barrier_end(bar);
+}
+}  // namespace souffle
+
+extern "C" int souffle_stage_floor_probe(void *ws, size_t ws_bytes, int stages, int mode, souffle_stream_t stream) {
+  if (!ws) return fail(SOUFFLE_ERR_NULL, "workspace is NULL");
+  if (stages <= 0 || stages > 100000) return fail(SOUFFLE_ERR_SHAPE, "stages must be in 1..100000 (got %d)", stages);
+  if (mode != 0 && mode != 1) return fail(SOUFFLE_ERR_SHAPE, "mode must be 0 or 1");
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  const size_t ctl_bytes = round_up(kCtlWords * 4, 256), need = ctl_bytes + (size_t)df.num_cus * (2 * 16 + 4);
+  if (ws_bytes < need) return fail(SOUFFLE_ERR_WORKSPACE, "workspace too small: need %zu bytes", need);
+  if (!aligned16(ws)) return fail(SOUFFLE_ERR_ALIGN, "workspace must be 16-byte aligned");
+  unsigned *ctl = static_cast<unsigned *>(ws);
+  u4 *buf = reinterpret_cast<u4 *>(static_cast<char *>(ws) + ctl_bytes);
+  unsigned *out = reinterpret_cast<unsigned *>(static_cast<char *>(ws) + ctl_bytes + (size_t)df.num_cus * 32);
+  void *args[] = {&ctl, &buf, &stages, &mode, &out};
+  return launch_persistent((const void *)souffle::k_stage_floor, df.num_cus, 256, args, 0, static_cast<hipStream_t>(stream));
+}
+
 extern "C" int souffle_set_cooperative_launch(int on) {
   souffle::g_cooperative.store(on ? 1 : 0);
   return SOUFFLE_OK;

@@ -76,6 +76,7 @@ SIGNATURES = {
     "souffle_last_error": (C.c_char_p, []),
     "souffle_version": (C.c_char_p, []),
     "souffle_device_info": (C.c_int, [C.POINTER(DevInfo)]),
+    "souffle_stage_floor_probe": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]),
     "souffle_mfma_probe": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double), C.c_void_p]),
     "souffle_set_stage_trace": (C.c_int, [C.c_void_p, C.c_size_t]),
     "souffle_set_cooperative_launch": (C.c_int, [C.c_int]),
@@ -211,6 +212,21 @@ def device_info():
     info = DevInfo()
     check(lib().souffle_device_info(C.byref(info)))
     return {n: (getattr(info, n).decode() if n == "arch" else getattr(info, n)) for n, _ in DevInfo._fields_}
+
+
+def stage_floor_us(stages, device="cuda:0"):
+    """(barrier only, barrier + hand-over) time in us of `stages` dependent grid-wide stages without
+    arithmetic: the latency floor of a persistent kernel with that many stages.  Synchronises."""
+    ws = Workspace(16384, device)
+    res = []
+    for mode in (0, 1):
+        def probe():
+            check(lib().souffle_stage_floor_probe(ws.ptr, ws.nbytes, stages, mode, current_stream()))
+        mn, _ = bench_us(probe, warmup=3, rounds=3, repeat=10)
+        res.append(mn)
+    if ws.status() != 0:
+        raise SouffleError(-4, "a bounded wait inside the probe gave up")
+    return tuple(res)
 
 
 def measured_ceilings(device="cuda:0"):
