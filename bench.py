@@ -122,6 +122,15 @@ def bench_encoder(args, B, S, L, name):
     cold_wall, cold_ev = time_steps(lambda i: encs[i % len(encs)](x, out=out), args.steps, args.warmup)
     warm_wall, warm_ev = time_steps(lambda i: encs[0](x, out=out), args.steps, args.warmup)
     unf_wall, unf_ev = time_steps(lambda i: encs[i % len(encs)](x, out=out, fused=False), max(10, args.steps // 4), 5)
+    # the per-op chain again as one HIP graph (no launch gaps): the strongest form of the unfused baseline
+    graph_ev = None
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            encs[0](x, out=out, fused=False)
+        _, graph_ev = time_steps(lambda i: g.replay(), max(10, args.steps // 4), 5)
+    except Exception as e:                      # a capture failure must not cost the headline number
+        print("graph capture of the per-op chain failed: %s" % e, file=sys.stderr)
     # the reference's own timing rule (min over rounds of the mean of repeated event-timed launches)
     mn, med = sh.bench_us(lambda: encs[0](x, out=out), warmup=10, rounds=5, repeat=max(10, args.steps // 5))
 
@@ -153,6 +162,7 @@ def bench_encoder(args, B, S, L, name):
         "roofline": roof,
         "extra": {"per_layer_us_cold": cold_ev * 1e3 / L, "warm_cache_us": warm_ev * 1e3, "per_layer_us_warm": warm_ev * 1e3 / L,
                   "unfused_per_op_us": unf_ev * 1e3, "fused_speedup_vs_unfused": unf_ev / cold_ev,
+                  "unfused_per_op_hip_graph_us": None if graph_ev is None else graph_ev * 1e3,
                   "min_of_means_us_warm": mn, "median_us_warm": med, "parity": parity,
                   "launches_fused": 1, "launches_unfused": (6 if M < 1024 else 7) * L},
     }

@@ -160,6 +160,34 @@ def test_sequence_lengths_that_are_not_built(B, S, layers, masked):
         assert torch.equal(outs[-1], y_f)
 
 
+@pytest.mark.parametrize("fused", [True, False])
+def test_encoder_replays_from_a_hip_graph(fused):
+    """The entry points allocate nothing and queue only kernels, so a caller may capture them: a graph
+    of the encoder is replayed several times, with eager launches and synchronisations in between, and
+    every replay must give the eager result."""
+    announce("bert encoder in a HIP graph fused=%s" % fused)
+    import bert_binding
+    B, S, layers = 1, 128, 3
+    ws = [synth.bert_layer_weights(2, l) for l in range(layers)]
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    x1, x2 = dev(synth.bert_input(2, B, S)), dev(synth.bert_input(3, B, S))
+    eager1, eager2 = enc(x1, fused=fused).clone(), enc(x2, fused=fused).clone()
+    xin = x1.clone()
+    out = torch.empty_like(eager1)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        enc(xin, out=out, fused=fused)
+    for i, (xs, ref) in enumerate([(x1, eager1), (x2, eager2), (x1, eager1), (x2, eager2)]):
+        xin.copy_(xs)
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref), "replay %d differs from the eager result" % i
+        assert torch.equal(enc(xs, fused=fused), ref)          # eager work between the replays
+    assert enc.ws.status() == 0
+
+
 def test_souffle_bert_base_module():
     """The reference's zero-weight 12-layer driver (cpp/bert/bert_base_impl.cu:277-308): returns 0."""
     announce("souffle_bert_base")
