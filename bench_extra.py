@@ -110,7 +110,7 @@ def bench_se(args):
     from bench import time_steps
     shapes = [(32, 112, 8), (96, 56, 4), (144, 56, 6), (144, 28, 6), (240, 28, 10), (240, 14, 10), (480, 14, 20),
               (672, 14, 28), (672, 7, 28), (1152, 7, 48)]
-    a100 = [23.33, 14.14, 15.65, 12.48, 12.86, 12.03, 12.86, 13.86, 13.28, 15.36]   # reference xlsx, A100
+    a100 = [23.33, 14.14, 15.65, 12.48, 12.86, 12.03, 12.86, 13.86, 13.28, 15.36]   # cpp/efficientnet/scripts/efficientnet-se_module_v2-max-block.xlsx, column "Duration [usecond]", A100
     rows = []
     for (Cc, Hh, R), ref_us in zip(shapes, a100):
         x = torch.rand((1, Cc, Hh, Hh), device="cuda:0")
