@@ -6,7 +6,8 @@
 // (:173-195), the squeeze-excite operators (reduce_mean :131-141, se_module_pointwise_conv
 // :270-282, fused_pointwise_conv_bias_add_sigmoid_mul :252-267) and pointwise_conv2d_bn
 // (:41-57) / pointwise_conv2d_bn_short_cut_add (:83-101).  The reference launches 7 to 9
-// kernels per block; here a block is three stages of one launch, separated by grid barriers:
+// kernels per block; here a block is three stages of one launch (four barrier-separated steps:
+// the depthwise stage has a barrier of its own in the middle):
 //
 //   expand   : E = swish(bn(X . We^T))                      one 16x16 MFMA tile per wave
 //   depthwise: D = swish(bn(dwconv(E))), and per workgroup the contribution of its pixels or
@@ -16,11 +17,11 @@
 //   project  : Y = bn((D * gate) . Wp^T) (+ X), the gate applied to the activation operand on
 //              its way into the MFMA
 //
-// The whole network moves 0.4 GFLOP over ~7 MB of weights and ~12 MB of activations: every
-// stage is latency bound, so the design goal is few, short stages, not MFMA utilisation.  The
-// GEMMs therefore take both operands straight from global memory/L2 in MFMA operand layout
-// (weights are [out][in], as pointwise_conv2d_bn stores them, so a lane's 8 consecutive
-// k-values are one 16-byte load): no LDS staging, no workgroup barrier inside a stage.
+// The whole network moves 0.7 GFLOP over ~7 MB of weights and ~12 MB of activations: every
+// stage is latency bound, so the design goal is few, short stages with all their loads in flight
+// at once, not MFMA utilisation.  The GEMMs therefore take both operands straight from global
+// memory/L2 in MFMA operand layout (weights are [out][in], as pointwise_conv2d_bn stores them, so
+// a lane's 8 consecutive k-values are one 16-byte load): no LDS staging of operands.
 //
 // Activations written by one stage and read by the next are stored write-through and read
 // with agent-coherent loads: tiles of 16 output channels of neighbouring pixels share cache
