@@ -217,6 +217,11 @@ typedef struct {   /* fp16 device pointers, biases / LN vectors nullable */
   const void *w_fc2, *b_fc2;    /* [rC][C] */
 } souffle_swin_block_w;
 size_t souffle_swin_workspace_bytes(const souffle_swin_cfg *cfg);
+/* How souffle_swin_block_pair_fused spreads a window: on != 0 (default) four workgroups per window (one
+ * attention head and a quarter of the MLP each, two hand-overs through memory per block) while there are
+ * at most half as many windows as CUs; 0: one workgroup per window.  SOUFFLE_SWIN_SPLIT=0 sets the
+ * initial value.  Same arithmetic up to the order of the fp32 additions of FC2. */
+int souffle_set_swin_split(int on);
 /* Regular + shifted window block in one cooperative launch.  The op list is
  * python/models/swin_transformer/swin_transformer_main.py:11-61 (Part-1..8), which the
  * reference only runs as separate TVM kernels (:196-330).  x,y: fp16 [H*W][C]. */

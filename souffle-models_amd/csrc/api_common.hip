@@ -51,6 +51,16 @@ int device_facts(DeviceFacts *out) {
 
 static void *g_trace_buf = nullptr;
 static size_t g_trace_bytes = 0;
+static std::atomic<int> g_swin_split{-1};
+int swin_split_mode() {
+  int v = g_swin_split.load();
+  if (v < 0) {
+    const char *e = getenv("SOUFFLE_SWIN_SPLIT");
+    v = (e && e[0] == '0') ? 0 : 1;
+    g_swin_split.store(v);
+  }
+  return v;
+}
 static std::atomic<int> g_bert_sync{-1};
 int bert_sync_mode() {
   int v = g_bert_sync.load();
@@ -240,6 +250,11 @@ extern "C" int souffle_stage_floor_probe(void *ws, size_t ws_bytes, int stages, 
 
 extern "C" int souffle_set_cooperative_launch(int on) {
   souffle::g_cooperative.store(on ? 1 : 0);
+  return SOUFFLE_OK;
+}
+
+extern "C" int souffle_set_swin_split(int on) {
+  souffle::g_swin_split.store(on ? 1 : 0);
   return SOUFFLE_OK;
 }
 

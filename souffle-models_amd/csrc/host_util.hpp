@@ -23,6 +23,9 @@ struct DeviceFacts {
 // Cached per process for the current device; returns a negative status on failure.
 int device_facts(DeviceFacts *out);
 
+// 1: the Swin block pair runs four workgroups per window (souffle_set_swin_split / SOUFFLE_SWIN_SPLIT).
+int swin_split_mode();
+
 // SOUFFLE_SYNC_* selected by souffle_set_bert_sync / SOUFFLE_BERT_SYNC.
 int bert_sync_mode();
 

@@ -33,6 +33,9 @@ struct Args {
   half_t *mid, *y;
   unsigned *ctl;
   unsigned long long *trace;   // optional phase stamps: trace[block * 32 + phase] (development aid)
+  half_t *xctx;                // quad kernel: [window][64][C] attention output, a head's columns written by its workgroup
+  float *xpart;                // quad kernel: [window][head][64][C] fp32 FC2 partial sums
+  unsigned *xflags;            // quad kernel: [window][16] hand-over words (4 used)
   BlockW w[2];
 };
 
@@ -410,6 +413,298 @@ __global__ void __launch_bounds__(256) k_block_pair(Args a) {
   grid_barrier_end(bar);
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Four workgroups per window.  A window's block is bound by how fast ONE CU can take in the 393 KB
+// of weights (a direct-to-LDS load occupies the CU's load unit ~57 cycles per KB, and the issuing
+// wave with it) while three quarters of the CUs idle (64 windows, 256 CUs).  Here workgroup h of a
+// window owns attention head h, the h-th quarter of FC1's columns and the matching quarter of FC2's
+// K range, so it takes in 120 KB per block:
+//   LN1 (all rows, redundantly) -> Q_h, K_h, V_h -> attention of head h (one query tile per wave)
+//   -> [hand-over 1: the four heads' context columns, fp16, through memory]
+//   -> projection + shortcut (all columns, redundantly: 32 KB of weights) -> LN2
+//   -> H_h = gelu(LN2 . W1[:, quarter h]) -> P_h = H_h . W2[quarter h, :] (fp32 partial sums)
+//   -> [hand-over 2: partial sums through memory] -> workgroup h adds the four partials, the bias
+//      and the shortcut for output columns [32h, 32h+32) in a fixed order and stores them.
+// A hand-over is a write-through store of the data, one flag word per workgroup, and a bounded poll
+// of the three other flags.  Flag values grow from launch to launch (they are derived from the
+// grid barrier's launch-persistent count), so nothing is reset.
+constexpr int QN = 32, QCHUNK_BYTES = CHUNK_K * QN * 2, QCHUNKS = 15, QLOADS = QCHUNK_BYTES / 1024 / 4;
+static_assert(F / NH == CHUNK_K && HD == QN, "a head's FC2 share is one chunk deep, its q/k/v slices one chunk wide");
+
+__device__ __forceinline__ Chunk qchunk_of(const BlockW &w, int c, int h) {
+  if (c < 3) return Chunk{w.w_qkv, 3 * C, 0, c * C + h * HD};
+  if (c < 7) return Chunk{w.w_proj, C, 0, (c - 3) * QN};
+  if (c < 11) return Chunk{w.w_fc1, F, 0, h * (F / NH) + (c - 7) * QN};
+  return Chunk{w.w_fc2, C, h * (F / NH), (c - 11) * QN};
+}
+// W[128 k][32 n] chunk: slot(k, c4) = 4 k + (c4 ^ (k & 2)) (16-byte slots), for the transposing read.
+__device__ __forceinline__ void qring_issue(WeightRing &r, const BlockW &w, int c, int h) {
+  const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6;
+  const Chunk ch = qchunk_of(w, c, h);
+  const unsigned base = r.lds_addr + (r.issued % RING) * QCHUNK_BYTES;
+#pragma unroll
+  for (int q = 0; q < QLOADS; ++q) {
+    const int inst = q * 4 + wave, sl = inst * 64 + lane, k = sl >> 2, c4 = (sl & 3) ^ (k & 2);
+    load_lds16(ch.W + (size_t)(ch.k0 + k) * ch.ldw + ch.n0 + c4 * 8, base + inst * 1024);
+  }
+  r.issued++;
+}
+__device__ __forceinline__ const unsigned char *qring_take(WeightRing &r) {
+  const int more = r.issued - r.used - 1;
+  if (more >= 2) wait_vmcnt<2 * QLOADS>();
+  else if (more == 1) wait_vmcnt<QLOADS>();
+  else wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  const unsigned char *buf = r.lds + (r.used % RING) * QCHUNK_BYTES;
+  r.used++;
+  return buf;
+}
+// acc[j] (rows 16 wave .. +15, columns 16 j .. +15 of the chunk) += A[rows][ka .. ka+128) . chunk
+__device__ __forceinline__ void qchunk_mma(const unsigned char *buf, const half_t *A, int lda, int ka, f4 (&acc)[2]) {
+  const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+  const half_t *ws = reinterpret_cast<const half_t *>(buf);
+  h8 xop[CHUNK_K / 32], wop[CHUNK_K / 32][2];
+#pragma unroll
+  for (int ks = 0; ks < CHUNK_K / 32; ++ks) {
+    xop[ks] = *reinterpret_cast<const h8 *>(A + (wave * 16 + l16) * lda + ka + ks * 32 + g * 8);
+    const int k = ks * 32 + g * 8 + (l16 >> 2);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c4 = j * 2 + ((l16 & 3) >> 1);
+      const half_t *p = ws + (k * 4 + (c4 ^ (k & 2))) * 8 + (l16 & 1) * 4;
+      const h4 lo = lds_read_tr16(p), hi = lds_read_tr16(p + 4 * QN);
+      wop[ks][j] = h8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+  }
+#pragma unroll
+  for (int ks = 0; ks < CHUNK_K / 32; ++ks)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[j] = mfma_16x16x32(wop[ks][j], xop[ks], acc[j]);
+}
+// This workgroup's data of a hand-over are written: publish `val` in its flag word, then wait until
+// the window's four words have reached it.  Every thread calls it; the wait is bounded.
+__device__ __forceinline__ void quad_handover(unsigned *flags, unsigned *ctl, int win, int h, unsigned val) {
+  __builtin_amdgcn_s_waitcnt(0);                 // the write-through stores are acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0) __hip_atomic_store(flags + win * 16 + h, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x < 64) {
+    for (int spin = 0; spin < kMaxBarrierSpin; ++spin) {
+      bool ok = true;
+      if (threadIdx.x < NH)
+        ok = (int)(__hip_atomic_load(flags + win * 16 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - val) >= 0;
+      if (__all(ok)) break;
+      __builtin_amdgcn_s_sleep(1);
+      if (spin == kMaxBarrierSpin - 1 && threadIdx.x == 0)   // gave up: the launch's output is invalid
+        (void)__hip_atomic_fetch_or(ctl + kCtlErrWord, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  __syncthreads();
+}
+
+// One block for one window, as workgroup h of its four.  fv: the flag value of this block's first hand-over.
+__device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, const Args &a, const BlockW &w, const BlockW *next,
+                                      int shift, const half_t *xin, half_t *xout, int win, int h, unsigned fv) {
+  half_t *zs = reinterpret_cast<half_t *>(lds + OFF_ZS);
+  half_t *big = reinterpret_cast<half_t *>(lds + OFF_BIG);
+  half_t *x1s = reinterpret_cast<half_t *>(lds + OFF_X1);
+  float *tab = reinterpret_cast<float *>(lds + OFF_TAB);
+  int *tok = reinterpret_cast<int *>(lds + OFF_TOK);
+  int *reg = reinterpret_cast<int *>(lds + OFF_REG);
+  half_t *par = reinterpret_cast<half_t *>(lds + OFF_PAR);
+  const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+  const int nww = a.Ww / WS;
+  const int first_chunk = ring.used;
+  auto top_up = [&]() {
+    const int c = ring.issued - first_chunk;
+    if (c < QCHUNKS) qring_issue(ring, w, c, h);
+    else if (next && c < QCHUNKS + 2) qring_issue(ring, *next, c - QCHUNKS, h);
+  };
+  auto gemm_chunk = [&](const half_t *A, int lda, int ka, f4 (&acc)[2]) {
+    const unsigned char *buf = qring_take(ring);
+    top_up();
+    acc[0] = acc[1] = f4{0.f, 0.f, 0.f, 0.f};
+    qchunk_mma(buf, A, lda, ka, acc);
+  };
+  const int row = wave * 16 + l16;
+
+  __syncthreads();
+  while (ring.issued < first_chunk + 2) top_up();
+  if (tid < NP) {
+    int t = -1, rg = 0;
+    if (tid < N) {
+      const int i = (win / nww) * WS + tid / WS, j = (win % nww) * WS + tid % WS;
+      t = ((i + shift) % a.Hh) * a.Ww + (j + shift) % a.Ww;
+      if (shift > 0) rg = 3 * region_of(i, a.Hh, shift) + region_of(j, a.Ww, shift);
+    }
+    tok[tid] = t;
+    reg[tid] = rg;
+  }
+  for (int i = tid; i < TAB * NH; i += 256) tab[i] = w.rel_table ? (float)w.rel_table[i] : 0.f;
+  {
+    auto copy = [&](int off, const half_t *src, int n, float dflt) {
+      for (int i = tid; i < n; i += 256) par[off + i] = src ? src[i] : (half_t)dflt;
+    };
+    copy(P_BQKV, w.b_qkv, 3 * C, 0.f); copy(P_BPROJ, w.b_proj, C, 0.f); copy(P_BFC1, w.b_fc1, F, 0.f); copy(P_BFC2, w.b_fc2, C, 0.f);
+    copy(P_G1, w.ln1_g, C, 1.f); copy(P_B1, w.ln1_b, C, 0.f); copy(P_G2, w.ln2_g, C, 1.f); copy(P_B2, w.ln2_b, C, 0.f);
+  }
+  __syncthreads();
+
+  // LN1 of the gathered rows (kept in x1s as the shortcut of the projection)
+  layernorm_rows([&](int r, int c) {
+    const u4 v = ld16<true>(xin, (tok[r] * C + c) * 2);
+    *reinterpret_cast<u4 *>(x1s + r * ZLD + c) = v;
+    return v;
+  }, zs, par + P_G1, par + P_B1, a.eps);
+  __syncthreads();
+
+  // Q_h (pre-scaled), K_h, V_h in big[:, 0..32), [32..64), [64..96)
+  const float qscale = rsqrtf((float)HD);
+  for (int c = 0; c < 3; ++c) {
+    f4 acc[2];
+    gemm_chunk(zs, ZLD, 0, acc);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int nl = j * 16 + g * 4;
+      f4 v = add_bias4(acc[j], par + P_BQKV, c * C + h * HD + nl);
+      if (c == 0) v *= qscale;
+      *reinterpret_cast<u2 *>(big + row * BLD + c * HD + nl) = pack_h4(v);
+    }
+  }
+  __syncthreads();
+
+  // attention of head h: wave = query tile
+  {
+    const int q = wave * 16 + l16;
+    const h8 qop = *reinterpret_cast<const h8 *>(big + q * BLD + g * 8);
+    f4 sc[NP / 16];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < NP / 16; ++t) {
+      const h8 kop = *reinterpret_cast<const h8 *>(big + (t * 16 + l16) * BLD + HD + g * 8);
+      f4 s = mfma_16x16x32(kop, qop, f4{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int key = t * 16 + g * 4 + v;
+        if (key >= N) s[v] = -INFINITY;
+        else if (q < N) {
+          const int di = q / WS - key / WS + WS - 1, dj = q % WS - key % WS + WS - 1;
+          s[v] += tab[(di * (2 * WS - 1) + dj) * NH + h];
+          if (a.use_mask && reg[q] != reg[key]) s[v] += -100.0f;
+        }
+        mx = fmaxf(mx, s[v]);
+      }
+      sc[t] = s;
+    }
+    mx = fmaxf(mx, wave_xor(mx, 16));
+    mx = fmaxf(mx, wave_xor(mx, 32));
+    float sum = 0.f;
+#pragma unroll
+    for (int t = 0; t < NP / 16; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) { sc[t][v] = __expf(sc[t][v] - mx); sum += sc[t][v]; }
+    sum += wave_xor(sum, 16);
+    sum += wave_xor(sum, 32);
+    const float inv = 1.0f / sum;
+    f4 o[HD / 16];
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) o[dt] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < NP / 16; ++t) {
+      const f4 pr = sc[t] * inv;
+      const h4 p = {(half_t)pr[0], (half_t)pr[1], (half_t)pr[2], (half_t)pr[3]};
+#pragma unroll
+      for (int dt = 0; dt < HD / 16; ++dt) {
+        const h4 vop = lds_read_tr16(big + (t * 16 + g * 4 + (l16 >> 2)) * BLD + 2 * HD + dt * 16 + (l16 & 3) * 4);
+        o[dt] = mfma_16x16x16(vop, p, o[dt]);
+      }
+    }
+    // this head's context columns: into zs for this workgroup, through memory for the three others
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) {
+      const u2 pk = pack_h4(o[dt]);
+      *reinterpret_cast<u2 *>(zs + q * ZLD + h * HD + dt * 16 + g * 4) = pk;
+      st8<true>(a.xctx, ((win * NP + q) * C + h * HD + dt * 16 + g * 4) * 2, pk);
+    }
+  }
+  quad_handover(a.xflags, a.ctl, win, h, fv);
+  for (int idx = tid; idx < NP * (C / 8); idx += 256) {
+    const int r = idx / (C / 8), c8 = idx % (C / 8);
+    if (c8 / (HD / 8) != h) *reinterpret_cast<u4 *>(zs + r * ZLD + c8 * 8) = ld16<true>(a.xctx, ((win * NP + r) * C + c8 * 8) * 2);
+  }
+  __syncthreads();
+
+  // x1 = x + ctx.Wproj + b (all columns, in every workgroup of the window)
+  for (int nt = 0; nt < C / QN; ++nt) {
+    f4 acc[2];
+    gemm_chunk(zs, ZLD, 0, acc);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = nt * QN + j * 16 + g * 4;
+      f4 v = f4{0.f, 0.f, 0.f, 0.f};
+      if (row < N) {
+        const h4 sh = *reinterpret_cast<const h4 *>(x1s + row * ZLD + n);
+        v = add_bias4(acc[j], par + P_BPROJ, n) + f4{(float)sh[0], (float)sh[1], (float)sh[2], (float)sh[3]};
+      }
+      *reinterpret_cast<u2 *>(x1s + row * ZLD + n) = pack_h4(v);
+    }
+  }
+  __syncthreads();
+  layernorm_rows([&](int r, int c) { return *reinterpret_cast<const u4 *>(x1s + r * ZLD + c); }, zs, par + P_G2, par + P_B2, a.eps);
+  __syncthreads();
+
+  // H_h = gelu(Z2 . W1[:, quarter h] + b1) in big[:, 0..128)
+  for (int nt = 0; nt < (F / NH) / QN; ++nt) {
+    f4 acc[2];
+    gemm_chunk(zs, ZLD, 0, acc);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int nl = nt * QN + j * 16 + g * 4;
+      f4 v = add_bias4(acc[j], par + P_BFC1, h * (F / NH) + nl);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = gelu_tanh(v[i]);
+      *reinterpret_cast<u2 *>(big + row * BLD + nl) = pack_h4(v);
+    }
+  }
+  __syncthreads();
+
+  // P_h = H_h . W2[quarter h, :], fp32, through memory
+  for (int nt = 0; nt < C / QN; ++nt) {
+    f4 acc[2];
+    gemm_chunk(big, BLD, 0, acc);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      st16<true>(a.xpart, (((win * NH + h) * NP + row) * C + nt * QN + j * 16 + g * 4) * 4, __builtin_bit_cast(u4, acc[j]));
+  }
+  quad_handover(a.xflags, a.ctl, win, h, fv + 1);
+  // out[:, 32h .. 32h+32) = x1 + b2 + P_0 + P_1 + P_2 + P_3, scattered back to the token rows
+  for (int idx = tid; idx < N * (HD / 4); idx += 256) {
+    const int r = idx / (HD / 4), col = h * HD + (idx % (HD / 4)) * 4;
+    const h4 sh = *reinterpret_cast<const h4 *>(x1s + r * ZLD + col);
+    f4 v = add_bias4(f4{(float)sh[0], (float)sh[1], (float)sh[2], (float)sh[3]}, par + P_BFC2, col);
+#pragma unroll
+    for (int hh = 0; hh < NH; ++hh) v += __builtin_bit_cast(f4, ld16<true>(a.xpart, (((win * NH + hh) * NP + r) * C + col) * 4));
+    st8<true>(xout, (tok[r] * C + col) * 2, pack_h4(v));
+  }
+}
+
+__global__ void __launch_bounds__(256) k_block_pair_quad(Args a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  GridBarrier bar;
+  grid_barrier_begin(bar, a.ctl);
+  const unsigned fv = bar.epoch * 8u + 1u;      // grows from launch to launch (at least one barrier per launch)
+  WeightRing ring{lds + OFF_RING, lds_address(lds + OFF_RING), 0, 0};
+  const int nwin = (a.Hh / WS) * (a.Ww / WS), quads = gridDim.x / NH;
+  const int quad = blockIdx.x / NH, h = blockIdx.x % NH;
+  for (int win = quad; win < nwin; win += quads)
+    block_for_window_quad(lds, ring, a, a.w[0], win + quads < nwin ? &a.w[0] : &a.w[1], 0, a.x, a.mid, win, h, fv);
+  grid_sync(bar);
+  for (int win = quad; win < nwin; win += quads)
+    block_for_window_quad(lds, ring, a, a.w[1], win + quads < nwin ? &a.w[1] : nullptr, a.shift, a.mid, a.y, win, h, fv + 2);
+  grid_barrier_end(bar);
+}
+
 // ---- fused two-GEMM FFN: Y1 = X.W1 ; Y2 = Y1.W2 (split-K partials + reduce) ----
 struct FfnArgs {
   int M, K, F, splitk;
@@ -461,9 +756,18 @@ static int validate(const souffle_swin_cfg *c) {
   if (!(c->ln_eps >= 0.f)) return fail(SOUFFLE_ERR_SHAPE, "ln_eps must be >= 0");
   return SOUFFLE_OK;
 }
-static size_t pair_ws_bytes(const souffle_swin_cfg *c) {
-  return round_up(kCtlWords * 4, 256) + round_up((size_t)c->height * c->width * C * 2, 256);
+struct PairWs { size_t mid, xctx, xpart, xflags, total; };
+static PairWs pair_ws(const souffle_swin_cfg *c) {
+  const size_t nwin = (size_t)(c->height / WS) * (c->width / WS);
+  PairWs p;
+  p.mid = round_up(kCtlWords * 4, 256);
+  p.xctx = p.mid + round_up((size_t)c->height * c->width * C * 2, 256);
+  p.xpart = p.xctx + round_up(nwin * NP * C * 2, 256);
+  p.xflags = p.xpart + round_up(nwin * NH * NP * C * 4, 256);
+  p.total = p.xflags + round_up(nwin * 16 * 4, 256);
+  return p;
 }
+static size_t pair_ws_bytes(const souffle_swin_cfg *c) { return pair_ws(c).total; }
 
 }  // namespace swin
 }  // namespace souffle
@@ -486,7 +790,11 @@ extern "C" int souffle_swin_block_pair_fused(const souffle_swin_cfg *cfg, const 
   a.Hh = cfg->height; a.Ww = cfg->width; a.shift = cfg->shift; a.use_mask = cfg->use_shift_mask && cfg->shift > 0; a.eps = cfg->ln_eps;
   a.x = static_cast<const half_t *>(x); a.y = static_cast<half_t *>(y);
   a.ctl = static_cast<unsigned *>(ws);
-  a.mid = reinterpret_cast<half_t *>(static_cast<char *>(ws) + round_up(kCtlWords * 4, 256));
+  const swin::PairWs pw = swin::pair_ws(cfg);
+  a.mid = reinterpret_cast<half_t *>(static_cast<char *>(ws) + pw.mid);
+  a.xctx = reinterpret_cast<half_t *>(static_cast<char *>(ws) + pw.xctx);
+  a.xpart = reinterpret_cast<float *>(static_cast<char *>(ws) + pw.xpart);
+  a.xflags = reinterpret_cast<unsigned *>(static_cast<char *>(ws) + pw.xflags);
   {
     int cap = 0;
     stage_trace(&a.trace, &cap, 256);
@@ -507,10 +815,15 @@ extern "C" int souffle_swin_block_pair_fused(const souffle_swin_cfg *cfg, const 
   static bool attr_done = false;
   if (!attr_done) {
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)swin::k_block_pair, hipFuncAttributeMaxDynamicSharedMemorySize, swin::LDS_BYTES));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)swin::k_block_pair_quad, hipFuncAttributeMaxDynamicSharedMemorySize, swin::LDS_BYTES));
     attr_done = true;
   }
   const int nwin = (cfg->height / swin::WS) * (cfg->width / swin::WS);
   void *args[] = {&a};
+  // four workgroups per window (unless switched off) while that gives a window at most two turns per quad
+  if (swin_split_mode() && df.num_cus >= 4 && (long long)nwin * swin::NH <= 2ll * df.num_cus)
+    return launch_persistent((const void *)swin::k_block_pair_quad, (df.num_cus / 4) * 4 < nwin * swin::NH ? (df.num_cus / 4) * 4 : nwin * swin::NH,
+                             256, args, swin::LDS_BYTES, static_cast<hipStream_t>(stream));
   return launch_persistent((const void *)swin::k_block_pair, df.num_cus, 256, args, swin::LDS_BYTES,
                            static_cast<hipStream_t>(stream));
 }

@@ -98,6 +98,7 @@ SIGNATURES = {
     "souffle_lstm_workspace_bytes": (C.c_size_t, [C.POINTER(LstmCfg)]),
     "souffle_lstm_fused": (C.c_int, [C.POINTER(LstmCfg), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                      C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "souffle_set_swin_split": (C.c_int, [C.c_int]),
     "souffle_swin_workspace_bytes": (C.c_size_t, [C.POINTER(SwinCfg)]),
     "souffle_swin_block_pair_fused": (C.c_int, [C.POINTER(SwinCfg), C.POINTER(SwinBlockW), C.c_void_p, C.c_void_p,
                                                 C.c_void_p, C.c_size_t, C.c_void_p]),
@@ -201,6 +202,11 @@ def set_bert_sync(mode):
     """Hand-over between the stages of the skinny fused encoder: "dataflow" (default) or "barrier"."""
     modes = {"dataflow": SYNC_DATAFLOW, "barrier": SYNC_BARRIER, SYNC_DATAFLOW: SYNC_DATAFLOW, SYNC_BARRIER: SYNC_BARRIER}
     check(lib().souffle_set_bert_sync(modes[mode]))
+
+
+def set_swin_split(on):
+    """Swin block pair: four workgroups per window (True, the default) or one (False)."""
+    check(lib().souffle_set_swin_split(1 if on else 0))
 
 
 def set_cooperative_launch(on):

@@ -25,6 +25,35 @@ def test_block_pair_matches_oracle(hw, with_bias, mask):
     assert_close("swin y", y, ref)
 
 
+@pytest.mark.parametrize("hw,with_bias", [(56, True), (28, False), (7, True)])
+def test_block_pair_split_and_unsplit_agree_and_repeat(hw, with_bias):
+    """Four workgroups per window (default) against one workgroup per window: same result up to the
+    order of FC2's fp32 additions, both within tolerance of the oracle, and every launch of a mode gives
+    the same bits (the hand-over words of the split kernel grow from launch to launch, nothing is reset)."""
+    announce("swin pair split/unsplit %dx%d bias=%s" % (hw, hw, with_bias))
+    import souffle_hip as sh
+    import swin_transformer_binding as sb
+    ws = [synth.swin_block_weights(3, b, with_bias=with_bias) for b in range(2)]
+    x = synth.swin_input(3, hw * hw)
+    ref = oracle.swin_block_pair(x, ws, hw, hw)
+    dx, d0, d1 = dev(x), dev_weights(ws[0]), dev_weights(ws[1])
+    try:
+        sh.set_swin_split(True)
+        a1 = sb.swin_block_pair(dx, d0, d1, hw, hw).clone()
+        a2 = sb.swin_block_pair(dx, d0, d1, hw, hw).clone()
+        sh.set_swin_split(False)
+        b1 = sb.swin_block_pair(dx, d0, d1, hw, hw).clone()
+        sh.set_swin_split(True)
+        a3 = sb.swin_block_pair(dx, d0, d1, hw, hw).clone()
+    finally:
+        sh.set_swin_split(True)
+    torch.cuda.synchronize()
+    assert torch.equal(a1, a2) and torch.equal(a1, a3)
+    assert_close("split", a1, ref)
+    assert_close("unsplit", b1, ref)
+    assert (a1.float() - b1.float()).abs().max().item() <= 2 ** -6
+
+
 def test_shift_zero_pair_and_identity_blocks():
     """With zero projection and FC2 weights both blocks are the identity whatever the window
     gather / scatter does: the permutation must be undone exactly (bit-exact on fp16 data)."""
