@@ -528,6 +528,9 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
     qchunk_mma(buf, A, lda, ka, acc);
   };
   const int row = wave * 16 + l16;
+  int mark_id = shift > 0 ? 16 : 0;
+  auto mark = [&]() { if (a.trace && tid == 0 && win == (int)blockIdx.x / NH) a.trace[blockIdx.x * 32 + mark_id] = wall_clock64(); ++mark_id; };
+  mark();
 
   __syncthreads();
   while (ring.issued < first_chunk + 2) top_up();
@@ -550,6 +553,7 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
     copy(P_G1, w.ln1_g, C, 1.f); copy(P_B1, w.ln1_b, C, 0.f); copy(P_G2, w.ln2_g, C, 1.f); copy(P_B2, w.ln2_b, C, 0.f);
   }
   __syncthreads();
+  mark();
 
   // LN1 of the gathered rows (kept in x1s as the shortcut of the projection)
   layernorm_rows([&](int r, int c) {
@@ -558,6 +562,7 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
     return v;
   }, zs, par + P_G1, par + P_B1, a.eps);
   __syncthreads();
+  mark();
 
   // Q_h (pre-scaled), K_h, V_h in big[:, 0..32), [32..64), [64..96)
   const float qscale = rsqrtf((float)HD);
@@ -573,6 +578,7 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
     }
   }
   __syncthreads();
+  mark();
 
   // attention of head h: wave = query tile
   {
@@ -628,12 +634,15 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
       st8<true>(a.xctx, ((win * NP + q) * C + h * HD + dt * 16 + g * 4) * 2, pk);
     }
   }
+  mark();
   quad_handover(a.xflags, a.ctl, win, h, fv);
+  mark();
   for (int idx = tid; idx < NP * (C / 8); idx += 256) {
     const int r = idx / (C / 8), c8 = idx % (C / 8);
     if (c8 / (HD / 8) != h) *reinterpret_cast<u4 *>(zs + r * ZLD + c8 * 8) = ld16<true>(a.xctx, ((win * NP + r) * C + c8 * 8) * 2);
   }
   __syncthreads();
+  mark();
 
   // x1 = x + ctx.Wproj + b (all columns, in every workgroup of the window)
   for (int nt = 0; nt < C / QN; ++nt) {
@@ -651,8 +660,10 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
     }
   }
   __syncthreads();
+  mark();
   layernorm_rows([&](int r, int c) { return *reinterpret_cast<const u4 *>(x1s + r * ZLD + c); }, zs, par + P_G2, par + P_B2, a.eps);
   __syncthreads();
+  mark();
 
   // H_h = gelu(Z2 . W1[:, quarter h] + b1) in big[:, 0..128)
   for (int nt = 0; nt < (F / NH) / QN; ++nt) {
@@ -668,6 +679,7 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
     }
   }
   __syncthreads();
+  mark();
 
   // P_h = H_h . W2[quarter h, :], fp32, through memory
   for (int nt = 0; nt < C / QN; ++nt) {
@@ -677,7 +689,9 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
     for (int j = 0; j < 2; ++j)
       st16<true>(a.xpart, (((win * NH + h) * NP + row) * C + nt * QN + j * 16 + g * 4) * 4, __builtin_bit_cast(u4, acc[j]));
   }
+  mark();
   quad_handover(a.xflags, a.ctl, win, h, fv + 1);
+  mark();
   // out[:, 32h .. 32h+32) = x1 + b2 + P_0 + P_1 + P_2 + P_3, scattered back to the token rows
   for (int idx = tid; idx < N * (HD / 4); idx += 256) {
     const int r = idx / (HD / 4), col = h * HD + (idx % (HD / 4)) * 4;
@@ -687,6 +701,7 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
     for (int hh = 0; hh < NH; ++hh) v += __builtin_bit_cast(f4, ld16<true>(a.xpart, (((win * NH + hh) * NP + r) * C + col) * 4));
     st8<true>(xout, (tok[r] * C + col) * 2, pack_h4(v));
   }
+  mark();
 }
 
 __global__ void __launch_bounds__(256) k_block_pair_quad(Args a) {
