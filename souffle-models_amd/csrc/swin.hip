@@ -427,8 +427,11 @@ __global__ void __launch_bounds__(256) k_block_pair(Args a) {
 //   -> [hand-over 2: partial sums through memory] -> workgroup h adds the four partials, the bias
 //      and the shortcut for output columns [32h, 32h+32) in a fixed order and stores them.
 // A hand-over is a write-through store of the data, one flag word per workgroup, and a bounded poll
-// of the three other flags.  Flag values grow from launch to launch (they are derived from the
-// grid barrier's launch-persistent count), so nothing is reset.
+// of the three other flags.  Flag values grow from launch to launch (a launch count kept next to
+// them), so nothing is reset.
+// The hand-over words sit right behind the control block, at the same place for every image size, so
+// that a workspace used for several sizes keeps one consistent set of them.
+constexpr int kMaxSplitWindows = 256;
 constexpr int QN = 32, QCHUNK_BYTES = CHUNK_K * QN * 2, QCHUNKS = 15, QLOADS = QCHUNK_BYTES / 1024 / 4;
 static_assert(F / NH == CHUNK_K && HD == QN, "a head's FC2 share is one chunk deep, its q/k/v slices one chunk wide");
 
@@ -708,15 +711,22 @@ __global__ void __launch_bounds__(256) k_block_pair_quad(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   GridBarrier bar;
   grid_barrier_begin(bar, a.ctl);
-  const unsigned fv = bar.epoch * 8u + 1u;      // grows from launch to launch (at least one barrier per launch)
   WeightRing ring{lds + OFF_RING, lds_address(lds + OFF_RING), 0, 0};
   const int nwin = (a.Hh / WS) * (a.Ww / WS), quads = gridDim.x / NH;
+  // The hand-over words grow from launch to launch: a launch uses four values above those of the one
+  // before.  The launch count lives next to the words (behind the last of them), so that clearing the workspace or
+  // only its control block cannot set one back without the other.  Everybody reads it here, before the
+  // grid barrier below; workgroup 0 advances it after that barrier.
+  const unsigned seq = __hip_atomic_load(a.xflags + kMaxSplitWindows * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned fv = seq * 4u + 1u;
   const int quad = blockIdx.x / NH, h = blockIdx.x % NH;
   for (int win = quad; win < nwin; win += quads)
     block_for_window_quad(lds, ring, a, a.w[0], win + quads < nwin ? &a.w[0] : &a.w[1], 0, a.x, a.mid, win, h, fv);
   grid_sync(bar);
   for (int win = quad; win < nwin; win += quads)
     block_for_window_quad(lds, ring, a, a.w[1], win + quads < nwin ? &a.w[1] : nullptr, a.shift, a.mid, a.y, win, h, fv + 2);
+  if (blockIdx.x == 0 && threadIdx.x == 0)
+    __hip_atomic_store(a.xflags + kMaxSplitWindows * 16, seq + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   grid_barrier_end(bar);
 }
 
@@ -775,11 +785,11 @@ struct PairWs { size_t mid, xctx, xpart, xflags, total; };
 static PairWs pair_ws(const souffle_swin_cfg *c) {
   const size_t nwin = (size_t)(c->height / WS) * (c->width / WS);
   PairWs p;
-  p.mid = round_up(kCtlWords * 4, 256);
+  p.xflags = round_up(kCtlWords * 4, 256);
+  p.mid = p.xflags + round_up((kMaxSplitWindows * 16 + 1) * 4, 256);      // hand-over words + the launch count
   p.xctx = p.mid + round_up((size_t)c->height * c->width * C * 2, 256);
   p.xpart = p.xctx + round_up(nwin * NP * C * 2, 256);
-  p.xflags = p.xpart + round_up(nwin * NH * NP * C * 4, 256);
-  p.total = p.xflags + round_up(nwin * 16 * 4, 256);
+  p.total = p.xpart + round_up(nwin * NH * NP * C * 4, 256);
   return p;
 }
 static size_t pair_ws_bytes(const souffle_swin_cfg *c) { return pair_ws(c).total; }
@@ -836,7 +846,7 @@ extern "C" int souffle_swin_block_pair_fused(const souffle_swin_cfg *cfg, const 
   const int nwin = (cfg->height / swin::WS) * (cfg->width / swin::WS);
   void *args[] = {&a};
   // four workgroups per window (unless switched off) while that gives a window at most two turns per quad
-  if (swin_split_mode() && df.num_cus >= 4 && (long long)nwin * swin::NH <= 2ll * df.num_cus)
+  if (swin_split_mode() && df.num_cus >= 4 && nwin <= swin::kMaxSplitWindows && (long long)nwin * swin::NH <= 2ll * df.num_cus)
     return launch_persistent((const void *)swin::k_block_pair_quad, (df.num_cus / 4) * 4 < nwin * swin::NH ? (df.num_cus / 4) * 4 : nwin * swin::NH,
                              256, args, swin::LDS_BYTES, static_cast<hipStream_t>(stream));
   return launch_persistent((const void *)swin::k_block_pair, df.num_cus, 256, args, swin::LDS_BYTES,

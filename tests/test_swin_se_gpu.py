@@ -54,6 +54,28 @@ def test_block_pair_split_and_unsplit_agree_and_repeat(hw, with_bias):
     assert (a1.float() - b1.float()).abs().max().item() <= 2 ** -6
 
 
+def test_block_pair_one_workspace_for_several_image_sizes():
+    """A caller may keep ONE workspace for several image sizes (sized for the largest): the hand-over
+    words of the split kernel must stay consistent when the sizes alternate."""
+    announce("swin pair shared workspace")
+    import ctypes as C
+    import souffle_hip as sh
+    ws_np = [synth.swin_block_weights(3, b) for b in range(2)]
+    dws = [dev_weights(w) for w in ws_np]
+    arr = (sh.SwinBlockW * 2)(*[sh.SwinBlockW(*[sh.ptr(w.get(k)) for k in sh.SWIN_W_FIELDS]) for w in dws])
+    cfgs = {hw: sh.SwinCfg(hw, hw, 128, 4, 7, 3, 4, 1, 1e-5) for hw in (56, 14, 28)}
+    ws = sh.Workspace(max(sh.lib().souffle_swin_workspace_bytes(C.byref(c)) for c in cfgs.values()))
+    for hw in (56, 14, 28, 14, 56, 28):
+        x = synth.swin_input(3, hw * hw)
+        dx = dev(x)
+        y = torch.empty_like(dx)
+        sh.check(sh.lib().souffle_swin_block_pair_fused(C.byref(cfgs[hw]), arr, dx.data_ptr(), y.data_ptr(), ws.ptr, ws.nbytes,
+                                                        sh.current_stream()))
+        torch.cuda.synchronize()
+        assert ws.status() == 0
+        assert_close("swin y %d" % hw, y, oracle.swin_block_pair(x, ws_np, hw, hw))
+
+
 def test_shift_zero_pair_and_identity_blocks():
     """With zero projection and FC2 weights both blocks are the identity whatever the window
     gather / scatter does: the permutation must be undone exactly (bit-exact on fp16 data)."""
