@@ -10,8 +10,9 @@
  *     pointers, 16-byte aligned, and the work is queued on the given HIP stream
  *     (souffle_stream_t is a hipStream_t; NULL = the default stream);
  *   - a workspace must be zeroed once with souffle_workspace_init() before its
- *     first use (it holds grid-barrier state); it may then be reused by any number
- *     of calls, one at a time.  Calls that share a workspace must not overlap;
+ *     first use (all of it: it holds grid-barrier state, step tags and hand-over
+ *     words); it may then be reused by any number of calls of any entry point and
+ *     configuration, one at a time.  Calls that share a workspace must not overlap;
  *   - weights are fp16 matrices stored [K][N] with N contiguous, Y = X.W
  *     (reference: cpp/bert/kernels/gemm_three_stages.h:95-131,
  *      cpp/bert/test_souffle_bert_layer.py:139-143); activations are fp16 row-major.
@@ -51,18 +52,19 @@ typedef struct {
   char arch[64];
 } souffle_devinfo;
 int souffle_device_info(souffle_devinfo *out);
-/* Queues one MFMA-only kernel (4 waves per CU, `iters` x 16 independent fp16 16x16x32 MFMAs per wave, no
- * memory traffic) and reports the flops it performs: timed by the caller, it gives the empirical
- * matrix-core ceiling that the published peak is compared with.  `out` takes 2 KiB per CU of results. */
 /* Queues a persistent kernel of `stages` dependent grid-wide stages without arithmetic on an initialised
  * workspace (souffle_workspace_init; 16 KiB are enough).  mode 0: the grid barrier alone; mode 1: 16 bytes
  * written through, the barrier, and a read of what a workgroup of another XCD wrote, per stage.  Timed by
  * the caller it gives the latency floor of a chain of dependent stages on this device, which bounds the
  * skinny shapes (B*S < 1024) rather than the HBM or MFMA roofline. */
 int souffle_stage_floor_probe(void *workspace, size_t workspace_bytes, int stages, int mode, souffle_stream_t stream);
+/* Queues one MFMA-only kernel (4 waves per CU, `iters` x 16 independent fp16 16x16x32 MFMAs per wave, no
+ * memory traffic) and reports the flops it performs: timed by the caller, it gives the empirical
+ * matrix-core ceiling that the published peak is compared with.  `out` takes 2 KiB per CU of results. */
 int souffle_mfma_probe(float *out, size_t out_bytes, int iters, double *flops, souffle_stream_t stream);
 
-/* Zero the control block at the head of a workspace (stream-ordered, no allocation).
+/* Zero a workspace, all workspace_bytes of it (stream-ordered fill kernel, no allocation, capturable).
+ * Once before the first use, and again after a launch that reported a failed wait.
  * The reference instead zero-allocates its scratch on every call
  * (cpp/bert/bert_binding.cu:32-78). */
 int souffle_workspace_init(void *workspace, size_t workspace_bytes, souffle_stream_t stream);

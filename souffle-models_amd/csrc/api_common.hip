@@ -117,6 +117,10 @@ __global__ void k_zero_words(unsigned *p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0u;
 }
+// 16 bytes per thread and step, any size (n16 = number of 16-byte units).
+__global__ void __launch_bounds__(256) k_zero_bytes(u4 *p, size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) p[i] = u4{0u, 0u, 0u, 0u};
+}
 
 // Plain Y = X.W (fp16 in/out, fp32 accumulate): one tile per workgroup.
 template <class Tile>
@@ -288,9 +292,13 @@ extern "C" int souffle_workspace_init(void *ws, size_t bytes, souffle_stream_t s
   if (!ws) return fail(SOUFFLE_ERR_WORKSPACE, "workspace is NULL");
   if (!aligned16(ws)) return fail(SOUFFLE_ERR_ALIGN, "workspace must be 16-byte aligned");
   if (bytes < (size_t)kCtlWords * 4) return fail(SOUFFLE_ERR_WORKSPACE, "workspace smaller than its %d-byte control block", kCtlWords * 4);
+  // The whole workspace, not only the control block: behind it live step tags (LSTM), hand-over words
+  // (Swin) and not-yet-written markers that must not start from whatever the memory held before.
   // A fill kernel rather than a memset node, so that callers may capture this call.
-  hipLaunchKernelGGL(k_zero_words, dim3((kCtlWords + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<unsigned *>(ws), kCtlWords);
+  const size_t n16 = bytes / 16;
+  const size_t want = (n16 + 255) / 256;
+  hipLaunchKernelGGL(k_zero_bytes, dim3((unsigned)(want < 4096 ? want : 4096)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<u4 *>(ws), n16);
   SOUFFLE_HIP_TRY(hipGetLastError());
   return SOUFFLE_OK;
 }

@@ -54,3 +54,35 @@ def test_all_ones_smoke_of_reference():
     y = run(np.ones((100, 256), np.float32), one, one).cpu().numpy()
     np.testing.assert_allclose(y[:, 0], np.tanh(np.arange(1, 101)), atol=1e-3)
     assert np.all(y == y[:, :1])
+
+
+def test_workspace_of_unknown_content_is_usable_after_init():
+    """A C caller's workspace comes from hipMalloc with whatever the memory held: souffle_workspace_init
+    zeroes all of it (step tags, hand-over words), after which any entry point may use it, one after the
+    other.  Here the workspace is filled with ones first, and serves the LSTM and the Swin block pair."""
+    announce("dirty workspace -> init -> lstm, swin")
+    import ctypes as C
+    import souffle_hip as sh
+    w_ih, w_hh, x = synth.lstm_tensors(5, layers=3, timesteps=9)
+    lcfg = sh.LstmCfg(3, 256, 9, 1, sh.GATES_IFGO, 0.0)
+    scfg = sh.SwinCfg(14, 14, 128, 4, 7, 3, 4, 1, 1e-5)
+    nbytes = max(sh.lib().souffle_lstm_workspace_bytes(C.byref(lcfg)), sh.lib().souffle_swin_workspace_bytes(C.byref(scfg)))
+    buf = torch.full(((nbytes + 15) // 16 * 4,), 0x3F800001, dtype=torch.int32, device="cuda:0")
+    sh.check(sh.lib().souffle_workspace_init(buf.data_ptr(), buf.numel() * 4, sh.current_stream()))
+    assert int(buf.abs().max().item()) == 0
+    dx, dwi, dwh = dev(x, torch.float32), dev(w_ih), dev(w_hh)
+    y = torch.empty((9, 256), dtype=torch.float32, device="cuda:0")
+    ws_np = [synth.swin_block_weights(3, b) for b in range(2)]
+    dws = [{k: dev(v) for k, v in w.items()} for w in ws_np]
+    arr = (sh.SwinBlockW * 2)(*[sh.SwinBlockW(*[sh.ptr(w.get(k)) for k in sh.SWIN_W_FIELDS]) for w in dws])
+    xs = synth.swin_input(3, 14 * 14)
+    dxs = dev(xs)
+    ys = torch.empty_like(dxs)
+    for _ in range(2):
+        sh.check(sh.lib().souffle_lstm_fused(C.byref(lcfg), dwi.data_ptr(), dwh.data_ptr(), None, dx.data_ptr(), y.data_ptr(),
+                                            buf.data_ptr(), buf.numel() * 4, sh.current_stream()))
+        sh.check(sh.lib().souffle_swin_block_pair_fused(C.byref(scfg), arr, dxs.data_ptr(), ys.data_ptr(), buf.data_ptr(),
+                                                        buf.numel() * 4, sh.current_stream()))
+        torch.cuda.synchronize()
+        assert_close("lstm y", y, oracle.lstm(x, w_ih, w_hh))
+        assert_close("swin y", ys, oracle.swin_block_pair(xs, ws_np, 14, 14))
