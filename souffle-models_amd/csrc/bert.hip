@@ -34,6 +34,12 @@ struct LayerW {
 // one stage of one layer and read only afterwards: readers can then use ordinary cached
 // loads (an XCD's L2 never holds an older version of a line) and each XCD fetches a line of
 // an activation once instead of every workgroup fetching it from memory.
+// The many-rows megakernel (82 MB of such buffers per layer at 4096 rows) rotates through
+// `layer_sets` sets instead, which stay in the memory-side cache, and restores the property at
+// the barrier that ends a layer: one wave of every workgroup invalidates its L1 and its XCD's L2
+// (an agent-scope acquire fence) after arriving and before it polls, so the invalidation has been
+// performed when the poll returns.  In the last stage of a layer nobody reads a buffer that a later
+// layer writes before reading, so no line dropped there can come back in an old version.
 struct Params {
   int B, S, M, act, num_layers, splitk_o, splitk_f;
   int big;             // rows are a multiple of 256 and many: the 256-row GEMM tiles are used
@@ -43,9 +49,11 @@ struct Params {
   half_t *qkv, *ctx, *z1, *y1, *h, *yl, *probs;
   float *part;
   unsigned *ctl;
+  unsigned *rbflags;   // many-rows megakernel: 16 hand-over words per 256-row block (see rowblock_ln)
   unsigned long long *trace;
   int trace_cap;
   size_t layer_stride;
+  int layer_sets;      // layer l uses buffer set l % layer_sets
   // dataflow kernel: bytes of one layer's buffers from `qkv` up to (not including) `yl`, and the
   // marker the control block holds while all buffers of this layout are in the unwritten state
   size_t flow_bytes;
@@ -57,7 +65,7 @@ struct Args : Params {
 
 __device__ __forceinline__ Params layer_params(const Params &a, int l) {
   Params p = a;
-  const size_t off = (size_t)l * a.layer_stride;
+  const size_t off = (size_t)(l % a.layer_sets) * a.layer_stride;
   auto adv = [&](half_t *q) { return reinterpret_cast<half_t *>(reinterpret_cast<char *>(q) + off); };
   p.qkv = adv(a.qkv); p.ctx = adv(a.ctx); p.z1 = adv(a.z1); p.y1 = adv(a.y1); p.h = adv(a.h); p.yl = adv(a.yl);
   p.part = reinterpret_cast<float *>(reinterpret_cast<char *>(a.part) + off);
@@ -395,13 +403,16 @@ __device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, 
     BigOut::run(lds, X, K, tm * 256, 0, K / 32, wptr, cvt, store16);
   }
 }
-// A pre-LayerNorm sum in two halves of K: z1 = X[:, :K/2].W[:K/2] + bias + resid and
-// z2 (in the otherwise unused partials area) = X[:, K/2:].W[K/2:], both fp16; big_ln adds them.
+// A pre-LayerNorm sum in two halves of K: X[:, :K/2].W[:K/2] + bias + resid and X[:, K/2:].W[K/2:],
+// both fp16, into the two halves of the (here otherwise unused) partials area (see fc2_sum_lo /
+// fc2_sum_hi; not into z1, which the out-projection of the same layer has written); big_ln adds them.
+__device__ __forceinline__ half_t *fc2_sum_lo(const Params &a) { return reinterpret_cast<half_t *>(a.part); }
+__device__ __forceinline__ half_t *fc2_sum_hi(const Params &a) { return reinterpret_cast<half_t *>(a.part) + (size_t)a.M * H; }
 template <bool COH>
 __device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a, const half_t *X, int K, const half_t *W,
                                             const half_t *bias, const half_t *resid, int first, int stride) {
   const int m_tiles = a.M / 256, n_tiles = H / BigFc2::kBN;
-  half_t *z2 = reinterpret_cast<half_t *>(a.part);
+  half_t *zlo = fc2_sum_lo(a), *zhi = fc2_sum_hi(a);
   for (int it = first; it < m_tiles * n_tiles * 2; it += stride) {
     int tm, tn2;
     big_tile(it, m_tiles, n_tiles * 2, &tm, &tn2);
@@ -415,30 +426,36 @@ __device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a,
       }
       return pack_h4(v);
     };
-    auto store16 = [&](int m, int nr, u4 v) { st16<COH>(ks == 0 ? a.z1 : z2, (m * H + n0 + nr) * 2, v); };
+    auto store16 = [&](int m, int nr, u4 v) { st16<COH>(ks == 0 ? zlo : zhi, (m * H + n0 + nr) * 2, v); };
     BigFc2::run(lds, X, K, tm * 256, k0, (K / 2) / 32, wptr, cvt, store16);
   }
 }
-// out[m] = LN(z1[m] (+ z2[m])) * g + b; one wave per row, two-pass statistics in fp32 registers
-template <bool COH>
-__device__ __forceinline__ void big_ln(const Params &a, const half_t *z2, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
+// out[m] = LN(z1[m] (+ z2[m])) * g + b; one wave per row, two-pass statistics in fp32 registers.
+// NR rows (m0, m0 + mstep, ...) per call: their loads are all issued before the first is used.
+template <bool COH, int NR>
+__device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z1, const half_t *z2, const half_t *gam, const half_t *bet, half_t *out, int m0, int mstep) {
   const int lane = opaque_thread_id() & 63;
-  for (int m = first_row; m < a.M; m += row_stride) {
-    u2 raw[3], raw2[3];
+  u2 raw[NR][3], raw2[NR][3];
+#pragma unroll
+  for (int r = 0; r < NR; ++r)
 #pragma unroll
     for (int c = 0; c < 3; ++c) {
-      raw[c] = ld8<false>(a.z1, (m * H + c * 256 + lane * 4) * 2);
-      if (z2) raw2[c] = ld8<false>(z2, (m * H + c * 256 + lane * 4) * 2);
+      const int m = m0 + r * mstep;
+      raw[r][c] = ld8<false>(z1, (m * H + c * 256 + lane * 4) * 2);
+      if (z2) raw2[r][c] = ld8<false>(z2, (m * H + c * 256 + lane * 4) * 2);
     }
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int m = m0 + r * mstep;
     f4 v[3];
     float sum = 0.f;
 #pragma unroll
     for (int c = 0; c < 3; ++c) {
-      const h4 r = as_h4(raw[c]);
-      v[c] = f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+      const h4 q = as_h4(raw[r][c]);
+      v[c] = f4{(float)q[0], (float)q[1], (float)q[2], (float)q[3]};
       if (z2) {
-        const h4 r2 = as_h4(raw2[c]);
-        v[c] += f4{(float)r2[0], (float)r2[1], (float)r2[2], (float)r2[3]};
+        const h4 q2 = as_h4(raw2[r][c]);
+        v[c] += f4{(float)q2[0], (float)q2[1], (float)q2[2], (float)q2[3]};
       }
       sum += v[c][0] + v[c][1] + v[c][2] + v[c][3];
     }
@@ -465,6 +482,51 @@ __device__ __forceinline__ void big_ln(const Params &a, const half_t *z2, const 
       }
       st8<COH>(out, (m * H + n) * 2, pack_h4(o));
     }
+  }
+}
+template <bool COH>
+__device__ __forceinline__ void big_ln(const Params &a, const half_t *z1, const half_t *z2, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
+  for (int m = first_row; m < a.M; m += row_stride) big_ln_rows<COH, 1>(a, z1, z2, gam, bet, out, m, 0);
+}
+
+// The LayerNorm that follows a pre-LayerNorm sum, without a grid barrier in between.  A 256-row
+// block of the sum is produced by 16 tiles (16 column tiles, or 8 column tiles x 2 halves of K).
+// A workgroup first finishes ALL its tiles of the stage, then publishes `tag` in the word of each
+// (row block, tile), then, per tile, waits for the 16 words of that row block and normalises 16
+// of its rows (tile t: rows 16t .. 16t+15, four per wave).  Nobody waits before all its own tiles
+// are published, so the waits end whatever the tile-to-workgroup mapping is; they are bounded all
+// the same.  The words are cleared by the launch itself before its first grid barrier and tags grow
+// within a launch.  Rows are normalised by the same routine as in the separate LayerNorm stage:
+// identical results.
+static_assert(H / BigOut::kBN == 16 && 2 * (H / BigFc2::kBN) == 16, "16 tiles per row block");
+template <bool COH>
+__device__ __forceinline__ void rowblock_ln(const Params &a, unsigned tag, const half_t *z1, const half_t *z2, const half_t *gam, const half_t *bet,
+                                            half_t *out, int first, int stride) {
+  const int m_tiles = a.M / 256, wave = threadIdx.x >> 6;
+  __builtin_amdgcn_s_waitcnt(0);                 // this wave's write-through stores are acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0)
+    for (int it = first; it < m_tiles * 16; it += stride) {
+      int tm, tn;
+      big_tile(it, m_tiles, 16, &tm, &tn);
+      __hip_atomic_store(a.rbflags + tm * 16 + tn, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  for (int it = first; it < m_tiles * 16; it += stride) {
+    int tm, tn;
+    big_tile(it, m_tiles, 16, &tm, &tn);
+    if (threadIdx.x < 64) {
+      for (int spin = 0; spin < kMaxBarrierSpin; ++spin) {
+        bool ok = true;
+        if (threadIdx.x < 16)
+          ok = (int)(__hip_atomic_load(a.rbflags + tm * 16 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - tag) >= 0;
+        if (__all(ok)) break;
+        __builtin_amdgcn_s_sleep(1);
+        if (spin == kMaxBarrierSpin - 1 && threadIdx.x == 0)   // gave up: the launch's output is invalid
+          (void)__hip_atomic_fetch_or(a.ctl + kCtlErrWord, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    __syncthreads();
+    big_ln_rows<COH, 4>(a, z1, z2, gam, bet, out, tm * 256 + tn * 16 + wave * 4, 1);
   }
 }
 
@@ -1082,6 +1144,9 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
   bool qkv_ready = false;
   // this kernel leaves data in the workspace buffers: the dataflow kernel must refill them
   if (first == 0 && threadIdx.x == 0) __hip_atomic_store(args.ctl + kCtlFlowWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if constexpr (BIG)   // the row-block hand-over words start every launch at 0 (two grid barriers before their first use)
+    for (int i = first * 256 + threadIdx.x; i < (args.M / 256) * 16; i += stride * 256)
+      __hip_atomic_store(args.rbflags + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   for (int l = 0; l < args.num_layers; ++l) {
     const LayerW w = args.layers[l];
     const Params a = layer_params(args, l);
@@ -1092,20 +1157,26 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       grid_sync(bar);
       stage_attn_t<true, NKT>(lds, a, first, stride);
       grid_sync(bar);
-      if constexpr (BIG) big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, xin, first, stride);
-      else stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
-      grid_sync(bar);
-      if constexpr (BIG) big_ln<true>(a, nullptr, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
-      else stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
+      if constexpr (BIG) {
+        big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, xin, first, stride);
+        rowblock_ln<true>(a, 2u * l + 1u, a.z1, nullptr, w.ln1_g, w.ln1_b, a.y1, first, stride);
+      } else {
+        stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
+        grid_sync(bar);
+        stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
+      }
       grid_sync(bar);
       if constexpr (BIG) big_fc1<true>(lds_raw, a, w, first, stride);
       else stage_fc1<true, Tile>(lds, a, w, first, stride);
       grid_sync(bar);
-      if constexpr (BIG) big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, a.y1, first, stride);
-      else stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
-      grid_sync(bar);
-      if constexpr (BIG) big_ln<true>(a, reinterpret_cast<const half_t *>(a.part), w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
-      else stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
+      if constexpr (BIG) {
+        big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, a.y1, first, stride);
+        rowblock_ln<true>(a, 2u * l + 2u, fc2_sum_lo(a), fc2_sum_hi(a), w.ln2_g, w.ln2_b, yout, first, stride);
+      } else {
+        stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
+        grid_sync(bar);
+        stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
+      }
     } else {
       // Weight slices are queued one stage ahead, from inside the grid barrier that precedes
       // the stage.
@@ -1131,7 +1202,9 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
     }
     qkv_ready = false;
     if (l + 1 < a.num_layers) {
-      if constexpr (LARGE) grid_sync(bar);
+      if constexpr (BIG)   // the next layers write this layer's buffers again: see Params
+        grid_sync(bar, [&]() { if (threadIdx.x < 64) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); });
+      else if constexpr (LARGE) grid_sync(bar);
       else grid_sync(bar, [&]() { qkv_ready = preissue_w<OsFull>(lds_raw, QkvItems{args.layers[l + 1].w_qkv, a.M}); });
     }
     xin = yout;
@@ -1302,8 +1375,8 @@ __global__ void __launch_bounds__(256) k_presum2_big(Args a, const half_t *X, in
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   big_presum2<false>(lds_raw, a, X, K, W, bias, resid, blockIdx.x, gridDim.x);
 }
-__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *z2, const half_t *gam, const half_t *bet, half_t *out) {
-  big_ln<false>(a, z2, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
+__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *z1, const half_t *z2, const half_t *gam, const half_t *bet, half_t *out) {
+  big_ln<false>(a, z1, z2, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
 }
 template <int MODE>
 __global__ void __launch_bounds__(256) k_fc1(Args a, int l) {
@@ -1353,12 +1426,15 @@ __global__ void __launch_bounds__(256) k_pad_mask(const half_t *mask, half_t *mp
 }
 
 // ------------------------------------------------------------------- host ----
+constexpr int kBigSets = 1;     // buffer sets the many-rows megakernel rotates through (1: 1604 us at 4096 rows, 2: 1777, 3: 1787, one per layer: 1808)
 struct Plan {
   bool large, big;
   int splitk_o, splitk_f;
   size_t off_ctl, off_qkv, off_ctx, off_z1, off_y1, off_h, off_yl, off_part, layer_stride, total;
+  int layer_sets;
   size_t flow_bytes;      // a layer's buffers without its output (which comes last)
   size_t off_xpad, off_ypad, off_maskpad;
+  size_t off_rbflags;     // 16 words per 256-row block (many-rows megakernel only)
   unsigned flow_marker;
 };
 
@@ -1401,7 +1477,16 @@ static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   p.off_yl = take(M * H * 2);
   p.layer_stride = off - first;                       // one set of inter-stage buffers per layer
   p.flow_bytes = p.off_yl - p.off_qkv;
-  p.total = first + p.layer_stride * (size_t)(num_layers < 1 ? 1 : num_layers);
+  const int nl = num_layers < 1 ? 1 : num_layers;
+  p.layer_sets = p.big && nl > kBigSets ? kBigSets : nl;
+  p.total = first + p.layer_stride * (size_t)p.layer_sets;
+  // (in front of the padding area: the plan of the padded configuration, which lacks that area, must agree)
+  p.off_rbflags = 0;
+  if (p.big) {
+    off = p.total;
+    p.off_rbflags = take(M / 256 * 64);
+    p.total = off;
+  }
   // a sequence length that is not built: padded copies of x and y and the padded additive mask
   p.off_xpad = p.off_ypad = p.off_maskpad = 0;
   if (padded_len(c->seq_len) != c->seq_len) {
@@ -1431,6 +1516,7 @@ static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_laye
   a.big = p.big ? 1 : 0;
   a.x = static_cast<const half_t *>(x); a.mask = static_cast<const half_t *>(mask); a.y = static_cast<half_t *>(y);
   a.ctl = reinterpret_cast<unsigned *>(base + p.off_ctl);
+  a.rbflags = p.big ? reinterpret_cast<unsigned *>(base + p.off_rbflags) : nullptr;
   a.qkv = reinterpret_cast<half_t *>(base + p.off_qkv);
   a.ctx = reinterpret_cast<half_t *>(base + p.off_ctx);
   a.z1 = reinterpret_cast<half_t *>(base + p.off_z1);
@@ -1438,6 +1524,7 @@ static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_laye
   a.h = reinterpret_cast<half_t *>(base + p.off_h);
   a.yl = reinterpret_cast<half_t *>(base + p.off_yl);
   a.layer_stride = p.layer_stride;
+  a.layer_sets = p.layer_sets;
   a.flow_bytes = p.flow_bytes;
   a.flow_marker = p.flow_marker;
   a.part = reinterpret_cast<float *>(base + p.off_part);
@@ -1612,7 +1699,7 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     else hipLaunchKernelGGL(k_attn_small, dim3(grid_for((a.B * NH + 7) / 8 * 8 * (a.S / 16))), dim3(256), attn_small_lds_bytes(a.S), st, a);
     if constexpr (MODE == 2) {
       hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * (H / BigOut::kBN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, w.b_o, xin);
-      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)nullptr, w.ln1_g, w.ln1_b, a.y1);
+      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.z1, (const half_t *)nullptr, w.ln1_g, w.ln1_b, a.y1);
     } else if constexpr (LARGE) {
       hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, 1);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, 1, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
@@ -1622,7 +1709,7 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     hipLaunchKernelGGL(k_fc1<MODE>, dim3(grid_for((a.M / BM_QKV) * (F / BN))), dim3(256), GEMM_LDS, st, a, l);
     if constexpr (MODE == 2) {
       hipLaunchKernelGGL(k_presum2_big, dim3(grid_for((a.M / 256) * (H / BigFc2::kBN) * 2)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, w.b_fc2, a.y1);
-      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, reinterpret_cast<const half_t *>(a.part), w.ln2_g, w.ln2_b, yout);
+      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.part, (const half_t *)a.part + (size_t)a.M * H, w.ln2_g, w.ln2_b, yout);
     } else {
       hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_FC2) * (H / BN) * a.splitk_f)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, a.splitk_f);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout);

@@ -102,6 +102,29 @@ def test_encoder_matches_oracle(B, S, layers):
     assert torch.equal(y_f, y_u)
 
 
+@pytest.mark.parametrize("B,S,layers", [(32, 128, 5), (16, 128, 4), (64, 128, 3)])
+def test_many_rows_encoder_reuses_its_buffers(B, S, layers):
+    """At many rows all layers of the fused launch share one set of inter-stage buffers (kept coherent
+    by a cache invalidation at the barrier that ends a layer) and the LayerNorms are handed over per
+    256-row block: results equal the per-op chain bit for bit over several layers, on repeated launches
+    and with a different input in between (a line that survived from an earlier layer or launch would
+    show), and no bounded wait gives up."""
+    announce("bert encoder many rows, shared buffers B=%d S=%d L=%d" % (B, S, layers))
+    import bert_binding
+    ws = [synth.bert_layer_weights(2, l) for l in range(layers)]
+    x0, x1 = synth.bert_input(2, B, S), synth.bert_input(3, B, S)
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    y_u0 = enc(dev(x0), fused=False).clone()
+    y_u1 = enc(dev(x1), fused=False).clone()
+    y_a = enc(dev(x0)).clone()
+    y_b = enc(dev(x1)).clone()
+    y_c = enc(dev(x0)).clone()
+    torch.cuda.synchronize()
+    assert enc.ws.status() == 0
+    assert torch.equal(y_a, y_u0) and torch.equal(y_c, y_u0) and torch.equal(y_b, y_u1)
+    assert_close("encoder many rows", y_a, oracle.bert_encoder(x0, ws, B, S))
+
+
 @pytest.mark.parametrize("B,S,layers", [(1, 128, 12), (1, 384, 2), (2, 64, 3), (1, 128, 1)])
 def test_dataflow_sync_equals_barrier_sync(B, S, layers):
     """The dataflow hand-over (consumers poll the data) runs the same arithmetic as the grid-barrier
