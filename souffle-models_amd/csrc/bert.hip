@@ -153,9 +153,15 @@ __device__ __forceinline__ void poll_x(unsigned char *lds_x, const half_t *X, in
 }
 
 // ------------------------------------------------------------------ stages ----
+// Stands in for a bias the caller did not give, where a test per result would cost more than adding zeros.
+__device__ const half_t g_zero_row[F] = {};
+__device__ __forceinline__ f4 add_row4(f4 v, const half_t *row, int n) {
+  const h4 bb = ldg<h4>(row + n);
+  return v + f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+}
 __device__ __forceinline__ f4 add_bias4(f4 v, const half_t *bias, int n) {
   if (bias) {
-    const h4 bb = *reinterpret_cast<const h4 *>(bias + n);
+    const h4 bb = ldg<h4>(bias + n);
     v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
   }
   return v;
@@ -163,7 +169,7 @@ __device__ __forceinline__ f4 add_bias4(f4 v, const half_t *bias, int n) {
 
 __device__ __forceinline__ void add_bias8(f4 &lo, f4 &hi, const half_t *bias, int n) {
   if (bias) {
-    const h8 bb = *reinterpret_cast<const h8 *>(bias + n);
+    const h8 bb = ldg<h8>(bias + n);
     lo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
     hi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]};
   }
@@ -184,7 +190,7 @@ __device__ __forceinline__ void stage_qkv(half_t *lds, const Params &a, const La
     auto aload = [&](int m, int k) { return ld16<false>(xin, (m * H + k) * 2); };
     auto epi = [&](int m, int n, f4 v) {
       if (w.b_qkv) {
-        const h4 bb = *reinterpret_cast<const h4 *>(w.b_qkv + j * H + n);
+        const h4 bb = ldg<h4>(w.b_qkv + j * H + n);
         v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
       }
       const int b = m / a.S, s = m % a.S, hh = n / HD, d = n % HD;
@@ -204,7 +210,7 @@ __device__ __forceinline__ void stage_fc1(half_t *lds, const Params &a, const La
     auto aload = [&](int m, int k) { return ld16<false>(a.y1, (m * H + k) * 2); };
     auto epi = [&](int m, int n, f4 v) {
       if (w.b_fc1) {
-        const h4 bb = *reinterpret_cast<const h4 *>(w.b_fc1 + n);
+        const h4 bb = ldg<h4>(w.b_fc1 + n);
         v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
       }
 #pragma unroll
@@ -280,7 +286,7 @@ __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, 
       const h4 r = as_h4(rres[c]);
       s += f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
       if (bias) {
-        const h4 bb = *reinterpret_cast<const h4 *>(bias + n);
+        const h4 bb = ldg<h4>(bias + n);
         s += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
       }
       v[c] = s;
@@ -302,11 +308,11 @@ __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, 
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[i] = (v[c][i] - mean) * rstd;
       if (gam) {
-        const h4 gg = *reinterpret_cast<const h4 *>(gam + n);
+        const h4 gg = ldg<h4>(gam + n);
         o *= f4{(float)gg[0], (float)gg[1], (float)gg[2], (float)gg[3]};
       }
       if (bet) {
-        const h4 bb = *reinterpret_cast<const h4 *>(bet + n);
+        const h4 bb = ldg<h4>(bet + n);
         o += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
       }
       st8<COH>(out, (m * H + n) * 2, pack_h4(o));
@@ -341,7 +347,7 @@ __device__ __forceinline__ void big_tile(int it, int m_tiles, int n_tiles, int *
 }
 
 template <bool COH>
-__device__ __forceinline__ void big_qkv(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, int first, int stride) {
+__device__ __forceinline__ void big_qkv(unsigned char *lds, const Params &a, const LayerW &w, const half_t *xin, int first, int stride, const GridBarrier *tb = nullptr) {
   const int m_tiles = a.M / 256, n_tiles = 3 * H / BigQkv::kBN;
   for (int it = first; it < m_tiles * n_tiles; it += stride) {
     int tm, tn;
@@ -352,34 +358,46 @@ __device__ __forceinline__ void big_qkv(unsigned char *lds, const Params &a, con
       const int c = n0 + col, j = c / H;
       return w.w_qkv + ((size_t)j * H + k) * H + (c - j * H);
     };
+    const half_t *bq = w.b_qkv ? w.b_qkv : g_zero_row;
+    const int bq_stride = w.b_qkv ? H : 0;
     auto cvt = [&](int, int nr, f4 v) {
       const int c = n0 + nr, j = c / H, n = c - j * H;
-      return pack_h4(add_bias4(v, w.b_qkv ? w.b_qkv + j * H : nullptr, n));
+      return pack_h4(add_row4(v, bq + j * bq_stride, n));
     };
     auto store16 = [&](int m, int nr, u4 v) {                // 8 columns never straddle a head (64 columns)
       const int c = n0 + nr, j = c / H, n = c - j * H;
       const int b = m / a.S, s = m % a.S, hh = n / HD, d = n % HD;
       st16<COH>(a.qkv, ((((j * a.B + b) * NH + hh) * a.S + s) * HD + d) * 2, v);
     };
-    BigQkv::run(lds, xin, H, tm * 256, 0, H / 32, wptr, cvt, store16);
+    BigQkv::run(lds, xin, H, tm * 256, 0, H / 32, wptr, cvt, store16, tb);
   }
 }
 template <bool COH>
-__device__ __forceinline__ void big_fc1(unsigned char *lds, const Params &a, const LayerW &w, int first, int stride) {
+__device__ __forceinline__ void big_fc1(unsigned char *lds, const Params &a, const LayerW &w, int first, int stride, const GridBarrier *tb = nullptr) {
   const int m_tiles = a.M / 256, n_tiles = F / BigFc1::kBN;
   for (int it = first; it < m_tiles * n_tiles; it += stride) {
     int tm, tn;
     big_tile(it, m_tiles, n_tiles, &tm, &tn);
     const int n0 = tn * BigFc1::kBN;
     auto wptr = [&](int k, int col) { return w.w_fc1 + (size_t)k * F + n0 + col; };
-    auto cvt = [&](int, int nr, f4 v) {
-      v = add_bias4(v, w.b_fc1, n0 + nr);
+    const half_t *b1 = w.b_fc1 ? w.b_fc1 : g_zero_row;
+    auto cvt_relu = [&](int, int nr, f4 v) {
+      v = add_row4(v, b1, n0 + nr);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(v[i], 0.f) : gelu_tanh(v[i]);
+      for (int i = 0; i < 4; ++i) v[i] = fmaxf(v[i], 0.f);
+      return pack_h4(v);
+    };
+    auto cvt_gelu = [&](int, int nr, f4 v) {
+      v = add_row4(v, b1, n0 + nr);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = gelu_tanh(v[i]);
       return pack_h4(v);
     };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.h, (m * F + n0 + nr) * 2, v); };
-    BigFc1::run(lds, a.y1, H, tm * 256, 0, H / 32, wptr, cvt, store16);
+    f4 acc[4][BigFc1::NT];
+    BigFc1::mainloop(lds, a.y1, H, tm * 256, 0, H / 32, wptr, acc, tb);
+    if (a.act == SOUFFLE_ACT_RELU) BigFc1::epilogue(lds, tm * 256, acc, cvt_relu, store16, tb);
+    else BigFc1::epilogue(lds, tm * 256, acc, cvt_gelu, store16, tb);
   }
 }
 // z = X[M][K].W[K][768] + bias + resid, fp16, into a.z1 (the pre-LayerNorm sum of the out-projection
@@ -393,10 +411,11 @@ __device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, 
     big_tile(it, m_tiles, n_tiles, &tm, &tn);
     const int n0 = tn * BigOut::kBN;
     auto wptr = [&](int k, int col) { return W + (size_t)k * H + n0 + col; };
+    const half_t *bz = bias ? bias : g_zero_row;
     auto cvt = [&](int m, int nr, f4 v) {
       const int n = n0 + nr;
       const h4 r = as_h4(ld8<false>(resid, (m * H + n) * 2));
-      v = add_bias4(v, bias, n) + f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+      v = add_row4(v, bz, n) + f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
       return pack_h4(v);
     };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.z1, (m * H + n0 + nr) * 2, v); };
@@ -418,16 +437,20 @@ __device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a,
     big_tile(it, m_tiles, n_tiles * 2, &tm, &tn2);
     const int ks = tn2 & 1, n0 = (tn2 >> 1) * BigFc2::kBN, k0 = ks * (K / 2);
     auto wptr = [&](int k, int col) { return W + (size_t)k * H + n0 + col; };
-    auto cvt = [&](int m, int nr, f4 v) {
-      if (ks == 0) {
-        const int n = n0 + nr;
-        const h4 r = as_h4(ld8<false>(resid, (m * H + n) * 2));
-        v = add_bias4(v, bias, n) + f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
-      }
+    const half_t *bz = bias ? bias : g_zero_row;
+    auto cvt_lo = [&](int m, int nr, f4 v) {
+      const int n = n0 + nr;
+      const h4 r = as_h4(ld8<false>(resid, (m * H + n) * 2));
+      v = add_row4(v, bz, n) + f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
       return pack_h4(v);
     };
-    auto store16 = [&](int m, int nr, u4 v) { st16<COH>(ks == 0 ? zlo : zhi, (m * H + n0 + nr) * 2, v); };
-    BigFc2::run(lds, X, K, tm * 256, k0, (K / 2) / 32, wptr, cvt, store16);
+    auto cvt_hi = [&](int, int, f4 v) { return pack_h4(v); };
+    auto store_lo = [&](int m, int nr, u4 v) { st16<COH>(zlo, (m * H + n0 + nr) * 2, v); };
+    auto store_hi = [&](int m, int nr, u4 v) { st16<COH>(zhi, (m * H + n0 + nr) * 2, v); };
+    f4 acc[4][BigFc2::NT];
+    BigFc2::mainloop(lds, X, K, tm * 256, k0, (K / 2) / 32, wptr, acc);
+    if (ks == 0) BigFc2::epilogue(lds, tm * 256, acc, cvt_lo, store_lo);
+    else BigFc2::epilogue(lds, tm * 256, acc, cvt_hi, store_hi);
   }
 }
 // out[m] = LN(z1[m] (+ z2[m])) * g + b; one wave per row, two-pass statistics in fp32 registers.
@@ -473,11 +496,11 @@ __device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z1, c
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[i] = (v[c][i] - mean) * rstd;
       if (gam) {
-        const h4 gg = *reinterpret_cast<const h4 *>(gam + n);
+        const h4 gg = ldg<h4>(gam + n);
         o *= f4{(float)gg[0], (float)gg[1], (float)gg[2], (float)gg[3]};
       }
       if (bet) {
-        const h4 bb = *reinterpret_cast<const h4 *>(bet + n);
+        const h4 bb = ldg<h4>(bet + n);
         o += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
       }
       st8<COH>(out, (m * H + n) * 2, pack_h4(o));
@@ -501,10 +524,12 @@ __device__ __forceinline__ void big_ln(const Params &a, const half_t *z1, const 
 static_assert(H / BigOut::kBN == 16 && 2 * (H / BigFc2::kBN) == 16, "16 tiles per row block");
 template <bool COH>
 __device__ __forceinline__ void rowblock_ln(const Params &a, unsigned tag, const half_t *z1, const half_t *z2, const half_t *gam, const half_t *bet,
-                                            half_t *out, int first, int stride) {
+                                            half_t *out, int first, int stride, const GridBarrier *tb = nullptr) {
   const int m_tiles = a.M / 256, wave = threadIdx.x >> 6;
+  STAGE_MARK(tb, 0);
   __builtin_amdgcn_s_waitcnt(0);                 // this wave's write-through stores are acknowledged
   __syncthreads();
+  STAGE_MARK(tb, 1);
   if (threadIdx.x == 0)
     for (int it = first; it < m_tiles * 16; it += stride) {
       int tm, tn;
@@ -526,7 +551,9 @@ __device__ __forceinline__ void rowblock_ln(const Params &a, unsigned tag, const
       }
     }
     __syncthreads();
+    STAGE_MARK(tb, 2);
     big_ln_rows<COH, 4>(a, z1, z2, gam, bet, out, tm * 256 + tn * 16 + wave * 4, 1);
+    STAGE_MARK(tb, 3);
   }
 }
 
@@ -620,11 +647,6 @@ __device__ __forceinline__ bool preissue_w(unsigned char *lds, const Items &item
 }
 
 // Fine-grained time stamps inside a stage (development builds only: they cost scalar registers).
-#ifdef SOUFFLE_STAGE_MARKS
-#define STAGE_MARK(tb, id) do { if (tb) trace_mark(*(tb), (id)); } while (0)
-#else
-#define STAGE_MARK(tb, id) do { (void)(tb); } while (0)
-#endif
 
 // Driver of a skinny GEMM stage.  `w_ready`: the weight slice of this workgroup's first item
 // was queued earlier (inside the preceding grid barrier, or after the previous stage in the
@@ -716,7 +738,7 @@ __device__ __forceinline__ void ln_rows_in_lds(unsigned char *lds_x, bool has_ga
     h8 o;
     if (gam || bet) {
       h8 g8, b8;
-      if (gam) g8 = *reinterpret_cast<const h8 *>(gam + k);
+      if (gam) g8 = *reinterpret_cast<const h8 *>(gam + k);     // (LDS copies of the parameters)
       if (bet) b8 = *reinterpret_cast<const h8 *>(bet + k);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -866,7 +888,7 @@ __device__ __forceinline__ void attn_item(half_t *lds_h, const Params &a, int it
   for (int t = 0; t < NKT; ++t) {
     f4 sv = sc[t] * a.scale;
     if (a.mask) {
-      const h4 mk = *reinterpret_cast<const h4 *>(a.mask + ((size_t)b * S + q) * S + t * 16 + g * 4);
+      const h4 mk = ldg<h4>(a.mask + ((size_t)b * S + q) * S + t * 16 + g * 4);
       sv += f4{(float)mk[0], (float)mk[1], (float)mk[2], (float)mk[3]};
     }
     sc[t] = sv;
@@ -992,7 +1014,7 @@ __device__ __forceinline__ void attn_item_split(unsigned char *lds, const Params
     f4 sv = mfma_16x16x32(k1, qop[1], mfma_16x16x32(k0, qop[0], f4{0.f, 0.f, 0.f, 0.f})) * a.scale;
     // sv[v] = score(key = 16t + 4g + v, query = q)
     if (a.mask) {
-      const h4 mk = *reinterpret_cast<const h4 *>(a.mask + ((size_t)b * S + q) * S + t * 16 + g * 4);
+      const h4 mk = ldg<h4>(a.mask + ((size_t)b * S + q) * S + t * 16 + g * 4);
       sv += f4{(float)mk[0], (float)mk[1], (float)mk[2], (float)mk[3]};
     }
     sc[tt] = sv;
@@ -1152,26 +1174,26 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
     const Params a = layer_params(args, l);
     half_t *yout = (l == a.num_layers - 1) ? a.y : a.yl;
     if constexpr (LARGE) {
-      if constexpr (BIG) big_qkv<true>(lds_raw, a, w, xin, first, stride);
+      if constexpr (BIG) big_qkv<true>(lds_raw, a, w, xin, first, stride, &bar);
       else stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
       grid_sync(bar);
       stage_attn_t<true, NKT>(lds, a, first, stride);
       grid_sync(bar);
       if constexpr (BIG) {
         big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, xin, first, stride);
-        rowblock_ln<true>(a, 2u * l + 1u, a.z1, nullptr, w.ln1_g, w.ln1_b, a.y1, first, stride);
+        rowblock_ln<true>(a, 2u * l + 1u, a.z1, nullptr, w.ln1_g, w.ln1_b, a.y1, first, stride, &bar);
       } else {
         stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
         grid_sync(bar);
         stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
       }
       grid_sync(bar);
-      if constexpr (BIG) big_fc1<true>(lds_raw, a, w, first, stride);
+      if constexpr (BIG) big_fc1<true>(lds_raw, a, w, first, stride, &bar);
       else stage_fc1<true, Tile>(lds, a, w, first, stride);
       grid_sync(bar);
       if constexpr (BIG) {
         big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, a.y1, first, stride);
-        rowblock_ln<true>(a, 2u * l + 2u, fc2_sum_lo(a), fc2_sum_hi(a), w.ln2_g, w.ln2_b, yout, first, stride);
+        rowblock_ln<true>(a, 2u * l + 2u, fc2_sum_lo(a), fc2_sum_hi(a), w.ln2_g, w.ln2_b, yout, first, stride, &bar);
       } else {
         stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
         grid_sync(bar);

@@ -107,15 +107,23 @@ __device__ __forceinline__ auto make_rsrc(const void *base) {
 }
 constexpr int kAuxSc1 = 16;
 
+// A load the compiler knows to come from global memory.  Where it cannot infer the address space of
+// a pointer it emits a flat load, which may alias LDS: such a load is not moved across the LDS
+// accesses around it and each is waited for before the next LDS store (an epilogue that reads a
+// bias or a residual per result group then pays one memory latency per group).
+template <class T>
+__device__ __forceinline__ T ldg(const void *p) {
+  return *(const __attribute__((address_space(1))) T *)p;
+}
 template <bool COH>
 __device__ __forceinline__ u4 ld16(const void *base, int byte_off) {
   if constexpr (COH) return __builtin_amdgcn_raw_buffer_load_b128(make_rsrc(base), byte_off, 0, kAuxSc1);
-  else return *reinterpret_cast<const u4 *>(reinterpret_cast<const char *>(base) + byte_off);
+  else return ldg<u4>(reinterpret_cast<const char *>(base) + byte_off);
 }
 template <bool COH>
 __device__ __forceinline__ u2 ld8(const void *base, int byte_off) {
   if constexpr (COH) return __builtin_amdgcn_raw_buffer_load_b64(make_rsrc(base), byte_off, 0, kAuxSc1);
-  else return *reinterpret_cast<const u2 *>(reinterpret_cast<const char *>(base) + byte_off);
+  else return ldg<u2>(reinterpret_cast<const char *>(base) + byte_off);
 }
 // 8-byte relaxed agent-scope atomics: a (value, tag) pair that is published and polled
 // as one unit.  Being atomic operations, polling loads are re-issued on every spin.
@@ -131,7 +139,7 @@ __device__ __forceinline__ void st8_atomic(void *p, u2 v) {
 template <bool COH>
 __device__ __forceinline__ unsigned ld4(const void *base, int byte_off) {
   if constexpr (COH) return __builtin_amdgcn_raw_buffer_load_b32(make_rsrc(base), byte_off, 0, kAuxSc1);
-  else return *reinterpret_cast<const unsigned *>(reinterpret_cast<const char *>(base) + byte_off);
+  else return ldg<unsigned>(reinterpret_cast<const char *>(base) + byte_off);
 }
 template <bool COH>
 __device__ __forceinline__ void st16(void *base, int byte_off, u4 v) {
@@ -174,10 +182,14 @@ __device__ __forceinline__ float wave_max(float v) {
 // ---------------------------------------------------------- activations ----
 // 0.5 x (1 + tanh(0.79788456 (x + 0.044715 x^3)))  (cpp/bert/bert_base_impl.cu:722-734)
 __device__ __forceinline__ float gelu_tanh(float x) {
-  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  // 0.5 (1 + tanh(u)) = 1 - 1 / (exp(2u) + 1); exp overflow gives the correct limit 1.  The
-  // hardware reciprocal (1 ulp) replaces the IEEE division, which costs some 10 instructions.
-  return x * (1.0f - __builtin_amdgcn_rcpf(__expf(2.0f * u) + 1.0f));
+  // 0.5 (1 + tanh(u)) = 1 - 1 / (exp(2u) + 1) with u = 0.79788456 (x + 0.044715 x^3), and
+  // exp(2u) = exp2(x (K1 + K2 x^2)): five full-rate operations and two quarter-rate ones (the bare
+  // v_exp_f32 and v_rcp_f32, 1 ulp each; the library exp and an IEEE division cost some 20 more
+  // instructions, which at 192 results per lane made the FC1 epilogue at 4096 rows 12.8 us long).
+  // exp2 overflow gives the limit x, underflow the limit 0.
+  constexpr float K1 = 2.0f * 0.7978845608028654f * 1.4426950408889634f, K2 = K1 * 0.044715f;
+  const float e = __builtin_amdgcn_exp2f(x * __builtin_fmaf(x * x, K2, K1));
+  return x - x * __builtin_amdgcn_rcpf(e + 1.0f);
 }
 
 // -------------------------------------------------------- grid barrier ----
@@ -227,6 +239,13 @@ __device__ __forceinline__ void trace_mark(const GridBarrier &b, int id) {
   if (b.trace && b.trace_idx < b.trace_cap && threadIdx.x == 0)
     b.trace[(size_t)(2 * b.trace_cap + 8 * b.trace_idx + id) * b.nblk + blockIdx.x] = wall_clock64();
 }
+
+// Development marks inside a stage (compiled in only with SOUFFLE_STAGE_MARKS).
+#ifdef SOUFFLE_STAGE_MARKS
+#define STAGE_MARK(tb, id) do { if (tb) trace_mark(*(tb), (id)); } while (0)
+#else
+#define STAGE_MARK(tb, id) do { (void)(tb); } while (0)
+#endif
 
 __device__ __forceinline__ void grid_barrier_begin(GridBarrier &b, unsigned *ctl) {
   b.ctl = ctl;

@@ -107,9 +107,21 @@ struct GemmBig {
   // issued just before it cover.  (Issued as one burst after the barrier, the loads of the four
   // waves queue up behind each other and every SIMD idles: measured 2x the time per step.)
   template <class WPtr, class Cvt, class Store16>
-  __device__ static __forceinline__ void run(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, int nkt, WPtr wptr, Cvt cvt, Store16 store16) {
-    const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+  __device__ static __forceinline__ void run(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, int nkt, WPtr wptr, Cvt cvt, Store16 store16,
+                                             const GridBarrier *tb = nullptr) {
     f4 acc[4][NT];
+    mainloop(lds, X, ldx, m0, k0, nkt, wptr, acc, tb);
+    epilogue(lds, m0, acc, cvt, store16, tb);
+  }
+
+  // The two halves of run(), for callers whose epilogue depends on a run-time choice (an activation,
+  // which half of K): they branch once between two epilogue() calls.  A uniform condition tested inside
+  // cvt is not hoisted by the compiler but tested per result, and the tiny basic blocks in between
+  // serialise every dependent chain (FC1 with GELU: 12.8 us per tile instead of 5).
+  template <class WPtr>
+  __device__ static __forceinline__ void mainloop(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, int nkt, WPtr wptr, f4 (&acc)[4][NT],
+                                                  const GridBarrier *tb = nullptr) {
+    const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -117,6 +129,7 @@ struct GemmBig {
 #pragma unroll
     for (int i = 0; i < 4; ++i) mfma_pin(acc[i], true);
 
+    STAGE_MARK(tb, 0);
     __syncthreads();                                        // the previous user of the ring is done
     const unsigned ring = lds_address(lds);
 #pragma unroll
@@ -142,6 +155,7 @@ struct GemmBig {
     wait_ahead<NSTAGE - 2>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+    STAGE_MARK(tb, 1);
 #pragma unroll
     for (int i = 0; i < 4; ++i) x[i] = as_h8(lds_load16(lds + xoff[i]));
 #pragma unroll
@@ -200,25 +214,41 @@ struct GemmBig {
     if constexpr (NSTAGE >= 6) step(main_end + 4, F{}, F{}, std::integral_constant<int, 0>{});
 #pragma unroll
     for (int i = 0; i < 4; ++i) mfma_pin(acc[i], false);
+    STAGE_MARK(tb, 2);
+  }
 
+  template <class Cvt, class Store16>
+  __device__ static __forceinline__ void epilogue(unsigned char *lds, int m0, f4 (&acc)[4][NT], Cvt cvt, Store16 store16, const GridBarrier *tb = nullptr) {
+    const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
     // Epilogue.  A lane holds 4 consecutive columns of 16 rows per accumulator tile; stored
     // directly that would be 8-byte pieces of 32-byte row segments.  The converted tile instead
     // goes through the wave's own slice of the (now idle) ring, and leaves as 16 bytes per lane
-    // along whole rows.
+    // along whole rows.  It does so in ECH groups of columns: the stores of a group (which the
+    // memory system takes at its own pace, 3 us for the 98 KB of an FC1 tile when every workgroup
+    // stores at once) drain while the next group is converted.
     __syncthreads();                                        // every wave has left the ring
     unsigned char *mine = lds + wave * (64 * EPITCH);
+    constexpr int ECH = (NT % 3 == 0 && BN >= 144) ? 3 : (BN == 96 ? 2 : 1);
+    constexpr int TPC = NT / ECH, CPC = TPC * 2;             // accumulator tiles / 16-byte chunks per row and group
+    static_for<0, ECH>([&](auto chc) {
+      constexpr int ch = decltype(chc)::value;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
-        lds_store8(mine + (i * 16 + l16) * EPITCH + (j * 16 + g * 4) * 2, cvt(m0 + wave * 64 + i * 16 + l16, j * 16 + g * 4, acc[i][j]));
-    constexpr int CPR = BN / 8;                              // 16-byte chunks per row
+        for (int j = ch * TPC; j < (ch + 1) * TPC; ++j)
+          lds_store8(mine + (i * 16 + l16) * EPITCH + (j * 16 + g * 4) * 2, cvt(m0 + wave * 64 + i * 16 + l16, j * 16 + g * 4, acc[i][j]));
+      if constexpr (ch == ECH - 1) STAGE_MARK(tb, 3);
 #pragma unroll
-    for (int t = 0; t < CPR; ++t) {                          // 64 rows x CPR chunks = CPR per lane
-      const int c = t * 64 + lane, row = c / CPR, col8 = c % CPR;
-      const u4 v = lds_load16(mine + row * EPITCH + col8 * 16);
-      store16(m0 + wave * 64 + row, col8 * 8, v);
-    }
+      for (int t = 0; t < CPC; ++t) {                        // 64 rows x CPC chunks = CPC per lane
+        const int c = t * 64 + lane, row = c / CPC, col8 = ch * CPC + c % CPC;
+        const u4 v = lds_load16(mine + row * EPITCH + col8 * 16);
+        store16(m0 + wave * 64 + row, col8 * 8, v);
+      }
+    });
+    STAGE_MARK(tb, 4);
+#ifdef SOUFFLE_STAGE_MARKS
+    if (tb && tb->trace) { __builtin_amdgcn_s_waitcnt(0); trace_mark(*tb, 5); }
+#endif
   }
 };
 
