@@ -329,7 +329,11 @@ __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, 
 using BigQkv = GemmBig<144, 5>;
 using BigFc1 = GemmBig<192, 5>;
 using BigOut = GemmBig<48, 5>;
-using BigFc2 = GemmBig<96, 5>;                 // FC2: 8 column tiles x 2 halves of K = 256 tiles at M = 4096
+// FC2: parts of K, each a partial sum of its own.  16 tiles per row block: 8 column tiles x 2 parts of K
+// (4 x 4 with 192-column tiles has the better operand reuse but twice the partial sums to write and to
+// read back: 1564 us against 1535 for the 12 layers at M = 4096).
+constexpr int kFc2Split = 2;
+using BigFc2 = GemmBig<H * kFc2Split / 16, 5>;
 constexpr int kBigLds = BigFc1::LDS_BYTES;
 static_assert(BigQkv::LDS_BYTES <= kBigLds && BigOut::LDS_BYTES <= kBigLds && BigFc2::LDS_BYTES <= kBigLds, "FC1 has the largest ring");
 
@@ -422,51 +426,52 @@ __device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, 
     BigOut::run(lds, X, K, tm * 256, 0, K / 32, wptr, cvt, store16);
   }
 }
-// A pre-LayerNorm sum in two halves of K: X[:, :K/2].W[:K/2] + bias + resid and X[:, K/2:].W[K/2:],
-// both fp16, into the two halves of the (here otherwise unused) partials area (see fc2_sum_lo /
-// fc2_sum_hi; not into z1, which the out-projection of the same layer has written); big_ln adds them.
-__device__ __forceinline__ half_t *fc2_sum_lo(const Params &a) { return reinterpret_cast<half_t *>(a.part); }
-__device__ __forceinline__ half_t *fc2_sum_hi(const Params &a) { return reinterpret_cast<half_t *>(a.part) + (size_t)a.M * H; }
+// A pre-LayerNorm sum in kFc2Split parts of K: part 0 = X[:, part 0].W[part 0] + bias + resid, part
+// p = X[:, part p].W[part p], all fp16, M x H each, one after the other in the (here otherwise
+// unused) partials area (not in z1, which the out-projection of the same layer has written); the
+// LayerNorm adds them in order.
+__device__ __forceinline__ half_t *fc2_sums(const Params &a) { return reinterpret_cast<half_t *>(a.part); }
 template <bool COH>
 __device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a, const half_t *X, int K, const half_t *W,
                                             const half_t *bias, const half_t *resid, int first, int stride) {
-  const int m_tiles = a.M / 256, n_tiles = H / BigFc2::kBN;
-  half_t *zlo = fc2_sum_lo(a), *zhi = fc2_sum_hi(a);
-  for (int it = first; it < m_tiles * n_tiles * 2; it += stride) {
+  const int m_tiles = a.M / 256;
+  for (int it = first; it < m_tiles * 16; it += stride) {
     int tm, tn2;
-    big_tile(it, m_tiles, n_tiles * 2, &tm, &tn2);
-    const int ks = tn2 & 1, n0 = (tn2 >> 1) * BigFc2::kBN, k0 = ks * (K / 2);
+    big_tile(it, m_tiles, 16, &tm, &tn2);
+    const int ks = tn2 % kFc2Split, n0 = (tn2 / kFc2Split) * BigFc2::kBN, k0 = ks * (K / kFc2Split);
+    half_t *zp = fc2_sums(a) + (size_t)ks * a.M * H;
     auto wptr = [&](int k, int col) { return W + (size_t)k * H + n0 + col; };
     const half_t *bz = bias ? bias : g_zero_row;
-    auto cvt_lo = [&](int m, int nr, f4 v) {
+    auto cvt_first = [&](int m, int nr, f4 v) {
       const int n = n0 + nr;
       const h4 r = as_h4(ld8<false>(resid, (m * H + n) * 2));
       v = add_row4(v, bz, n) + f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
       return pack_h4(v);
     };
-    auto cvt_hi = [&](int, int, f4 v) { return pack_h4(v); };
-    auto store_lo = [&](int m, int nr, u4 v) { st16<COH>(zlo, (m * H + n0 + nr) * 2, v); };
-    auto store_hi = [&](int m, int nr, u4 v) { st16<COH>(zhi, (m * H + n0 + nr) * 2, v); };
+    auto cvt_rest = [&](int, int, f4 v) { return pack_h4(v); };
+    auto store16 = [&](int m, int nr, u4 v) { st16<COH>(zp, (m * H + n0 + nr) * 2, v); };
     f4 acc[4][BigFc2::NT];
-    BigFc2::mainloop(lds, X, K, tm * 256, k0, (K / 2) / 32, wptr, acc);
-    if (ks == 0) BigFc2::epilogue(lds, tm * 256, acc, cvt_lo, store_lo);
-    else BigFc2::epilogue(lds, tm * 256, acc, cvt_hi, store_hi);
+    BigFc2::mainloop(lds, X, K, tm * 256, k0, (K / kFc2Split) / 32, wptr, acc);
+    if (ks == 0) BigFc2::epilogue(lds, tm * 256, acc, cvt_first, store16);
+    else BigFc2::epilogue(lds, tm * 256, acc, cvt_rest, store16);
   }
 }
-// out[m] = LN(z1[m] (+ z2[m])) * g + b; one wave per row, two-pass statistics in fp32 registers.
+// out[m] = LN(z[0][m] + ... + z[NZ-1][m]) * g + b (z[p] = z + p M H; summed in this order); one wave
+// per row, two-pass statistics in fp32 registers.
 // NR rows (m0, m0 + mstep, ...) per call: their loads are all issued before the first is used.
-template <bool COH, int NR>
-__device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z1, const half_t *z2, const half_t *gam, const half_t *bet, half_t *out, int m0, int mstep) {
+template <bool COH, int NR, int NZ>
+__device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z, const half_t *gam, const half_t *bet, half_t *out, int m0, int mstep) {
   const int lane = opaque_thread_id() & 63;
-  u2 raw[NR][3], raw2[NR][3];
+  u2 raw[NR][NZ][3];
 #pragma unroll
   for (int r = 0; r < NR; ++r)
 #pragma unroll
-    for (int c = 0; c < 3; ++c) {
-      const int m = m0 + r * mstep;
-      raw[r][c] = ld8<false>(z1, (m * H + c * 256 + lane * 4) * 2);
-      if (z2) raw2[r][c] = ld8<false>(z2, (m * H + c * 256 + lane * 4) * 2);
-    }
+    for (int p = 0; p < NZ; ++p)
+#pragma unroll
+      for (int c = 0; c < 3; ++c) {
+        const int m = m0 + r * mstep;
+        raw[r][p][c] = ld8<false>(z + (size_t)p * a.M * H, (m * H + c * 256 + lane * 4) * 2);
+      }
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
     const int m = m0 + r * mstep;
@@ -474,10 +479,11 @@ __device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z1, c
     float sum = 0.f;
 #pragma unroll
     for (int c = 0; c < 3; ++c) {
-      const h4 q = as_h4(raw[r][c]);
+      const h4 q = as_h4(raw[r][0][c]);
       v[c] = f4{(float)q[0], (float)q[1], (float)q[2], (float)q[3]};
-      if (z2) {
-        const h4 q2 = as_h4(raw2[r][c]);
+#pragma unroll
+      for (int p = 1; p < NZ; ++p) {
+        const h4 q2 = as_h4(raw[r][p][c]);
         v[c] += f4{(float)q2[0], (float)q2[1], (float)q2[2], (float)q2[3]};
       }
       sum += v[c][0] + v[c][1] + v[c][2] + v[c][3];
@@ -507,9 +513,9 @@ __device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z1, c
     }
   }
 }
-template <bool COH>
-__device__ __forceinline__ void big_ln(const Params &a, const half_t *z1, const half_t *z2, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
-  for (int m = first_row; m < a.M; m += row_stride) big_ln_rows<COH, 1>(a, z1, z2, gam, bet, out, m, 0);
+template <bool COH, int NZ>
+__device__ __forceinline__ void big_ln(const Params &a, const half_t *z, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
+  for (int m = first_row; m < a.M; m += row_stride) big_ln_rows<COH, 1, NZ>(a, z, gam, bet, out, m, 0);
 }
 
 // The LayerNorm that follows a pre-LayerNorm sum, without a grid barrier in between.  A 256-row
@@ -521,9 +527,9 @@ __device__ __forceinline__ void big_ln(const Params &a, const half_t *z1, const 
 // the same.  The words are cleared by the launch itself before its first grid barrier and tags grow
 // within a launch.  Rows are normalised by the same routine as in the separate LayerNorm stage:
 // identical results.
-static_assert(H / BigOut::kBN == 16 && 2 * (H / BigFc2::kBN) == 16, "16 tiles per row block");
-template <bool COH>
-__device__ __forceinline__ void rowblock_ln(const Params &a, unsigned tag, const half_t *z1, const half_t *z2, const half_t *gam, const half_t *bet,
+static_assert(H / BigOut::kBN == 16 && kFc2Split * (H / BigFc2::kBN) == 16, "16 tiles per row block");
+template <bool COH, int NZ>
+__device__ __forceinline__ void rowblock_ln(const Params &a, unsigned tag, const half_t *z, const half_t *gam, const half_t *bet,
                                             half_t *out, int first, int stride, const GridBarrier *tb = nullptr) {
   const int m_tiles = a.M / 256, wave = threadIdx.x >> 6;
   STAGE_MARK(tb, 0);
@@ -552,7 +558,7 @@ __device__ __forceinline__ void rowblock_ln(const Params &a, unsigned tag, const
     }
     __syncthreads();
     STAGE_MARK(tb, 2);
-    big_ln_rows<COH, 4>(a, z1, z2, gam, bet, out, tm * 256 + tn * 16 + wave * 4, 1);
+    big_ln_rows<COH, 4, NZ>(a, z, gam, bet, out, tm * 256 + tn * 16 + wave * 4, 1);
     STAGE_MARK(tb, 3);
   }
 }
@@ -1181,7 +1187,7 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       grid_sync(bar);
       if constexpr (BIG) {
         big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, xin, first, stride);
-        rowblock_ln<true>(a, 2u * l + 1u, a.z1, nullptr, w.ln1_g, w.ln1_b, a.y1, first, stride, &bar);
+        rowblock_ln<true, 1>(a, 2u * l + 1u, a.z1, w.ln1_g, w.ln1_b, a.y1, first, stride, &bar);
       } else {
         stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
         grid_sync(bar);
@@ -1193,7 +1199,7 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       grid_sync(bar);
       if constexpr (BIG) {
         big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, a.y1, first, stride);
-        rowblock_ln<true>(a, 2u * l + 2u, fc2_sum_lo(a), fc2_sum_hi(a), w.ln2_g, w.ln2_b, yout, first, stride, &bar);
+        rowblock_ln<true, kFc2Split>(a, 2u * l + 2u, fc2_sums(a), w.ln2_g, w.ln2_b, yout, first, stride, &bar);
       } else {
         stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
         grid_sync(bar);
@@ -1397,8 +1403,9 @@ __global__ void __launch_bounds__(256) k_presum2_big(Args a, const half_t *X, in
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   big_presum2<false>(lds_raw, a, X, K, W, bias, resid, blockIdx.x, gridDim.x);
 }
-__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *z1, const half_t *z2, const half_t *gam, const half_t *bet, half_t *out) {
-  big_ln<false>(a, z1, z2, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
+template <int NZ>
+__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *z, const half_t *gam, const half_t *bet, half_t *out) {
+  big_ln<false, NZ>(a, z, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
 }
 template <int MODE>
 __global__ void __launch_bounds__(256) k_fc1(Args a, int l) {
@@ -1495,7 +1502,8 @@ static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   p.off_z1 = take(M * H * 2);
   p.off_y1 = take(M * H * 2);
   p.off_h = take(M * F * 2);
-  p.off_part = take((size_t)(p.splitk_f > p.splitk_o ? p.splitk_f : p.splitk_o) * M * H * 4);
+  // fp32 split-K partial sums, or (many rows) FC2's kFc2Split fp16 pre-LayerNorm partial sums
+  p.off_part = take(p.big ? (size_t)kFc2Split * M * H * 2 : (size_t)(p.splitk_f > p.splitk_o ? p.splitk_f : p.splitk_o) * M * H * 4);
   p.off_yl = take(M * H * 2);
   p.layer_stride = off - first;                       // one set of inter-stage buffers per layer
   p.flow_bytes = p.off_yl - p.off_qkv;
@@ -1721,7 +1729,7 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     else hipLaunchKernelGGL(k_attn_small, dim3(grid_for((a.B * NH + 7) / 8 * 8 * (a.S / 16))), dim3(256), attn_small_lds_bytes(a.S), st, a);
     if constexpr (MODE == 2) {
       hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * (H / BigOut::kBN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, w.b_o, xin);
-      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.z1, (const half_t *)nullptr, w.ln1_g, w.ln1_b, a.y1);
+      hipLaunchKernelGGL(k_ln_big<1>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.z1, w.ln1_g, w.ln1_b, a.y1);
     } else if constexpr (LARGE) {
       hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, 1);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, 1, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
@@ -1730,8 +1738,8 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     }
     hipLaunchKernelGGL(k_fc1<MODE>, dim3(grid_for((a.M / BM_QKV) * (F / BN))), dim3(256), GEMM_LDS, st, a, l);
     if constexpr (MODE == 2) {
-      hipLaunchKernelGGL(k_presum2_big, dim3(grid_for((a.M / 256) * (H / BigFc2::kBN) * 2)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, w.b_fc2, a.y1);
-      hipLaunchKernelGGL(k_ln_big, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.part, (const half_t *)a.part + (size_t)a.M * H, w.ln2_g, w.ln2_b, yout);
+      hipLaunchKernelGGL(k_presum2_big, dim3(grid_for((a.M / 256) * 16)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, w.b_fc2, a.y1);
+      hipLaunchKernelGGL(k_ln_big<kFc2Split>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.part, w.ln2_g, w.ln2_b, yout);
     } else {
       hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_FC2) * (H / BN) * a.splitk_f)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, a.splitk_f);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout);

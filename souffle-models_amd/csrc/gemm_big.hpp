@@ -122,18 +122,18 @@ struct GemmBig {
   __device__ static __forceinline__ void mainloop(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, int nkt, WPtr wptr, f4 (&acc)[4][NT],
                                                   const GridBarrier *tb = nullptr) {
     const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+    STAGE_MARK(tb, 0);
+    __syncthreads();                                        // the previous user of the ring is done
+    const unsigned ring = lds_address(lds);
+#pragma unroll
+    for (int s = 0; s < NSTAGE - 1; ++s) issue_range<0, LPW>(tid, ring + s * STAGE, X, ldx, m0, k0 + s * 32, wptr);
+    // (the accumulators are cleared while the first stages travel)
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < NT; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < 4; ++i) mfma_pin(acc[i], true);
-
-    STAGE_MARK(tb, 0);
-    __syncthreads();                                        // the previous user of the ring is done
-    const unsigned ring = lds_address(lds);
-#pragma unroll
-    for (int s = 0; s < NSTAGE - 1; ++s) issue_range<0, LPW>(tid, ring + s * STAGE, X, ldx, m0, k0 + s * 32, wptr);
 
     // byte offsets of this lane's operand reads inside a stage
     int xoff[4];
