@@ -404,11 +404,12 @@ __device__ __forceinline__ void big_fc1(unsigned char *lds, const Params &a, con
     else BigFc1::epilogue(lds, tm * 256, acc, cvt_gelu, store16, tb);
   }
 }
-// z = X[M][K].W[K][768] + bias + resid, fp16, into a.z1 (the pre-LayerNorm sum of the out-projection
-// and of FC2; no split of K: 256 tiles already fill the device)
+// z = X[M][K].W[K][768] + bias, fp16, into a.z1 (the out-projection; no split of K: 256 tiles already
+// fill the device).  The residual is added by the LayerNorm that follows, which reads whole rows: read
+// here, 8 bytes per lane across 16 rows per instruction, it cost a tile 5 us.
 template <bool COH>
 __device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, const half_t *X, int K, const half_t *W,
-                                           const half_t *bias, const half_t *resid, int first, int stride) {
+                                           const half_t *bias, int first, int stride) {
   const int m_tiles = a.M / 256, n_tiles = H / BigOut::kBN;
   for (int it = first; it < m_tiles * n_tiles; it += stride) {
     int tm, tn;
@@ -416,24 +417,19 @@ __device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, 
     const int n0 = tn * BigOut::kBN;
     auto wptr = [&](int k, int col) { return W + (size_t)k * H + n0 + col; };
     const half_t *bz = bias ? bias : g_zero_row;
-    auto cvt = [&](int m, int nr, f4 v) {
-      const int n = n0 + nr;
-      const h4 r = as_h4(ld8<false>(resid, (m * H + n) * 2));
-      v = add_row4(v, bz, n) + f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
-      return pack_h4(v);
-    };
+    auto cvt = [&](int, int nr, f4 v) { return pack_h4(add_row4(v, bz, n0 + nr)); };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.z1, (m * H + n0 + nr) * 2, v); };
     BigOut::run(lds, X, K, tm * 256, 0, K / 32, wptr, cvt, store16);
   }
 }
-// A pre-LayerNorm sum in kFc2Split parts of K: part 0 = X[:, part 0].W[part 0] + bias + resid, part
+// A pre-LayerNorm sum in kFc2Split parts of K: part 0 = X[:, part 0].W[part 0] + bias, part
 // p = X[:, part p].W[part p], all fp16, M x H each, one after the other in the (here otherwise
 // unused) partials area (not in z1, which the out-projection of the same layer has written); the
-// LayerNorm adds them in order.
+// LayerNorm adds them in order, then the residual.
 __device__ __forceinline__ half_t *fc2_sums(const Params &a) { return reinterpret_cast<half_t *>(a.part); }
 template <bool COH>
 __device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a, const half_t *X, int K, const half_t *W,
-                                            const half_t *bias, const half_t *resid, int first, int stride) {
+                                            const half_t *bias, int first, int stride) {
   const int m_tiles = a.M / 256;
   for (int it = first; it < m_tiles * 16; it += stride) {
     int tm, tn2;
@@ -442,12 +438,7 @@ __device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a,
     half_t *zp = fc2_sums(a) + (size_t)ks * a.M * H;
     auto wptr = [&](int k, int col) { return W + (size_t)k * H + n0 + col; };
     const half_t *bz = bias ? bias : g_zero_row;
-    auto cvt_first = [&](int m, int nr, f4 v) {
-      const int n = n0 + nr;
-      const h4 r = as_h4(ld8<false>(resid, (m * H + n) * 2));
-      v = add_row4(v, bz, n) + f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
-      return pack_h4(v);
-    };
+    auto cvt_first = [&](int, int nr, f4 v) { return pack_h4(add_row4(v, bz, n0 + nr)); };
     auto cvt_rest = [&](int, int, f4 v) { return pack_h4(v); };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(zp, (m * H + n0 + nr) * 2, v); };
     f4 acc[4][BigFc2::NT];
@@ -456,13 +447,13 @@ __device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a,
     else BigFc2::epilogue(lds, tm * 256, acc, cvt_rest, store16);
   }
 }
-// out[m] = LN(z[0][m] + ... + z[NZ-1][m]) * g + b (z[p] = z + p M H; summed in this order); one wave
-// per row, two-pass statistics in fp32 registers.
+// out[m] = LN(z[0][m] + ... + z[NZ-1][m] + resid[m]) * g + b (z[p] = z + p M H; summed in this order);
+// one wave per row, two-pass statistics in fp32 registers.
 // NR rows (m0, m0 + mstep, ...) per call: their loads are all issued before the first is used.
 template <bool COH, int NR, int NZ>
-__device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z, const half_t *gam, const half_t *bet, half_t *out, int m0, int mstep) {
+__device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z, const half_t *resid, const half_t *gam, const half_t *bet, half_t *out, int m0, int mstep) {
   const int lane = opaque_thread_id() & 63;
-  u2 raw[NR][NZ][3];
+  u2 raw[NR][NZ + 1][3];
 #pragma unroll
   for (int r = 0; r < NR; ++r)
 #pragma unroll
@@ -471,6 +462,7 @@ __device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z, co
       for (int c = 0; c < 3; ++c) {
         const int m = m0 + r * mstep;
         raw[r][p][c] = ld8<false>(z + (size_t)p * a.M * H, (m * H + c * 256 + lane * 4) * 2);
+        if (p == 0) raw[r][NZ][c] = ld8<false>(resid, (m * H + c * 256 + lane * 4) * 2);
       }
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
@@ -482,7 +474,7 @@ __device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z, co
       const h4 q = as_h4(raw[r][0][c]);
       v[c] = f4{(float)q[0], (float)q[1], (float)q[2], (float)q[3]};
 #pragma unroll
-      for (int p = 1; p < NZ; ++p) {
+      for (int p = 1; p <= NZ; ++p) {
         const h4 q2 = as_h4(raw[r][p][c]);
         v[c] += f4{(float)q2[0], (float)q2[1], (float)q2[2], (float)q2[3]};
       }
@@ -514,8 +506,8 @@ __device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z, co
   }
 }
 template <bool COH, int NZ>
-__device__ __forceinline__ void big_ln(const Params &a, const half_t *z, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
-  for (int m = first_row; m < a.M; m += row_stride) big_ln_rows<COH, 1, NZ>(a, z, gam, bet, out, m, 0);
+__device__ __forceinline__ void big_ln(const Params &a, const half_t *z, const half_t *resid, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
+  for (int m = first_row; m < a.M; m += row_stride) big_ln_rows<COH, 1, NZ>(a, z, resid, gam, bet, out, m, 0);
 }
 
 // The LayerNorm that follows a pre-LayerNorm sum, without a grid barrier in between.  A 256-row
@@ -529,7 +521,7 @@ __device__ __forceinline__ void big_ln(const Params &a, const half_t *z, const h
 // identical results.
 static_assert(H / BigOut::kBN == 16 && kFc2Split * (H / BigFc2::kBN) == 16, "16 tiles per row block");
 template <bool COH, int NZ>
-__device__ __forceinline__ void rowblock_ln(const Params &a, unsigned tag, const half_t *z, const half_t *gam, const half_t *bet,
+__device__ __forceinline__ void rowblock_ln(const Params &a, unsigned tag, const half_t *z, const half_t *resid, const half_t *gam, const half_t *bet,
                                             half_t *out, int first, int stride, const GridBarrier *tb = nullptr) {
   const int m_tiles = a.M / 256, wave = threadIdx.x >> 6;
   STAGE_MARK(tb, 0);
@@ -558,7 +550,7 @@ __device__ __forceinline__ void rowblock_ln(const Params &a, unsigned tag, const
     }
     __syncthreads();
     STAGE_MARK(tb, 2);
-    big_ln_rows<COH, 4, NZ>(a, z, gam, bet, out, tm * 256 + tn * 16 + wave * 4, 1);
+    big_ln_rows<COH, 4, NZ>(a, z, resid, gam, bet, out, tm * 256 + tn * 16 + wave * 4, 1);
     STAGE_MARK(tb, 3);
   }
 }
@@ -1186,8 +1178,8 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       stage_attn_t<true, NKT>(lds, a, first, stride);
       grid_sync(bar);
       if constexpr (BIG) {
-        big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, xin, first, stride);
-        rowblock_ln<true, 1>(a, 2u * l + 1u, a.z1, w.ln1_g, w.ln1_b, a.y1, first, stride, &bar);
+        big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, first, stride);
+        rowblock_ln<true, 1>(a, 2u * l + 1u, a.z1, xin, w.ln1_g, w.ln1_b, a.y1, first, stride, &bar);
       } else {
         stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
         grid_sync(bar);
@@ -1198,8 +1190,8 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       else stage_fc1<true, Tile>(lds, a, w, first, stride);
       grid_sync(bar);
       if constexpr (BIG) {
-        big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, a.y1, first, stride);
-        rowblock_ln<true, kFc2Split>(a, 2u * l + 2u, fc2_sums(a), w.ln2_g, w.ln2_b, yout, first, stride, &bar);
+        big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, first, stride);
+        rowblock_ln<true, kFc2Split>(a, 2u * l + 2u, fc2_sums(a), a.y1, w.ln2_g, w.ln2_b, yout, first, stride, &bar);
       } else {
         stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
         grid_sync(bar);
@@ -1395,17 +1387,17 @@ __global__ void __launch_bounds__(256) k_ln(Args a, int splitk, const half_t *bi
                                             const half_t *gam, const half_t *bet, half_t *out) {
   stage_ln<false>(a, splitk, bias, resid, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
 }
-__global__ void __launch_bounds__(256) k_presum_big(Args a, const half_t *X, int K, const half_t *W, const half_t *bias, const half_t *resid) {
+__global__ void __launch_bounds__(256) k_presum_big(Args a, const half_t *X, int K, const half_t *W, const half_t *bias) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  big_presum<false>(lds_raw, a, X, K, W, bias, resid, blockIdx.x, gridDim.x);
+  big_presum<false>(lds_raw, a, X, K, W, bias, blockIdx.x, gridDim.x);
 }
-__global__ void __launch_bounds__(256) k_presum2_big(Args a, const half_t *X, int K, const half_t *W, const half_t *bias, const half_t *resid) {
+__global__ void __launch_bounds__(256) k_presum2_big(Args a, const half_t *X, int K, const half_t *W, const half_t *bias) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  big_presum2<false>(lds_raw, a, X, K, W, bias, resid, blockIdx.x, gridDim.x);
+  big_presum2<false>(lds_raw, a, X, K, W, bias, blockIdx.x, gridDim.x);
 }
 template <int NZ>
-__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *z, const half_t *gam, const half_t *bet, half_t *out) {
-  big_ln<false, NZ>(a, z, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
+__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *z, const half_t *resid, const half_t *gam, const half_t *bet, half_t *out) {
+  big_ln<false, NZ>(a, z, resid, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
 }
 template <int MODE>
 __global__ void __launch_bounds__(256) k_fc1(Args a, int l) {
@@ -1728,8 +1720,8 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     if (LARGE) hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), 2 * a.S * 128 + 64 * 128, st, a);
     else hipLaunchKernelGGL(k_attn_small, dim3(grid_for((a.B * NH + 7) / 8 * 8 * (a.S / 16))), dim3(256), attn_small_lds_bytes(a.S), st, a);
     if constexpr (MODE == 2) {
-      hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * (H / BigOut::kBN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, w.b_o, xin);
-      hipLaunchKernelGGL(k_ln_big<1>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.z1, w.ln1_g, w.ln1_b, a.y1);
+      hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * (H / BigOut::kBN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, w.b_o);
+      hipLaunchKernelGGL(k_ln_big<1>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.z1, xin, w.ln1_g, w.ln1_b, a.y1);
     } else if constexpr (LARGE) {
       hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, 1);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, 1, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
@@ -1738,8 +1730,8 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     }
     hipLaunchKernelGGL(k_fc1<MODE>, dim3(grid_for((a.M / BM_QKV) * (F / BN))), dim3(256), GEMM_LDS, st, a, l);
     if constexpr (MODE == 2) {
-      hipLaunchKernelGGL(k_presum2_big, dim3(grid_for((a.M / 256) * 16)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, w.b_fc2, a.y1);
-      hipLaunchKernelGGL(k_ln_big<kFc2Split>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.part, w.ln2_g, w.ln2_b, yout);
+      hipLaunchKernelGGL(k_presum2_big, dim3(grid_for((a.M / 256) * 16)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, w.b_fc2);
+      hipLaunchKernelGGL(k_ln_big<kFc2Split>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.part, (const half_t *)a.y1, w.ln2_g, w.ln2_b, yout);
     } else {
       hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_FC2) * (H / BN) * a.splitk_f)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, a.splitk_f);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout);
