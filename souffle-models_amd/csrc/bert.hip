@@ -843,24 +843,82 @@ __device__ __forceinline__ void issue_rows64(unsigned char *lds, const half_t *s
   }
 }
 
+// The loads of one attention item (K and V of the head, 64 query rows), through inline assembly so
+// that the caller decides what to wait for (see load_lds16); every wave issues kAttnLoads<NKT> of them.
+template <int NKT>
+constexpr int kAttnLoads = 2 * (NKT * 16 / 32) + 2;
+template <int MODE>
+__device__ __forceinline__ void issue_rows64_nowait(unsigned lds_addr, const half_t *src, int rows) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int inst = wave; inst < rows / 8; inst += 4) {
+    const int sl = inst * 64 + lane, r = sl >> 3, c = (sl & 7) ^ (MODE == 0 ? ((r >> 1) & 7) : (r & 2));
+    load_lds16(src + (size_t)r * HD + c * 8, lds_addr + inst * 1024);
+  }
+}
+template <int NKT>
+__device__ __forceinline__ void attn_issue(unsigned char *lds, const Params &a, int item) {
+  constexpr int S = NKT * 16;
+  const int qblocks = S / 64;
+  const int qb = item % qblocks, bh = item / qblocks;
+  const int head_off = bh * S * HD;                              // halves, within one of q/k/v
+  const size_t plane = (size_t)a.B * NH * S * HD;
+  const unsigned base = lds_address(lds);
+  issue_rows64_nowait<0>(base, a.qkv + plane + head_off, S);
+  issue_rows64_nowait<1>(base + S * 128, a.qkv + 2 * plane + head_off, S);
+  issue_rows64_nowait<0>(base + 2 * S * 128, a.qkv + head_off + (size_t)qb * 64 * HD, 64);
+}
+template <int NKT>
+constexpr int kAttnItemLds = 2 * NKT * 16 * 128 + 64 * 128;
+
+// PLAIN: no mask and no probabilities to write (tested once per item: a uniform test per key tile
+// inside the unrolled loops is not hoisted by the compiler and breaks them into small blocks).
+template <bool COH, int NKT, bool PLAIN>
+__device__ __forceinline__ void attn_compute_t(unsigned char *lds, const Params &a, int item);
+template <bool COH, int NKT>
+__device__ __forceinline__ void attn_compute(unsigned char *lds, const Params &a, int item) {
+  if (!a.mask && !a.probs) attn_compute_t<COH, NKT, true>(lds, a, item);
+  else attn_compute_t<COH, NKT, false>(lds, a, item);
+}
+
 template <bool COH, int NKT>
 __device__ __forceinline__ void attn_item(half_t *lds_h, const Params &a, int item) {
-  constexpr int S = NKT * 16;
   unsigned char *lds = reinterpret_cast<unsigned char *>(lds_h);
+  __syncthreads();   // LDS reuse
+  attn_issue<NKT>(lds, a, item);
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  attn_compute<COH, NKT>(lds, a, item);
+}
+
+// One work unit after the other with the loads of the next in flight while this one is computed
+// (two LDS buffers).  `item_of(it)`: work unit -> item.
+template <bool COH, int NKT, class ItemOf>
+__device__ __forceinline__ void attn_items_pipelined(unsigned char *lds, const Params &a, int first, int stride, int items, ItemOf item_of) {
+  if (first >= items) return;
+  __syncthreads();   // LDS reuse
+  attn_issue<NKT>(lds, a, item_of(first));
+  int cur = 0;
+  for (int it = first; it < items; it += stride) {
+    if (it + stride < items) {
+      attn_issue<NKT>(lds + (cur ^ 1) * kAttnItemLds<NKT>, a, item_of(it + stride));
+      wait_vmcnt<kAttnLoads<NKT>>();      // all but the loads just issued (results stored earlier included)
+    } else {
+      wait_vmcnt<0>();
+    }
+    __syncthreads();
+    attn_compute<COH, NKT>(lds + cur * kAttnItemLds<NKT>, a, item_of(it));
+    __syncthreads();   // this buffer is refilled in the next turn
+    cur ^= 1;
+  }
+}
+
+template <bool COH, int NKT, bool PLAIN>
+__device__ __forceinline__ void attn_compute_t(unsigned char *lds, const Params &a, int item) {
+  constexpr int S = NKT * 16;
   unsigned char *ks_ = lds, *vs_ = lds + S * 128, *qs_ = lds + 2 * S * 128;
   const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
   const int qblocks = S / 64;
   const int qb = item % qblocks, bh = item / qblocks, b = bh / NH, hh = bh % NH;
-  const int head_off = ((b * NH + hh) * S) * HD;                 // halves, within one of q/k/v
-  const size_t plane = (size_t)a.B * NH * S * HD;
-  const half_t *Q = a.qkv + head_off + (size_t)qb * 64 * HD, *K = a.qkv + plane + head_off, *V = a.qkv + 2 * plane + head_off;
-
-  __syncthreads();   // LDS reuse
-  issue_rows64<false, 0>(ks_, K, S);
-  issue_rows64<false, 1>(vs_, V, S);
-  issue_rows64<false, 0>(qs_, Q, 64);
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
 
   const half_t *kh = reinterpret_cast<const half_t *>(ks_), *vh = reinterpret_cast<const half_t *>(vs_),
                *qh = reinterpret_cast<const half_t *>(qs_);
@@ -881,13 +939,18 @@ __device__ __forceinline__ void attn_item(half_t *lds_h, const Params &a, int it
     sc[t] = mfma_16x16x32(k1, qop[1], c);
   }
   // sc[t][v] = score(key = 16t + 4g + v, query = q0 + l16)
+  // softmax in base 2: exp(s - max) = exp2(s log2(e) - max'), log2(e) folded into the scale
+  constexpr float kLog2e = 1.4426950408889634f;
+  const float scale2 = a.scale * kLog2e;
   float mx = -INFINITY;
 #pragma unroll
   for (int t = 0; t < NKT; ++t) {
-    f4 sv = sc[t] * a.scale;
-    if (a.mask) {
-      const h4 mk = ldg<h4>(a.mask + ((size_t)b * S + q) * S + t * 16 + g * 4);
-      sv += f4{(float)mk[0], (float)mk[1], (float)mk[2], (float)mk[3]};
+    f4 sv = sc[t] * scale2;
+    if constexpr (!PLAIN) {
+      if (a.mask) {
+        const h4 mk = ldg<h4>(a.mask + ((size_t)b * S + q) * S + t * 16 + g * 4);
+        sv += f4{(float)mk[0], (float)mk[1], (float)mk[2], (float)mk[3]} * kLog2e;
+      }
     }
     sc[t] = sv;
     mx = fmaxf(mx, fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
@@ -898,18 +961,20 @@ __device__ __forceinline__ void attn_item(half_t *lds_h, const Params &a, int it
 #pragma unroll
   for (int t = 0; t < NKT; ++t) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) { sc[t][i] = __expf(sc[t][i] - mx); sum += sc[t][i]; }
+    for (int i = 0; i < 4; ++i) { sc[t][i] = __builtin_amdgcn_exp2f(sc[t][i] - mx); sum += sc[t][i]; }
   }
   sum += wave_xor(sum, 16);
   sum += wave_xor(sum, 32);
-  const float inv = 1.0f / sum;
+  const float inv = __builtin_amdgcn_rcpf(sum);
   h4 p[NKT];
 #pragma unroll
   for (int t = 0; t < NKT; ++t) {
     const f4 pr = sc[t] * inv;
     p[t] = h4{(half_t)pr[0], (half_t)pr[1], (half_t)pr[2], (half_t)pr[3]};
-    if (a.probs)
-      st8<false>(a.probs, (int)((((size_t)(b * NH + hh) * S + q) * S + t * 16 + g * 4) * 2), as_u2(p[t]));
+    if constexpr (!PLAIN) {
+      if (a.probs)
+        st8<false>(a.probs, (int)((((size_t)(b * NH + hh) * S + q) * S + t * 16 + g * 4) * 2), as_u2(p[t]));
+    }
   }
   f4 o[HD / 16];
 #pragma unroll
@@ -1119,15 +1184,28 @@ __device__ __forceinline__ void stage_attn_small(unsigned char *lds, const Param
   }
 }
 
+// Work unit `it` (units it, it + 8, ... run on one XCD: workgroup b runs on XCD b % 8) -> attention
+// item.  The S / 64 query blocks of a head go to the same XCD, next to each other in time, so that
+// its L2 fetches the head's K and V once (at S = 128, B = 32: 19 MB instead of 30 MB per layer).
+__device__ __forceinline__ int attn_item_of(int it, int qblocks, int items) {
+  if ((gridDim.x & 7) != 0 || items % (8 * qblocks) != 0) return it;
+  const int x = it & 7, i = it >> 3;
+  return ((i / qblocks) * 8 + x) * qblocks + i % qblocks;
+}
 template <bool COH, int NKT>
 __device__ __forceinline__ void stage_attn_t(half_t *lds, const Params &a, int first, int stride) {
   const int items = a.B * NH * (a.S / 64);
-  for (int item = first; item < items; item += stride) attn_item<COH, NKT>(lds, a, item);
+  if constexpr (2 * kAttnItemLds<NKT> <= kBigLds)     // (the megakernel's LDS allocation is at least this)
+    attn_items_pipelined<COH, NKT>(reinterpret_cast<unsigned char *>(lds), a, first, stride, items,
+                                   [&](int it) { return attn_item_of(it, a.S / 64, items); });
+  else
+    for (int it = first; it < items; it += stride) attn_item<COH, NKT>(lds, a, attn_item_of(it, a.S / 64, items));
 }
 template <bool COH>
 __device__ __forceinline__ void stage_attn(half_t *lds, const Params &a, int first, int stride) {
   const int items = a.B * NH * (a.S / 64);
-  for (int item = first; item < items; item += stride) {
+  for (int it = first; it < items; it += stride) {
+    const int item = attn_item_of(it, a.S / 64, items);
     switch (a.S) {
       case 64: attn_item<COH, 4>(lds, a, item); break;
       case 128: attn_item<COH, 8>(lds, a, item); break;
