@@ -66,9 +66,9 @@ struct Args : Params {
 __device__ __forceinline__ Params layer_params(const Params &a, int l) {
   Params p = a;
   const size_t off = (size_t)(l % a.layer_sets) * a.layer_stride;
-  auto adv = [&](half_t *q) { return reinterpret_cast<half_t *>(reinterpret_cast<char *>(q) + off); };
+  auto adv = [&](half_t *q) { return uniform_ptr(reinterpret_cast<half_t *>(reinterpret_cast<char *>(q) + off)); };
   p.qkv = adv(a.qkv); p.ctx = adv(a.ctx); p.z1 = adv(a.z1); p.y1 = adv(a.y1); p.h = adv(a.h); p.yl = adv(a.yl);
-  p.part = reinterpret_cast<float *>(reinterpret_cast<char *>(a.part) + off);
+  p.part = uniform_ptr(reinterpret_cast<float *>(reinterpret_cast<char *>(a.part) + off));
   return p;
 }
 

@@ -101,9 +101,19 @@ __device__ __forceinline__ unsigned lds_address(const unsigned char *p) {
 // through (sc1) and read with sc1 so that it is coherent across the eight XCD L2s
 // without L2 write-back / invalidate fences.  Buffer instructions carry the cache
 // bits; the base pointer must be wave-uniform, the offset is in bytes (< 2 GiB).
+// A pointer that is the same in every lane, told to the compiler: computed with vector instructions
+// (a 64-bit multiply of a layer number by a stride is), a pointer sits in vector registers, and a
+// buffer access whose descriptor comes from there is wrapped in a loop over the distinct values
+// (four readfirstlanes, two compares, an exec-mask dance and a branch around every store).
+template <class T>
+__device__ __forceinline__ T *uniform_ptr(T *p) {
+  const unsigned long long v = reinterpret_cast<unsigned long long>(p);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+  return reinterpret_cast<T *>(((unsigned long long)hi << 32) | lo);
+}
 typedef __attribute__((address_space(8))) void *buf_rsrc_t;
 __device__ __forceinline__ auto make_rsrc(const void *base) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x7fffffff, 0x00027000);
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(uniform_ptr(base)), 0, 0x7fffffff, 0x00027000);
 }
 constexpr int kAuxSc1 = 16;
 
@@ -218,7 +228,7 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 constexpr int kCtlWords = 512;
 constexpr int kCtlErrWord = 400;
 constexpr int kCtlFlowWord = 401;
-constexpr int kMaxBarrierSpin = 1 << 24;
+constexpr int kMaxBarrierSpin = 1 << 20;       // about a second of polling; a barrier normally completes in microseconds
 
 struct GridBarrier {
   unsigned *ctl;
@@ -227,6 +237,7 @@ struct GridBarrier {
   unsigned epoch;    // number of the last barrier passed
   unsigned nblk;
   int count;         // barriers passed in this launch
+  bool failed;       // a wait of this launch gave up: later barriers are not waited for either
   // optional stage trace: thread 0 stamps the 100 MHz wall clock on entry to and exit from
   // every barrier: trace[(2*i + {0,1}) * nblk + block] for the i-th barrier of the launch,
   // plus up to 8 free-form marks inside the stage that precedes barrier i:
@@ -251,6 +262,7 @@ __device__ __forceinline__ void grid_barrier_begin(GridBarrier &b, unsigned *ctl
   b.ctl = ctl;
   b.nblk = gridDim.x;
   b.count = 0;
+  b.failed = false;
   b.trace = nullptr;
   b.trace_idx = 0;
   b.trace_cap = 0;
@@ -265,7 +277,11 @@ __device__ __forceinline__ void grid_barrier_begin(GridBarrier &b, unsigned *ctl
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  // No memory access of the program may cross the wait in either direction: a load hoisted above it
+  // would be one of the N youngest, and one of the loads the caller waits for could still be in flight.
+  asm volatile("" ::: "memory");
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+  asm volatile("" ::: "memory");
 }
 
 // `mid()` is called by every wave after the workgroup has arrived and before it starts to wait:
@@ -290,15 +306,17 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b, Mid mid) {
   }
   __builtin_amdgcn_s_barrier();            // the arrival (and the done flag) precede whatever mid() queues
   mid();
-  if (threadIdx.x < 64) {
+  if (threadIdx.x < 64 && !b.failed) {
     for (int spin = 0; spin < kMaxBarrierSpin; ++spin) {
       bool ok = true;
       if (threadIdx.x < 8 && threadIdx.x < b.nblk)
         ok = (int)(__hip_atomic_load(b.ctl + 256 + 32 * threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - b.epoch) >= 0;
       if (__all(ok)) break;
       __builtin_amdgcn_s_sleep(1);
-      if (spin == kMaxBarrierSpin - 1 && threadIdx.x == 0)   // gave up: the launch's output is invalid
-        (void)__hip_atomic_fetch_or(b.ctl + kCtlErrWord, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (spin == kMaxBarrierSpin - 1) {   // gave up: the launch's output is invalid, and it ends without further waits
+        b.failed = true;
+        if (threadIdx.x == 0) (void)__hip_atomic_fetch_or(b.ctl + kCtlErrWord, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
   }
   b.count++;
