@@ -329,10 +329,14 @@ __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, 
 using BigQkv = GemmBig<144, 5>;
 using BigFc1 = GemmBig<192, 5>;
 using BigOut = GemmBig<48, 5>;
-// FC2: parts of K, each a partial sum of its own.  16 tiles per row block: 8 column tiles x 2 parts of K
-// (4 x 4 with 192-column tiles has the better operand reuse but twice the partial sums to write and to
-// read back: 1564 us against 1535 for the 12 layers at M = 4096).
-constexpr int kFc2Split = 2;
+// FC2: parts of K, each a partial sum of its own.  16 tiles per row block: 4 column tiles of 192 x 4 parts of K
+// (the operand reuse of the FC1 tile; 8 column tiles of 96 x 2 parts writes and reads back half the partial
+// sums but runs its K loop at a worse ratio of operand bytes to MFMAs: 1434 us against 1417 for the 12
+// layers at M = 4096 in the fused kernel, 1430 against 1441 as separate launches).
+#ifndef SOUFFLE_FC2_SPLIT
+#define SOUFFLE_FC2_SPLIT 4
+#endif
+constexpr int kFc2Split = SOUFFLE_FC2_SPLIT;
 using BigFc2 = GemmBig<H * kFc2Split / 16, 5>;
 constexpr int kBigLds = BigFc1::LDS_BYTES;
 static_assert(BigQkv::LDS_BYTES <= kBigLds && BigOut::LDS_BYTES <= kBigLds && BigFc2::LDS_BYTES <= kBigLds, "FC1 has the largest ring");
