@@ -42,6 +42,14 @@ def test_bert_validation_without_gpu():
     big = sh.BertCfg(32, 128, 768, 12, 3072, 0, 0.125, 1e-12, 12, 0)
     n32 = lib.souffle_bert_workspace_bytes(C.byref(big))
     assert 0 < n1 < n32 < (1 << 30)
+    # few rows: one set of inter-stage buffers per layer; from 2048 rows (a multiple of 256) up: one set
+    # for all layers (plus 16 hand-over words per 256-row block), so the size no longer grows with depth
+    bytes_for = lambda b, s, layers: lib.souffle_bert_workspace_bytes(C.byref(sh.BertCfg(b, s, 768, 12, 3072, 0, 0.125, 1e-12, layers, 0)))
+    assert bytes_for(1, 128, 12) > 11 * (bytes_for(1, 128, 1) - 4096)
+    assert bytes_for(32, 128, 12) == bytes_for(32, 128, 1) == n32
+    per_row = 2 * (3 * 768 + 768 + 768 + 768 + 3072 + 768) + 4 * 768 * 2     # qkv, ctx, z1, y1, h, layer output; four fp16 partial sums
+    assert 4096 * per_row <= n32 <= 4096 * per_row + (1 << 16)
+    assert bytes_for(32, 100, 2) > bytes_for(32, 128, 2)                       # padded to 128 inside the call: room for the padded copies
     w = sh.BertLayerW()
     rc = lib.souffle_bert_layer_fused(C.byref(bad), C.byref(w), None, None, None, None, None, 0, None)
     assert rc == -2
