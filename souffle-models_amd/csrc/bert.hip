@@ -22,6 +22,11 @@ namespace souffle {
 namespace bert {
 
 constexpr int H = 768, NH = 12, HD = 64, F = 3072;
+#ifndef SOUFFLE_ROWBLOCK_LOCAL
+#define SOUFFLE_ROWBLOCK_LOCAL 1
+#endif
+constexpr bool kRowblockLocal = SOUFFLE_ROWBLOCK_LOCAL != 0;   // many rows: hand-overs among the 16 tiles of a row block instead of grid barriers
+
 constexpr int kMaxLayers = 24;
 constexpr int kMaxSplitK = 8;
 
@@ -514,7 +519,7 @@ __device__ __forceinline__ void big_ln(const Params &a, const half_t *z, const h
   for (int m = first_row; m < a.M; m += row_stride) big_ln_rows<COH, 1, NZ>(a, z, resid, gam, bet, out, m, 0);
 }
 
-// The LayerNorm that follows a pre-LayerNorm sum, without a grid barrier in between.  A 256-row
+// The LayerNorm that follows a pre-LayerNorm sum, without a grid barrier in between (rowblock_ln).  A 256-row
 // block of the sum is produced by 16 tiles (16 column tiles, or 8 column tiles x 2 halves of K).
 // A workgroup first finishes ALL its tiles of the stage, then publishes `tag` in the word of each
 // (row block, tile), then, per tile, waits for the 16 words of that row block and normalises 16
@@ -524,38 +529,56 @@ __device__ __forceinline__ void big_ln(const Params &a, const half_t *z, const h
 // within a launch.  Rows are normalised by the same routine as in the separate LayerNorm stage:
 // identical results.
 static_assert(H / BigOut::kBN == 16 && kFc2Split * (H / BigFc2::kBN) == 16, "16 tiles per row block");
-template <bool COH, int NZ>
-__device__ __forceinline__ void rowblock_ln(const Params &a, unsigned tag, const half_t *z, const half_t *resid, const half_t *gam, const half_t *bet,
-                                            half_t *out, int first, int stride, const GridBarrier *tb = nullptr) {
-  const int m_tiles = a.M / 256, wave = threadIdx.x >> 6;
-  STAGE_MARK(tb, 0);
+// Hand-over among the workgroups of a 256-row block: this workgroup's tiles of the stage are written
+// (all of them: nobody waits before that, so the waits end whatever the tile-to-workgroup mapping is):
+// publish `tag` in the word of each (row block, tile), run mid(), then wait until the 16 words of every
+// row block this workgroup has a tile in have reached `tag`.  Bounded like the grid barrier; a wait that
+// gave up ends all waiting of the launch.  With `bar.trace` the entry and exit times are stamped like
+// those of a grid barrier.
+template <class Mid>
+__device__ __forceinline__ void rowblock_sync(const Params &a, GridBarrier &bar, unsigned tag, int first, int stride, Mid mid) {
+  const int m_tiles = a.M / 256;
+  const bool tr = bar.trace && bar.trace_idx < bar.trace_cap && threadIdx.x == 0;
+  if (tr) bar.trace[(size_t)(2 * bar.trace_idx) * bar.nblk + blockIdx.x] = wall_clock64();
   __builtin_amdgcn_s_waitcnt(0);                 // this wave's write-through stores are acknowledged
   __syncthreads();
-  STAGE_MARK(tb, 1);
   if (threadIdx.x == 0)
     for (int it = first; it < m_tiles * 16; it += stride) {
       int tm, tn;
       big_tile(it, m_tiles, 16, &tm, &tn);
       __hip_atomic_store(a.rbflags + tm * 16 + tn, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-  for (int it = first; it < m_tiles * 16; it += stride) {
-    int tm, tn;
-    big_tile(it, m_tiles, 16, &tm, &tn);
-    if (threadIdx.x < 64) {
+  mid();
+  if (threadIdx.x < 64 && !bar.failed) {
+    for (int it = first; it < m_tiles * 16 && !bar.failed; it += stride) {
+      int tm, tn;
+      big_tile(it, m_tiles, 16, &tm, &tn);
       for (int spin = 0; spin < kMaxBarrierSpin; ++spin) {
         bool ok = true;
         if (threadIdx.x < 16)
           ok = (int)(__hip_atomic_load(a.rbflags + tm * 16 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - tag) >= 0;
         if (__all(ok)) break;
         __builtin_amdgcn_s_sleep(1);
-        if (spin == kMaxBarrierSpin - 1 && threadIdx.x == 0)   // gave up: the launch's output is invalid
-          (void)__hip_atomic_fetch_or(a.ctl + kCtlErrWord, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (spin == kMaxBarrierSpin - 1) {         // gave up: the launch's output is invalid
+          bar.failed = true;
+          if (threadIdx.x == 0) (void)__hip_atomic_fetch_or(a.ctl + kCtlErrWord, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
       }
     }
-    __syncthreads();
-    STAGE_MARK(tb, 2);
+  }
+  if (tr) bar.trace[(size_t)(2 * bar.trace_idx + 1) * bar.nblk + blockIdx.x] = wall_clock64();
+  bar.trace_idx++;
+  __syncthreads();
+}
+template <bool COH, int NZ>
+__device__ __forceinline__ void rowblock_ln(const Params &a, GridBarrier &bar, unsigned tag, const half_t *z, const half_t *resid, const half_t *gam,
+                                            const half_t *bet, half_t *out, int first, int stride) {
+  const int m_tiles = a.M / 256, wave = threadIdx.x >> 6;
+  rowblock_sync(a, bar, tag, first, stride, []() {});
+  for (int it = first; it < m_tiles * 16; it += stride) {
+    int tm, tn;
+    big_tile(it, m_tiles, 16, &tm, &tn);
     big_ln_rows<COH, 4, NZ>(a, z, resid, gam, bet, out, tm * 256 + tn * 16 + wave * 4, 1);
-    STAGE_MARK(tb, 3);
   }
 }
 
@@ -1205,6 +1228,21 @@ __device__ __forceinline__ void stage_attn_t(half_t *lds, const Params &a, int f
   else
     for (int it = first; it < items; it += stride) attn_item<COH, NKT>(lds, a, attn_item_of(it, a.S / 64, items));
 }
+// The attention items of the sequences of a 256-row block (48 of them whatever S <= 256 is), three to
+// each of the block's 16 tiles, for the tiles of this workgroup.
+template <bool COH, int NKT>
+__device__ __forceinline__ void stage_attn_rowblock(unsigned char *lds, const Params &a, int first, int stride) {
+  const int m_tiles = a.M / 256;
+  for (int it = first; it < m_tiles * 16; it += stride) {
+    int tm, tn;
+    big_tile(it, m_tiles, 16, &tm, &tn);
+    const int base = tm * 48 + tn * 3;
+    if constexpr (2 * kAttnItemLds<NKT> <= kBigLds)
+      attn_items_pipelined<COH, NKT>(lds, a, 0, 1, 3, [&](int j) { return base + j; });
+    else
+      for (int j = 0; j < 3; ++j) attn_item<COH, NKT>(reinterpret_cast<half_t *>(lds), a, base + j);
+  }
+}
 template <bool COH>
 __device__ __forceinline__ void stage_attn(half_t *lds, const Params &a, int first, int stride) {
   const int items = a.B * NH * (a.S / 64);
@@ -1246,39 +1284,59 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
   bool qkv_ready = false;
   // this kernel leaves data in the workspace buffers: the dataflow kernel must refill them
   if (first == 0 && threadIdx.x == 0) __hip_atomic_store(args.ctl + kCtlFlowWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if constexpr (BIG)   // the row-block hand-over words start every launch at 0 (two grid barriers before their first use)
+  if constexpr (BIG) {   // the row-block hand-over words start every launch at 0
     for (int i = first * 256 + threadIdx.x; i < (args.M / 256) * 16; i += stride * 256)
       __hip_atomic_store(args.rbflags + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    grid_sync(bar);
+  }
   for (int l = 0; l < args.num_layers; ++l) {
     const LayerW w = args.layers[l];
     const Params a = layer_params(args, l);
     half_t *yout = (l == a.num_layers - 1) ? a.y : a.yl;
-    if constexpr (LARGE) {
-      if constexpr (BIG) big_qkv<true>(lds_raw, a, w, xin, first, stride, &bar);
-      else stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
+    if constexpr (BIG) {
+      // Where a 256-row block holds whole sequences, every stage of a row block's tiles reads only what
+      // the 16 tiles of the same row block wrote in the stage before (attention included: the 48 items
+      // of the block's sequences go three to a tile), and the tile-to-workgroup mapping is the same in
+      // every stage: the 16 row blocks of M = 4096 then run as independent groups of 16 workgroups that
+      // hand over among themselves (rowblock_sync) and drift apart, so that the loads of one group
+      // overlap the MFMAs and the stores of others.  Otherwise (S = 384, 512) the stages are separated
+      // by grid barriers.  Hand-over k of layer l carries the tag 7 l + k.
+      const bool local = kRowblockLocal && 256 % a.S == 0;
+      auto sync = [&](unsigned k) {
+        if (local) rowblock_sync(a, bar, 7u * l + k, first, stride, []() {});
+        else grid_sync(bar);
+      };
+      big_qkv<true>(lds_raw, a, w, xin, first, stride, &bar);
+      sync(1);
+      if (local) stage_attn_rowblock<true, NKT>(lds_raw, a, first, stride);
+      else stage_attn_t<true, NKT>(lds, a, first, stride);
+      sync(2);
+      big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, first, stride);
+      rowblock_ln<true, 1>(a, bar, 7u * l + 3u, a.z1, xin, w.ln1_g, w.ln1_b, a.y1, first, stride);
+      sync(4);
+      big_fc1<true>(lds_raw, a, w, first, stride, &bar);
+      sync(5);
+      big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, first, stride);
+      rowblock_ln<true, kFc2Split>(a, bar, 7u * l + 6u, fc2_sums(a), a.y1, w.ln2_g, w.ln2_b, yout, first, stride);
+      if (l + 1 < a.num_layers) {   // the next layer writes this layer's buffers again: see Params
+        auto invalidate = [&]() { if (threadIdx.x < 64) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); };
+        if (local) rowblock_sync(a, bar, 7u * l + 7u, first, stride, invalidate);
+        else grid_sync(bar, invalidate);
+      }
+    } else if constexpr (LARGE) {
+      stage_qkv<true, Tile>(lds, a, w, xin, first, stride);
       grid_sync(bar);
       stage_attn_t<true, NKT>(lds, a, first, stride);
       grid_sync(bar);
-      if constexpr (BIG) {
-        big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, first, stride);
-        rowblock_ln<true, 1>(a, 2u * l + 1u, a.z1, xin, w.ln1_g, w.ln1_b, a.y1, first, stride, &bar);
-      } else {
-        stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
-        grid_sync(bar);
-        stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
-      }
+      stage_partial<true, Tile>(lds, a, a.ctx, H, w.w_o, a.splitk_o, first, stride);
       grid_sync(bar);
-      if constexpr (BIG) big_fc1<true>(lds_raw, a, w, first, stride, &bar);
-      else stage_fc1<true, Tile>(lds, a, w, first, stride);
+      stage_ln<true>(a, a.splitk_o, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1, first * 4 + wave, stride * 4);
       grid_sync(bar);
-      if constexpr (BIG) {
-        big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, first, stride);
-        rowblock_ln<true, kFc2Split>(a, 2u * l + 2u, fc2_sums(a), a.y1, w.ln2_g, w.ln2_b, yout, first, stride, &bar);
-      } else {
-        stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
-        grid_sync(bar);
-        stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
-      }
+      stage_fc1<true, Tile>(lds, a, w, first, stride);
+      grid_sync(bar);
+      stage_partial<true, Tile>(lds, a, a.h, F, w.w_fc2, a.splitk_f, first, stride);
+      grid_sync(bar);
+      stage_ln<true>(a, a.splitk_f, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout, first * 4 + wave, stride * 4);
     } else {
       // Weight slices are queued one stage ahead, from inside the grid barrier that precedes
       // the stage.
@@ -1304,8 +1362,7 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
     }
     qkv_ready = false;
     if (l + 1 < a.num_layers) {
-      if constexpr (BIG)   // the next layers write this layer's buffers again: see Params
-        grid_sync(bar, [&]() { if (threadIdx.x < 64) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); });
+      if constexpr (BIG) {}          // (done above)
       else if constexpr (LARGE) grid_sync(bar);
       else grid_sync(bar, [&]() { qkv_ready = preissue_w<OsFull>(lds_raw, QkvItems{args.layers[l + 1].w_qkv, a.M}); });
     }
