@@ -41,10 +41,11 @@ struct LayerW {
 // an activation once instead of every workgroup fetching it from memory.
 // The many-rows megakernel (82 MB of such buffers per layer at 4096 rows) rotates through
 // `layer_sets` sets instead, which stay in the memory-side cache, and restores the property at
-// the barrier that ends a layer: one wave of every workgroup invalidates its L1 and its XCD's L2
-// (an agent-scope acquire fence) after arriving and before it polls, so the invalidation has been
-// performed when the poll returns.  In the last stage of a layer nobody reads a buffer that a later
-// layer writes before reading, so no line dropped there can come back in an old version.
+// the hand-over (or barrier) that ends a layer: one wave of every workgroup invalidates its L1 and its
+// XCD's L2 (an agent-scope acquire fence) after arriving and before it polls, so the invalidation has
+// been performed when the poll returns.  In the last stage of a layer nobody reads a buffer that a later
+// layer writes before reading, so no line dropped there can come back in an old version; with
+// hand-overs per row block the same holds per row block, whose rows only its own workgroups read.
 struct Params {
   int B, S, M, act, num_layers, splitk_o, splitk_f;
   int big;             // rows are a multiple of 256 and many: the 256-row GEMM tiles are used
