@@ -125,6 +125,30 @@ def test_many_rows_encoder_reuses_its_buffers(B, S, layers):
     assert_close("encoder many rows", y_a, oracle.bert_encoder(x0, ws, B, S))
 
 
+def test_many_rows_encoder_in_a_workspace_of_unknown_content():
+    """The many-rows path clears its own hand-over words and writes every buffer before it reads it: a
+    workspace that held arbitrary bytes and was initialised again gives the same result, and so does one
+    that other shapes of the encoder have used in between."""
+    announce("bert encoder many rows, dirtied workspace")
+    import bert_binding
+    import souffle_hip as sh
+    B, S, layers = 16, 128, 3
+    ws = [synth.bert_layer_weights(2, l) for l in range(layers)]
+    x = dev(synth.bert_input(4, B, S))
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    y_u = enc(x, fused=False).clone()
+    enc.ws.buf.fill_(-1)
+    sh.check(sh.lib().souffle_workspace_init(enc.ws.ptr, enc.ws.nbytes, sh.current_stream()))
+    y_a = enc(x).clone()
+    small = bert_binding.Encoder([dev_weights(w) for w in ws[:1]], 1, 128)
+    small.ws = enc.ws                                    # another shape of the encoder in the same memory
+    small(dev(synth.bert_input(4, 1, 128)))
+    y_b = enc(x).clone()
+    torch.cuda.synchronize()
+    assert enc.ws.status() == 0
+    assert torch.equal(y_a, y_u) and torch.equal(y_b, y_u)
+
+
 @pytest.mark.parametrize("B,S,layers", [(1, 128, 12), (1, 384, 2), (2, 64, 3), (1, 128, 1)])
 def test_dataflow_sync_equals_barrier_sync(B, S, layers):
     """The dataflow hand-over (consumers poll the data) runs the same arithmetic as the grid-barrier
