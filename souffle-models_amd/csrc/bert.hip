@@ -536,8 +536,9 @@ static_assert(H / BigOut::kBN == 16 && kFc2Split * (H / BigFc2::kBN) == 16, "16 
 // row block this workgroup has a tile in have reached `tag`.  Bounded like the grid barrier; a wait that
 // gave up ends all waiting of the launch.  With `bar.trace` the entry and exit times are stamped like
 // those of a grid barrier.
+// `group`: row blocks that hand over together (1, or the 2 or 3 that hold whole sequences of 512 or 384).
 template <class Mid>
-__device__ __forceinline__ void rowblock_sync(const Params &a, GridBarrier &bar, unsigned tag, int first, int stride, Mid mid) {
+__device__ __forceinline__ void rowblock_sync(const Params &a, GridBarrier &bar, unsigned tag, int first, int stride, int group, Mid mid) {
   const int m_tiles = a.M / 256;
   const bool tr = bar.trace && bar.trace_idx < bar.trace_cap && threadIdx.x == 0;
   if (tr) bar.trace[(size_t)(2 * bar.trace_idx) * bar.nblk + blockIdx.x] = wall_clock64();
@@ -554,10 +555,11 @@ __device__ __forceinline__ void rowblock_sync(const Params &a, GridBarrier &bar,
     for (int it = first; it < m_tiles * 16 && !bar.failed; it += stride) {
       int tm, tn;
       big_tile(it, m_tiles, 16, &tm, &tn);
+      const int g0 = tm - tm % group;
       for (int spin = 0; spin < kMaxBarrierSpin; ++spin) {
         bool ok = true;
-        if (threadIdx.x < 16)
-          ok = (int)(__hip_atomic_load(a.rbflags + tm * 16 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - tag) >= 0;
+        if (threadIdx.x < 16 * group)
+          ok = (int)(__hip_atomic_load(a.rbflags + g0 * 16 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - tag) >= 0;
         if (__all(ok)) break;
         __builtin_amdgcn_s_sleep(1);
         if (spin == kMaxBarrierSpin - 1) {         // gave up: the launch's output is invalid
@@ -575,7 +577,7 @@ template <bool COH, int NZ>
 __device__ __forceinline__ void rowblock_ln(const Params &a, GridBarrier &bar, unsigned tag, const half_t *z, const half_t *resid, const half_t *gam,
                                             const half_t *bet, half_t *out, int first, int stride) {
   const int m_tiles = a.M / 256, wave = threadIdx.x >> 6;
-  rowblock_sync(a, bar, tag, first, stride, []() {});
+  rowblock_sync(a, bar, tag, first, stride, 1, []() {});
   for (int it = first; it < m_tiles * 16; it += stride) {
     int tm, tn;
     big_tile(it, m_tiles, 16, &tm, &tn);
@@ -1229,15 +1231,15 @@ __device__ __forceinline__ void stage_attn_t(half_t *lds, const Params &a, int f
   else
     for (int it = first; it < items; it += stride) attn_item<COH, NKT>(lds, a, attn_item_of(it, a.S / 64, items));
 }
-// The attention items of the sequences of a 256-row block (48 of them whatever S <= 256 is), three to
-// each of the block's 16 tiles, for the tiles of this workgroup.
+// The attention items of the sequences of a group of 256-row blocks that holds whole sequences (48 items
+// per row block whatever S is), three to each of the group's tiles, for the tiles of this workgroup.
 template <bool COH, int NKT>
 __device__ __forceinline__ void stage_attn_rowblock(unsigned char *lds, const Params &a, int first, int stride) {
   const int m_tiles = a.M / 256;
   for (int it = first; it < m_tiles * 16; it += stride) {
     int tm, tn;
     big_tile(it, m_tiles, 16, &tm, &tn);
-    const int base = tm * 48 + tn * 3;
+    const int base = tm * 48 + tn * 3;           // (the tiles of a group are numbered through: 16 tm + tn)
     if constexpr (2 * kAttnItemLds<NKT> <= kBigLds)
       attn_items_pipelined<COH, NKT>(lds, a, 0, 1, 3, [&](int j) { return base + j; });
     else
@@ -1295,16 +1297,17 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
     const Params a = layer_params(args, l);
     half_t *yout = (l == a.num_layers - 1) ? a.y : a.yl;
     if constexpr (BIG) {
-      // Where a 256-row block holds whole sequences, every stage of a row block's tiles reads only what
-      // the 16 tiles of the same row block wrote in the stage before (attention included: the 48 items
-      // of the block's sequences go three to a tile), and the tile-to-workgroup mapping is the same in
-      // every stage: the 16 row blocks of M = 4096 then run as independent groups of 16 workgroups that
-      // hand over among themselves (rowblock_sync) and drift apart, so that the loads of one group
-      // overlap the MFMAs and the stores of others.  Otherwise (S = 384, 512) the stages are separated
-      // by grid barriers.  Hand-over k of layer l carries the tag 7 l + k.
-      const bool local = kRowblockLocal && 256 % a.S == 0;
+      // Where a 256-row block (S = 64, 128, 256) or a group of 2 (S = 512) or 3 (S = 384) of them holds
+      // whole sequences, every stage of a group's tiles reads only what the tiles of the same group
+      // wrote in the stage before (attention included: the 48 items per row block go three to a tile),
+      // and the tile-to-workgroup mapping is the same in every stage: the 16 row blocks of M = 4096 then
+      // run as independent groups of 16 workgroups that hand over among themselves (rowblock_sync).
+      // Otherwise (a number of row blocks that is no multiple of the group) the stages are separated by
+      // grid barriers.  Hand-over k of layer l carries the tag 7 l + k.
+      const int group = a.S <= 256 ? 1 : a.S == 512 ? 2 : 3;
+      const bool local = kRowblockLocal && (group * 256) % a.S == 0 && (a.M / 256) % group == 0;
       auto sync = [&](unsigned k) {
-        if (local) rowblock_sync(a, bar, 7u * l + k, first, stride, []() {});
+        if (local) rowblock_sync(a, bar, 7u * l + k, first, stride, group, []() {});
         else grid_sync(bar);
       };
       big_qkv<true>(lds_raw, a, w, xin, first, stride, &bar);
@@ -1321,7 +1324,7 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       rowblock_ln<true, kFc2Split>(a, bar, 7u * l + 6u, fc2_sums(a), a.y1, w.ln2_g, w.ln2_b, yout, first, stride);
       if (l + 1 < a.num_layers) {   // the next layer writes this layer's buffers again: see Params
         auto invalidate = [&]() { if (threadIdx.x < 64) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); };
-        if (local) rowblock_sync(a, bar, 7u * l + 7u, first, stride, invalidate);
+        if (local) rowblock_sync(a, bar, 7u * l + 7u, first, stride, group, invalidate);
         else grid_sync(bar, invalidate);
       }
     } else if constexpr (LARGE) {

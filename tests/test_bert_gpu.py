@@ -102,7 +102,7 @@ def test_encoder_matches_oracle(B, S, layers):
     assert torch.equal(y_f, y_u)
 
 
-@pytest.mark.parametrize("B,S,layers", [(32, 128, 5), (16, 128, 4), (64, 128, 3), (8, 384, 3), (8, 256, 3), (32, 64, 3)])
+@pytest.mark.parametrize("B,S,layers", [(32, 128, 5), (16, 128, 4), (64, 128, 3), (8, 384, 3), (8, 256, 3), (32, 64, 3), (4, 512, 2), (6, 384, 2)])
 def test_many_rows_encoder_reuses_its_buffers(B, S, layers):
     """At many rows all layers of the fused launch share one set of inter-stage buffers (kept coherent
     by a cache invalidation at the barrier that ends a layer) and the LayerNorms are handed over per
