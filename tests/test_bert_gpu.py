@@ -125,6 +125,25 @@ def test_many_rows_encoder_reuses_its_buffers(B, S, layers):
     assert_close("encoder many rows", y_a, oracle.bert_encoder(x0, ws, B, S))
 
 
+def test_many_rows_encoder_large_batch_fused_equals_per_op():
+    """16384 rows (four tiles per workgroup and stage): too large for the oracle in a test, so the check is
+    the size-independent one: the fused launch and the per-op chain, which synchronise in different ways
+    (hand-overs per row block against kernel boundaries), agree bit for bit, twice."""
+    announce("bert encoder B=128 S=128 L=2 fused vs per-op")
+    import bert_binding
+    B, S, layers = 128, 128, 2
+    ws = [synth.bert_layer_weights(2, l) for l in range(layers)]
+    x = dev(synth.bert_input(6, B, S))
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    y_u = enc(x, fused=False).clone()
+    y_a = enc(x).clone()
+    y_b = enc(x).clone()
+    torch.cuda.synchronize()
+    assert enc.ws.status() == 0
+    assert torch.isfinite(y_a.float()).all()
+    assert torch.equal(y_a, y_u) and torch.equal(y_b, y_u)
+
+
 def test_many_rows_encoder_in_a_workspace_of_unknown_content():
     """The many-rows path clears its own hand-over words and writes every buffer before it reads it: a
     workspace that held arbitrary bytes and was initialised again gives the same result, and so does one
