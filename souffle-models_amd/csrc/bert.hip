@@ -219,8 +219,13 @@ __device__ __forceinline__ void stage_fc1(half_t *lds, const Params &a, const La
         const h4 bb = ldg<h4>(w.b_fc1 + n);
         v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
       }
+      if (a.act == SOUFFLE_ACT_RELU) {            // (one test per group of results, not one per result)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(v[i], 0.f) : gelu_tanh(v[i]);
+        for (int i = 0; i < 4; ++i) v[i] = fmaxf(v[i], 0.f);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = gelu_tanh(v[i]);
+      }
       st8<COH>(a.h, (m * F + n) * 2, pack_h4(v));
     };
     Tile::run(lds, w.w_fc1, F, tm * BM, n0, 0, H / BK, aload, epi);
@@ -835,10 +840,12 @@ __device__ __forceinline__ void small_fc1(unsigned char *lds, const Params &a, c
     [&](const Item &d) { ln_rows_in_lds<COH>(lds, w.ln1_g != nullptr, w.ln1_b != nullptr, a.eps, d.n0 == 0 ? a.y1 : nullptr, d.m0); },
     [&](const Item &, int m, int n, f4 lo, f4 hi) {
       add_bias8(lo, hi, w.b_fc1, n);
+      if (a.act == SOUFFLE_ACT_RELU) {            // (one test per group of results, not one per result)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        lo[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(lo[i], 0.f) : gelu_tanh(lo[i]);
-        hi[i] = a.act == SOUFFLE_ACT_RELU ? fmaxf(hi[i], 0.f) : gelu_tanh(hi[i]);
+        for (int i = 0; i < 4; ++i) { lo[i] = fmaxf(lo[i], 0.f); hi[i] = fmaxf(hi[i], 0.f); }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { lo[i] = gelu_tanh(lo[i]); hi[i] = gelu_tanh(hi[i]); }
       }
       st16<COH>(a.h, (m * F + n) * 2, pack_h8(lo, hi));
     }, tb, fl);
