@@ -337,9 +337,12 @@ __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, 
 // uses 96 columns and two halves of K, which asks the L2 for 0.6x the operand bytes of 48-column
 // tiles over the whole K (a CU takes in operands no faster than it multiplies them): 41 -> 31 us.
 // (The same split for the out-projection, K = 768, gains nothing: its tiles are too short.)
-using BigQkv = GemmBig<144, 5>;
-using BigFc1 = GemmBig<192, 5>;
-using BigOut = GemmBig<48, 5>;
+// (a ring of four stages: three in flight at the start of a tile cost 1.7 us to queue, four 2.3 us, and the
+// loop is no slower: 12 layers at M = 4096 1378 -> 1368 us fused, 1443 -> 1404 us as separate launches)
+constexpr int kBigRing = 4;
+using BigQkv = GemmBig<144, kBigRing>;
+using BigFc1 = GemmBig<192, kBigRing>;
+using BigOut = GemmBig<48, kBigRing>;
 // FC2: parts of K, each a partial sum of its own.  16 tiles per row block: 4 column tiles of 192 x 4 parts of K
 // (the operand reuse of the FC1 tile; 8 column tiles of 96 x 2 parts writes and reads back half the partial
 // sums but runs its K loop at a worse ratio of operand bytes to MFMAs: 1434 us against 1417 for the 12
@@ -348,7 +351,7 @@ using BigOut = GemmBig<48, 5>;
 #define SOUFFLE_FC2_SPLIT 4
 #endif
 constexpr int kFc2Split = SOUFFLE_FC2_SPLIT;
-using BigFc2 = GemmBig<H * kFc2Split / 16, 5>;
+using BigFc2 = GemmBig<H * kFc2Split / 16, kBigRing>;
 constexpr int kBigLds = BigFc1::LDS_BYTES;
 static_assert(BigQkv::LDS_BYTES <= kBigLds && BigOut::LDS_BYTES <= kBigLds && BigFc2::LDS_BYTES <= kBigLds, "FC1 has the largest ring");
 
