@@ -529,14 +529,11 @@ __device__ __forceinline__ void big_ln(const Params &a, const half_t *z, const h
 }
 
 // The LayerNorm that follows a pre-LayerNorm sum, without a grid barrier in between (rowblock_ln).  A 256-row
-// block of the sum is produced by 16 tiles (16 column tiles, or 8 column tiles x 2 halves of K).
-// A workgroup first finishes ALL its tiles of the stage, then publishes `tag` in the word of each
-// (row block, tile), then, per tile, waits for the 16 words of that row block and normalises 16
-// of its rows (tile t: rows 16t .. 16t+15, four per wave).  Nobody waits before all its own tiles
-// are published, so the waits end whatever the tile-to-workgroup mapping is; they are bounded all
-// the same.  The words are cleared by the launch itself before its first grid barrier and tags grow
-// within a launch.  Rows are normalised by the same routine as in the separate LayerNorm stage:
-// identical results.
+// block of the sum is produced by 16 tiles (16 column tiles, or 4 column tiles x 4 parts of K).
+// After the hand-over among them (rowblock_sync) tile t normalises rows 16t .. 16t+15 of the block,
+// four per wave, by the same routine as the separate LayerNorm kernel: identical results.  The
+// hand-over words are cleared by the launch itself (one grid barrier follows) and tags grow within a
+// launch.
 static_assert(H / BigOut::kBN == 16 && kFc2Split * (H / BigFc2::kBN) == 16, "16 tiles per row block");
 // Hand-over among the workgroups of a 256-row block: this workgroup's tiles of the stage are written
 // (all of them: nobody waits before that, so the waits end whatever the tile-to-workgroup mapping is):
