@@ -42,7 +42,7 @@ def test_bert_validation_without_gpu():
     big = sh.BertCfg(32, 128, 768, 12, 3072, 0, 0.125, 1e-12, 12, 0)
     n32 = lib.souffle_bert_workspace_bytes(C.byref(big))
     assert 0 < n1 < n32 < (1 << 30)
-    # few rows: one set of inter-stage buffers per layer; from 2048 rows (a multiple of 256) up: one set
+    # few rows: one set of inter-stage buffers per layer; from 1024 rows (a multiple of 256) up: one set
     # for all layers (plus 16 hand-over words per 256-row block), so the size no longer grows with depth
     bytes_for = lambda b, s, layers: lib.souffle_bert_workspace_bytes(C.byref(sh.BertCfg(b, s, 768, 12, 3072, 0, 0.125, 1e-12, layers, 0)))
     assert bytes_for(1, 128, 12) > 11 * (bytes_for(1, 128, 1) - 4096)

@@ -85,7 +85,7 @@ def test_fast_path_equals_dump_path_and_is_deterministic():
     assert torch.equal(a, c), "fused and per-op paths run the same arithmetic"
 
 
-@pytest.mark.parametrize("B,S,layers", [(1, 128, 12), (1, 384, 3), (32, 128, 2)])
+@pytest.mark.parametrize("B,S,layers", [(1, 128, 12), (1, 384, 3), (32, 128, 2), (9, 128, 2), (8, 128, 2), (3, 384, 2)])
 def test_encoder_matches_oracle(B, S, layers):
     announce("bert encoder B=%d S=%d L=%d" % (B, S, layers))
     import bert_binding
