@@ -332,6 +332,10 @@ __device__ __forceinline__ void grid_barrier_end(GridBarrier &b) {
   if (b.count > 0 && blockIdx.x < 8 && threadIdx.x == 0) {
     __hip_atomic_store(b.ctl + 384 + blockIdx.x, b.target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (blockIdx.x == 0) __hip_atomic_store(b.ctl + 392, b.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // The next launch on this control block reads these words first thing.  The wave does not end
+    // before they are acknowledged, so that their arrival does not rest on what the end of a kernel
+    // waits for when the runtime queues two launches without a cache release in between.
+    __builtin_amdgcn_s_waitcnt(0);
   }
 }
 

@@ -9,14 +9,26 @@
 // LDS layouts (16-byte slots; a direct load writes 64 consecutive slots, which global 16 bytes
 // each lane fetches is free, so swizzles cost nothing):
 //   X stage [256 rows][32 k]: slot(r, s) = 4r + (s ^ ((r >> 1) & 3)); an operand read of 16 rows is
-//            one contiguous KB and its 8-lane groups cover all 32 banks;
-//   W stage [32 k][BN]:       slot(k, c) = k*BN/8 + (c ^ swz(k)); the four rows a 16-lane group of
-//            the transposing read touches must fall into different banks: their distance is
-//            BN/2 banks, i.e. 8 (BN = 144), 24 (BN = 48) - fine as they are - or 0 (BN = 192),
-//            where swz(k) = 2(k & 3) moves them apart, or 16 (BN = 96), where swz(k) = k & 2 does.
+//            one contiguous KB and free of bank conflicts as measured (SQ_LDS_BANK_CONFLICT; a
+//            swizzle that also involves bit 3 of r costs one conflict cycle per read cycle);
+//   W stage [32 k][BN]:       row k is stored as LDS row wrow_of(k) (bits 2 and 3 of k swapped), slot(k, c)
+//            = wrow_of(k)*BN/8 + (c ^ wswz(wrow_of(k))).  The LDS has 64 banks of 4 bytes and serves
+//            the transposing read half a wave per cycle.  Half a wave touches 32 bytes of each of the
+//            rows k0..k0+3 and k0+8..k0+11, i.e. LDS rows rho0..rho0+7, which must cover the 64 banks
+//            once: consecutive LDS rows are 2 (BN = 144) or 6 (BN = 48) 16-byte slots apart modulo 16
+//            - eight of them cover everything - or 8 (BN = 192) or 12 (BN = 96), where wswz moves the
+//            rows that would coincide apart.  (Measured with SQ_LDS_BANK_CONFLICT: rows k0..k0+3 spread
+//            over 32 banks only, as a 32-bank LDS would want it, cost as many conflict cycles as the
+//            reads themselves, 192 per K step of a 192-column tile; what is left are the 48 per step
+//            of the epilogue's stores.)
 // W is row-major [K][N] as the reference stores it (cpp/bert/kernels/gemm_three_stages.h:95-131);
 // the MFMA takes W as operand A and X as operand B, so a lane ends up with 4 consecutive output
 // columns of one row.
+// Tried and dropped: X straight from global memory into registers (a wave's 64 rows are its own, and
+// a lane's 16 operand bytes are contiguous in the row-major X), which takes X out of LDS altogether.
+// Same results, 2 % slower (12 layers at M = 4096: 1421 us against 1393): a K step without any X
+// traffic is 16-18 % shorter, so the step is bound by the number of wave-wide loads the CU's load
+// unit takes, and a load that returns to registers costs it no less than one that lands in LDS.
 #pragma once
 #include <type_traits>
 #include "common.hpp"
@@ -56,7 +68,8 @@ struct GemmBig {
   typedef __attribute__((address_space(1))) const void *gptr_t;
   typedef __attribute__((address_space(3))) void *lptr_t;
 
-  __device__ static __forceinline__ int wswz(int k) { return BN == 192 ? ((k & 3) << 1) : (BN == 96 ? (k & 2) : 0); }
+  __device__ static __forceinline__ int wrow_of(int k) { return (k & 0x13) | ((k & 4) << 1) | ((k & 8) >> 1); }   // (its own inverse)
+  __device__ static __forceinline__ int wswz(int rho) { return BN == 192 ? (((rho >> 1) & 3) << 1) : (BN == 96 ? ((rho >> 1) & 2) : 0); }
 
   // Load number L (0 .. LPW-1) of this wave for the stage at LDS address `stage`, K offset kk.
   // wptr(k, col) -> address of W[k][col] (col relative to the tile's first column, multiple of 8)
@@ -67,8 +80,8 @@ struct GemmBig {
       const int q = wave + 4 * L, r = q * 16 + (lane >> 2), sl = (lane & 3) ^ ((r >> 1) & 3);
       load_lds16(X + (size_t)(m0 + r) * ldx + kk + sl * 8, stage + q * 1024);
     } else {
-      const int q = (wave + 4 * (L - 4)) % WI, sl = q * 64 + lane, k = sl / WSLOTS, c = (sl % WSLOTS) ^ wswz(k);
-      load_lds16(wptr(kk + k, c * 8), stage + X_STAGE + q * 1024);
+      const int q = (wave + 4 * (L - 4)) % WI, sl = q * 64 + lane, rho = sl / WSLOTS, c = (sl % WSLOTS) ^ wswz(rho);
+      load_lds16(wptr(kk + wrow_of(rho), c * 8), stage + X_STAGE + q * 1024);
     }
   }
   template <int L0, int L1, class WPtr>
@@ -142,12 +155,12 @@ struct GemmBig {
       const int r = wave * 64 + i * 16 + l16;
       xoff[i] = r * 64 + ((g ^ ((r >> 1) & 3)) << 4);
     }
-    const int kr = g * 8 + (l16 >> 2);                       // first of this lane's two k rows (kr, kr + 4)
-    const int wrow = X_STAGE + kr * (BN * 2) + (l16 & 1) * 8, wsw = wswz(kr), wc = (l16 & 3) >> 1;
+    const int rho = wrow_of(g * 8 + (l16 >> 2));             // LDS row of the first of this lane's two k rows (k, k + 4: LDS rows rho, rho + 8)
+    const int wrow = X_STAGE + rho * (BN * 2) + (l16 & 1) * 8, wsw = wswz(rho), wc = (l16 & 3) >> 1;
 
     auto read_w = [&](const unsigned char *st, int j) {
       const half_t *p = reinterpret_cast<const half_t *>(st + wrow + (((j * 2 + wc) ^ wsw) << 4));
-      const h4 lo = lds_read_tr16(p), hh = lds_read_tr16(p + 4 * BN);
+      const h4 lo = lds_read_tr16(p), hh = lds_read_tr16(p + 8 * BN);
       return h8{lo[0], lo[1], lo[2], lo[3], hh[0], hh[1], hh[2], hh[3]};
     };
 
