@@ -77,20 +77,26 @@ __device__ __forceinline__ Chunk chunk_of(const BlockW &w, int c) {
 }
 
 // The weight stream of one workgroup.  `issued` / `used` count chunks over the whole launch.
+// Slot swizzles of the weight chunks in LDS (64 banks of 4 bytes; the transposing read is served half a
+// wave per cycle: 32 bytes of each of the rows k0..k0+3 and k0+8..k0+11, which must not share banks).
+// 128-byte rows: rows of equal parity start in the same bank, bits 1 and 3 of k separate the four of them.
+// 64-byte rows: rows k and k+8 start in the same bank, bit 3 separates them (bit 1 is harmless).
+__device__ __forceinline__ int wswz8(int k) { return (k & 2) | ((k & 8) >> 1); }
+__device__ __forceinline__ int wswz4(int k) { return (k & 2) ^ ((k & 8) >> 2); }
 struct WeightRing {
   unsigned char *lds;
   unsigned lds_addr;
   int issued, used;
 };
 // Queue chunk c of block weights w into the next ring buffer.  Layout as GemmOneShot's W slice:
-// slot(k, c8) = 8 k + (c8 ^ (k & 2)), for the transposing operand read.
+// slot(k, c8) = 8 k + (c8 ^ wswz8(k)), for the transposing operand read.
 __device__ __forceinline__ void ring_issue(WeightRing &r, const BlockW &w, int c) {
   const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6;
   const Chunk ch = chunk_of(w, c);
   const unsigned base = r.lds_addr + (r.issued % RING) * CHUNK_BYTES;
 #pragma unroll
   for (int q = 0; q < CHUNK_LOADS; ++q) {
-    const int inst = q * 4 + wave, sl = inst * 64 + lane, k = sl >> 3, c8 = (sl & 7) ^ (k & 2);
+    const int inst = q * 4 + wave, sl = inst * 64 + lane, k = sl >> 3, c8 = (sl & 7) ^ wswz8(k);
     load_lds16(ch.W + (size_t)(ch.k0 + k) * ch.ldw + ch.n0 + c8 * 8, base + inst * 1024);
   }
   r.issued++;
@@ -123,7 +129,7 @@ __device__ __forceinline__ void chunk_mma(const unsigned char *buf, const half_t
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int c8 = j * 2 + ((l16 & 3) >> 1);
-      const half_t *p = ws + (k * 8 + (c8 ^ (k & 2))) * 8 + (l16 & 1) * 4;
+      const half_t *p = ws + (k * 8 + (c8 ^ wswz8(k))) * 8 + (l16 & 1) * 4;
       const h4 lo = lds_read_tr16(p), hi = lds_read_tr16(p + 4 * CHUNK_N);
       wop[ks][j] = h8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
@@ -441,14 +447,14 @@ __device__ __forceinline__ Chunk qchunk_of(const BlockW &w, int c, int h) {
   if (c < 11) return Chunk{w.w_fc1, F, 0, h * (F / NH) + (c - 7) * QN};
   return Chunk{w.w_fc2, C, h * (F / NH), (c - 11) * QN};
 }
-// W[128 k][32 n] chunk: slot(k, c4) = 4 k + (c4 ^ (k & 2)) (16-byte slots), for the transposing read.
+// W[128 k][32 n] chunk: slot(k, c4) = 4 k + (c4 ^ wswz4(k)) (16-byte slots), for the transposing read.
 __device__ __forceinline__ void qring_issue(WeightRing &r, const BlockW &w, int c, int h) {
   const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6;
   const Chunk ch = qchunk_of(w, c, h);
   const unsigned base = r.lds_addr + (r.issued % RING) * QCHUNK_BYTES;
 #pragma unroll
   for (int q = 0; q < QLOADS; ++q) {
-    const int inst = q * 4 + wave, sl = inst * 64 + lane, k = sl >> 2, c4 = (sl & 3) ^ (k & 2);
+    const int inst = q * 4 + wave, sl = inst * 64 + lane, k = sl >> 2, c4 = (sl & 3) ^ wswz4(k);
     load_lds16(ch.W + (size_t)(ch.k0 + k) * ch.ldw + ch.n0 + c4 * 8, base + inst * 1024);
   }
   r.issued++;
@@ -476,7 +482,7 @@ __device__ __forceinline__ void qchunk_mma(const unsigned char *buf, const half_
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int c4 = j * 2 + ((l16 & 3) >> 1);
-      const half_t *p = ws + (k * 4 + (c4 ^ (k & 2))) * 8 + (l16 & 1) * 4;
+      const half_t *p = ws + (k * 4 + (c4 ^ wswz4(k))) * 8 + (l16 & 1) * 4;
       const h4 lo = lds_read_tr16(p), hi = lds_read_tr16(p + 4 * QN);
       wop[ks][j] = h8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
