@@ -199,7 +199,7 @@ SYNC_DATAFLOW, SYNC_BARRIER = 0, 1
 
 
 def set_bert_sync(mode):
-    """Hand-over between the stages of the skinny fused encoder: "dataflow" (default) or "barrier"."""
+    """Hand-over between the stages of the skinny fused encoder: "barrier" (default) or "dataflow"."""
     modes = {"dataflow": SYNC_DATAFLOW, "barrier": SYNC_BARRIER, SYNC_DATAFLOW: SYNC_DATAFLOW, SYNC_BARRIER: SYNC_BARRIER}
     check(lib().souffle_set_bert_sync(modes[mode]))
 
