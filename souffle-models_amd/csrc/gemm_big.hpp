@@ -29,6 +29,10 @@
 // Same results, 2 % slower (12 layers at M = 4096: 1421 us against 1393): a K step without any X
 // traffic is 16-18 % shorter, so the step is bound by the number of wave-wide loads the CU's load
 // unit takes, and a load that returns to registers costs it no less than one that lands in LDS.
+// Also dropped: X staged two K steps at a time ([256][64 k] stages, a ring of three, so that a wave-wide
+// load takes 8 rows x 128 bytes, whole cache lines, instead of 16 rows x 64 bytes; alone in a kernel the
+// former costs a CU 51 cycles per KB, the latter 60).  Same results, 2 % slower (1421 us against 1393 on
+// one box).
 #pragma once
 #include <type_traits>
 #include "common.hpp"
