@@ -254,18 +254,6 @@ def test_encoder_replays_from_a_hip_graph(fused):
     assert enc.ws.status() == 0
 
 
-def test_device_probes_report_plausible_ceilings():
-    """The measurement helpers behind the bench line's measured ceilings and latency floor."""
-    announce("device probes")
-    import souffle_hip as sh
-    copy_gbs, mfma_tflops = sh.measured_ceilings()
-    assert 500 < copy_gbs < 8000 and 200 < mfma_tflops < 2600
-    bar_us, floor_us = sh.stage_floor_us(24)
-    assert 5 < bar_us < floor_us < 400
-    with pytest.raises(sh.SouffleError):
-        sh.check(sh.lib().souffle_stage_floor_probe(None, 0, 10, 0, None))
-
-
 def test_souffle_bert_base_module():
     """The reference's zero-weight 12-layer driver (cpp/bert/bert_base_impl.cu:277-308): returns 0."""
     announce("souffle_bert_base")
