@@ -333,7 +333,7 @@ __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, 
 
 // ---- many rows (M a multiple of 256): 256 x BN tiles, see gemm_big.hpp ----
 // BN is chosen per GEMM so that M = 4096 gives exactly 256 tiles, one per CU: 144 for the
-// 2304 QKV columns, 192 for FC1's 3072, 48 for the 768 of the out-projection; FC2 (K = 3072)
+// 2304 QKV columns, 192 for FC1's 3072, 128-row tiles of 96 columns for the 768 of the out-projection; FC2 (K = 3072)
 // uses 96 columns and two halves of K, which asks the L2 for 0.6x the operand bytes of 48-column
 // tiles over the whole K (a CU takes in operands no faster than it multiplies them): 41 -> 31 us.
 // (The same split for the out-projection, K = 768, gains nothing: its tiles are too short.)
@@ -342,7 +342,7 @@ __device__ __forceinline__ void stage_ln_t(const Params &a, const half_t *bias, 
 constexpr int kBigRing = 4;
 using BigQkv = GemmBig<144, kBigRing>;
 using BigFc1 = GemmBig<192, kBigRing>;
-using BigOut = GemmBig<48, kBigRing>;
+using BigOut = GemmBig<96, kBigRing, 128>;   // (128 x 96: 0.74x the operand bytes of 256 x 48 from the L2)
 // FC2: parts of K, each a partial sum of its own.  16 tiles per row block: 4 column tiles of 192 x 4 parts of K
 // (the operand reuse of the FC1 tile; 8 column tiles of 96 x 2 parts writes and reads back half the partial
 // sums but runs its K loop at a worse ratio of operand bytes to MFMAs: 1434 us against 1417 for the 12
@@ -416,7 +416,7 @@ __device__ __forceinline__ void big_fc1(unsigned char *lds, const Params &a, con
       return pack_h4(v);
     };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.h, (m * F + n0 + nr) * 2, v); };
-    f4 acc[4][BigFc1::NT];
+    f4 acc[BigFc1::MI][BigFc1::NT];
     BigFc1::mainloop(lds, a.y1, H, tm * 256, 0, H / 32, wptr, acc, tb);
     if (a.act == SOUFFLE_ACT_RELU) BigFc1::epilogue(lds, tm * 256, acc, cvt_relu, store16, tb);
     else BigFc1::epilogue(lds, tm * 256, acc, cvt_gelu, store16, tb);
@@ -428,16 +428,18 @@ __device__ __forceinline__ void big_fc1(unsigned char *lds, const Params &a, con
 template <bool COH>
 __device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, const half_t *X, int K, const half_t *W,
                                            const half_t *bias, int first, int stride) {
-  const int m_tiles = a.M / 256, n_tiles = H / BigOut::kBN;
-  for (int it = first; it < m_tiles * n_tiles; it += stride) {
+  // 16 tiles per 256-row block as in the other stages, dealt to the same workgroups: tile tn of row
+  // block tm is rows [128 (tn & 1), +128) of the block and column tile tn >> 1.
+  const int m_tiles = a.M / 256;
+  for (int it = first; it < m_tiles * 16; it += stride) {
     int tm, tn;
-    big_tile(it, m_tiles, n_tiles, &tm, &tn);
-    const int n0 = tn * BigOut::kBN;
+    big_tile(it, m_tiles, 16, &tm, &tn);
+    const int n0 = (tn >> 1) * BigOut::kBN, m0 = tm * 256 + (tn & 1) * BigOut::kBM;
     auto wptr = [&](int k, int col) { return W + (size_t)k * H + n0 + col; };
     const half_t *bz = bias ? bias : g_zero_row;
     auto cvt = [&](int, int nr, f4 v) { return pack_h4(add_row4(v, bz, n0 + nr)); };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.z1, (m * H + n0 + nr) * 2, v); };
-    BigOut::run(lds, X, K, tm * 256, 0, K / 32, wptr, cvt, store16);
+    BigOut::run(lds, X, K, m0, 0, K / 32, wptr, cvt, store16);
   }
 }
 // A pre-LayerNorm sum in kFc2Split parts of K: part 0 = X[:, part 0].W[part 0] + bias, part
@@ -459,7 +461,7 @@ __device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a,
     auto cvt_first = [&](int, int nr, f4 v) { return pack_h4(add_row4(v, bz, n0 + nr)); };
     auto cvt_rest = [&](int, int, f4 v) { return pack_h4(v); };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(zp, (m * H + n0 + nr) * 2, v); };
-    f4 acc[4][BigFc2::NT];
+    f4 acc[BigFc2::MI][BigFc2::NT];
     BigFc2::mainloop(lds, X, K, tm * 256, k0, (K / kFc2Split) / 32, wptr, acc);
     if (ks == 0) BigFc2::epilogue(lds, tm * 256, acc, cvt_first, store16);
     else BigFc2::epilogue(lds, tm * 256, acc, cvt_rest, store16);
@@ -534,7 +536,7 @@ __device__ __forceinline__ void big_ln(const Params &a, const half_t *z, const h
 // four per wave, by the same routine as the separate LayerNorm kernel: identical results.  The
 // hand-over words are cleared by the launch itself (one grid barrier follows) and tags grow within a
 // launch.
-static_assert(H / BigOut::kBN == 16 && kFc2Split * (H / BigFc2::kBN) == 16, "16 tiles per row block");
+static_assert((256 / BigOut::kBM) * (H / BigOut::kBN) == 16 && kFc2Split * (H / BigFc2::kBN) == 16, "16 tiles per row block");
 // Hand-over among the workgroups of a 256-row block: this workgroup's tiles of the stage are written
 // (all of them: nobody waits before that, so the waits end whatever the tile-to-workgroup mapping is):
 // publish `tag` in the word of each (row block, tile), run mid(), then wait until the 16 words of every
@@ -1873,7 +1875,7 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     if (LARGE) hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), 2 * a.S * 128 + 64 * 128, st, a);
     else hipLaunchKernelGGL(k_attn_small, dim3(grid_for((a.B * NH + 7) / 8 * 8 * (a.S / 16))), dim3(256), attn_small_lds_bytes(a.S), st, a);
     if constexpr (MODE == 2) {
-      hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * (H / BigOut::kBN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, w.b_o);
+      hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * 16)), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, w.b_o);
       hipLaunchKernelGGL(k_ln_big<1>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.z1, xin, w.ln1_g, w.ln1_b, a.y1);
     } else if constexpr (LARGE) {
       hipLaunchKernelGGL(k_partial<MODE>, dim3(grid_for((a.M / BM_OUT) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, 1);

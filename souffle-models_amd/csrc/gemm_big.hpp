@@ -49,23 +49,27 @@ __device__ __forceinline__ void static_for(Fn f) {
   }
 }
 
-template <int BN, int NSTAGE>
+// BM = 256 rows per tile, or 128 (wave w then owns rows [32w, 32w+32)): at N = 768 a 128 x 96 tile asks
+// the L2 for (128 + 96) x K x 2 bytes where a 256 x 48 tile of the same area asks for (256 + 48) x K x 2.
+template <int BN, int NSTAGE, int BM = 256>
 struct GemmBig {
+  static_assert(BM == 256 || BM == 128, "four waves of 64 or 32 rows");
   static_assert(BN % 16 == 0 && (BN * 64) % 1024 == 0, "whole MFMA tiles and whole wave-wide loads");
   static_assert(BN == 48 || BN == 96 || BN == 144 || BN == 192, "the W swizzle is worked out for these widths");
-  static constexpr int kBM = 256, kBN = BN, kBK = 32;
+  static constexpr int kBM = BM, kBN = BN, kBK = 32;
+  static constexpr int RW = BM / 4, MI = RW / 16;           // rows / accumulator row tiles per wave
   static constexpr int NT = BN / 16;                        // accumulator tiles per row block
   static constexpr int WSLOTS = BN / 8;                     // 16-byte slots per W row
-  static constexpr int X_STAGE = 256 * 32 * 2, W_STAGE = 32 * BN * 2, STAGE = X_STAGE + W_STAGE;
+  static constexpr int X_STAGE = BM * 32 * 2, W_STAGE = 32 * BN * 2, STAGE = X_STAGE + W_STAGE;
   static constexpr int LDS_BYTES = NSTAGE * STAGE;
   static constexpr int EPITCH = BN * 2 + 16;                // bytes per row of a wave's epilogue slice
-  static_assert(4 * 64 * EPITCH <= LDS_BYTES, "the epilogue slices fit in the ring");
+  static_assert(4 * RW * EPITCH <= LDS_BYTES, "the epilogue slices fit in the ring");
   static constexpr int XI = X_STAGE / 1024, WI = W_STAGE / 1024;   // wave-wide loads per stage
-  // Every wave issues LPW loads per stage: 4 of X and WPW of W.  Where WI is not a multiple of 4
+  // Every wave issues LPW loads per stage: XPW of X and WPW of W.  Where WI is not a multiple of 4
   // some waves fetch a chunk a second time (same bytes to the same place): the loop stays free of
   // wave-dependent branches and every wave can use the same vmcnt.
-  static constexpr int WPW = (WI + 3) / 4, LPW = XI / 4 + WPW;
-  static_assert(XI == 16, "256 rows x 32 k");
+  static constexpr int XPW = XI / 4, WPW = (WI + 3) / 4, LPW = XPW + WPW;
+  static_assert(XI == BM / 16 && XI % 4 == 0, "BM rows x 32 k");
   static_assert(NSTAGE >= 4 && NSTAGE <= 6, "ring depth");
   static_assert((NSTAGE - 2) * LPW < 64, "vmcnt is a 6-bit counter");
 
@@ -80,11 +84,11 @@ struct GemmBig {
   template <int L, class WPtr>
   __device__ static __forceinline__ void issue_one(int tid, unsigned stage, const half_t *X, int ldx, int m0, int kk, WPtr wptr) {
     const int lane = tid & 63, wave = tid >> 6;
-    if constexpr (L < 4) {
+    if constexpr (L < XPW) {
       const int q = wave + 4 * L, r = q * 16 + (lane >> 2), sl = (lane & 3) ^ ((r >> 1) & 3);
       load_lds16(X + (size_t)(m0 + r) * ldx + kk + sl * 8, stage + q * 1024);
     } else {
-      const int q = (wave + 4 * (L - 4)) % WI, sl = q * 64 + lane, rho = sl / WSLOTS, c = (sl % WSLOTS) ^ wswz(rho);
+      const int q = (wave + 4 * (L - XPW)) % WI, sl = q * 64 + lane, rho = sl / WSLOTS, c = (sl % WSLOTS) ^ wswz(rho);
       load_lds16(wptr(kk + wrow_of(rho), c * 8), stage + X_STAGE + q * 1024);
     }
   }
@@ -126,7 +130,7 @@ struct GemmBig {
   template <class WPtr, class Cvt, class Store16>
   __device__ static __forceinline__ void run(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, int nkt, WPtr wptr, Cvt cvt, Store16 store16,
                                              const GridBarrier *tb = nullptr) {
-    f4 acc[4][NT];
+    f4 acc[MI][NT];
     mainloop(lds, X, ldx, m0, k0, nkt, wptr, acc, tb);
     epilogue(lds, m0, acc, cvt, store16, tb);
   }
@@ -136,7 +140,7 @@ struct GemmBig {
   // cvt is not hoisted by the compiler but tested per result, and the tiny basic blocks in between
   // serialise every dependent chain (FC1 with GELU: 12.8 us per tile instead of 5).
   template <class WPtr>
-  __device__ static __forceinline__ void mainloop(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, int nkt, WPtr wptr, f4 (&acc)[4][NT],
+  __device__ static __forceinline__ void mainloop(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, int nkt, WPtr wptr, f4 (&acc)[MI][NT],
                                                   const GridBarrier *tb = nullptr) {
     const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
     STAGE_MARK(tb, 0);
@@ -146,17 +150,17 @@ struct GemmBig {
     for (int s = 0; s < NSTAGE - 1; ++s) issue_range<0, LPW>(tid, ring + s * STAGE, X, ldx, m0, k0 + s * 32, wptr);
     // (the accumulators are cleared while the first stages travel)
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < NT; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) mfma_pin(acc[i], true);
+    for (int i = 0; i < MI; ++i) mfma_pin(acc[i], true);
 
     // byte offsets of this lane's operand reads inside a stage
-    int xoff[4];
+    int xoff[MI];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = wave * 64 + i * 16 + l16;
+    for (int i = 0; i < MI; ++i) {
+      const int r = wave * RW + i * 16 + l16;
       xoff[i] = r * 64 + ((g ^ ((r >> 1) & 3)) << 4);
     }
     const int rho = wrow_of(g * 8 + (l16 >> 2));             // LDS row of the first of this lane's two k rows (k, k + 4: LDS rows rho, rho + 8)
@@ -168,13 +172,13 @@ struct GemmBig {
       return h8{lo[0], lo[1], lo[2], lo[3], hh[0], hh[1], hh[2], hh[3]};
     };
 
-    h8 x[4], xn[4], w[D + 1];
+    h8 x[MI], xn[MI], w[D + 1];
     wait_ahead<NSTAGE - 2>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     STAGE_MARK(tb, 1);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) x[i] = as_h8(lds_load16(lds + xoff[i]));
+    for (int i = 0; i < MI; ++i) x[i] = as_h8(lds_load16(lds + xoff[i]));
 #pragma unroll
     for (int j = 0; j < D; ++j) w[j] = read_w(lds, j);
 
@@ -197,12 +201,12 @@ struct GemmBig {
           __builtin_amdgcn_s_barrier();
           asm volatile("" ::: "memory");
 #pragma unroll
-          for (int i = 0; i < 4; ++i) xn[i] = as_h8(lds_load16(stn + xoff[i]));
+          for (int i = 0; i < MI; ++i) xn[i] = as_h8(lds_load16(stn + xoff[i]));
         }
         // (in the last step these read a stale buffer; the values are never used)
         w[(j + D) % (D + 1)] = j + D < NT ? read_w(st, j + D) : read_w(stn, j + D - NT);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < MI; ++i) {
           mfma_16x16x32_inplace(acc[i][j], w[j % (D + 1)], x[i]);
         }
         // this tile's share of the refill: slot t counts tiles from the barrier
@@ -214,7 +218,7 @@ struct GemmBig {
         }
       });
 #pragma unroll
-      for (int i = 0; i < 4; ++i) x[i] = xn[i];
+      for (int i = 0; i < MI; ++i) x[i] = xn[i];
     };
     using T = std::true_type;
     using F = std::false_type;
@@ -230,12 +234,12 @@ struct GemmBig {
     if constexpr (NSTAGE >= 5) step(main_end + 3, F{}, F{}, std::integral_constant<int, (NSTAGE - 6 > 0 ? NSTAGE - 6 : 0)>{});
     if constexpr (NSTAGE >= 6) step(main_end + 4, F{}, F{}, std::integral_constant<int, 0>{});
 #pragma unroll
-    for (int i = 0; i < 4; ++i) mfma_pin(acc[i], false);
+    for (int i = 0; i < MI; ++i) mfma_pin(acc[i], false);
     STAGE_MARK(tb, 2);
   }
 
   template <class Cvt, class Store16>
-  __device__ static __forceinline__ void epilogue(unsigned char *lds, int m0, f4 (&acc)[4][NT], Cvt cvt, Store16 store16, const GridBarrier *tb = nullptr) {
+  __device__ static __forceinline__ void epilogue(unsigned char *lds, int m0, f4 (&acc)[MI][NT], Cvt cvt, Store16 store16, const GridBarrier *tb = nullptr) {
     const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
     // Epilogue.  A lane holds 4 consecutive columns of 16 rows per accumulator tile; stored
     // directly that would be 8-byte pieces of 32-byte row segments.  The converted tile instead
@@ -244,22 +248,23 @@ struct GemmBig {
     // memory system takes at its own pace, 3 us for the 98 KB of an FC1 tile when every workgroup
     // stores at once) drain while the next group is converted.
     __syncthreads();                                        // every wave has left the ring
-    unsigned char *mine = lds + wave * (64 * EPITCH);
+    unsigned char *mine = lds + wave * (RW * EPITCH);
     constexpr int ECH = (NT % 3 == 0 && BN >= 144) ? 3 : (BN == 96 ? 2 : 1);
     constexpr int TPC = NT / ECH, CPC = TPC * 2;             // accumulator tiles / 16-byte chunks per row and group
     static_for<0, ECH>([&](auto chc) {
       constexpr int ch = decltype(chc)::value;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = ch * TPC; j < (ch + 1) * TPC; ++j)
-          lds_store8(mine + (i * 16 + l16) * EPITCH + (j * 16 + g * 4) * 2, cvt(m0 + wave * 64 + i * 16 + l16, j * 16 + g * 4, acc[i][j]));
+          lds_store8(mine + (i * 16 + l16) * EPITCH + (j * 16 + g * 4) * 2, cvt(m0 + wave * RW + i * 16 + l16, j * 16 + g * 4, acc[i][j]));
       if constexpr (ch == ECH - 1) STAGE_MARK(tb, 3);
+      static_assert((RW * CPC) % 64 == 0, "whole wave-wide stores");
 #pragma unroll
-      for (int t = 0; t < CPC; ++t) {                        // 64 rows x CPC chunks = CPC per lane
+      for (int t = 0; t < RW * CPC / 64; ++t) {              // RW rows x CPC chunks, 64 per pass
         const int c = t * 64 + lane, row = c / CPC, col8 = ch * CPC + c % CPC;
         const u4 v = lds_load16(mine + row * EPITCH + col8 * 16);
-        store16(m0 + wave * 64 + row, col8 * 8, v);
+        store16(m0 + wave * RW + row, col8 * 8, v);
       }
     });
     STAGE_MARK(tb, 4);
