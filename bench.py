@@ -171,6 +171,7 @@ def bench_encoder(args, B, S, L, name):
         copy_gbs, mfma_tflops = sh.measured_ceilings()
         roof["measured_copy_GBps"] = copy_gbs
         roof["measured_mfma_f16_TFLOPs"] = mfma_tflops
+        roof["measured_l2_to_lds_GBps"] = sh.measured_l2_stream_gbs()     # all CUs streaming L2-resident operands
         roof["frac_of_measured"] = ach / (mfma_tflops if mfma_bound else copy_gbs)
         if (B, S) == (1, 384):            # mixed shape: both fractions
             roof["mfma_frac"] = flops / (cold_ev * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS

@@ -62,6 +62,12 @@ int souffle_stage_floor_probe(void *workspace, size_t workspace_bytes, int stage
  * memory traffic) and reports the flops it performs: timed by the caller, it gives the empirical
  * matrix-core ceiling that the published peak is compared with.  `out` takes 2 KiB per CU of results. */
 int souffle_mfma_probe(float *out, size_t out_bytes, int iters, double *flops, souffle_stream_t stream);
+/* Queues a kernel in which every workgroup (one per CU) only streams `src` (device memory, 64 KiB..1 GiB,
+ * 16-byte aligned; a few MiB stay L2-resident) into LDS with wave-wide 16-byte direct loads, `iters` x 8 KiB
+ * per wave, and reports the bytes it moves: timed by the caller, it gives the rate at which the CUs can take
+ * operands from the L2s when they do nothing else (the GEMM tiles take theirs in at a third of it).  Like the probes
+ * above it has no counterpart in the reference (cpp/souffle_utils/cuda_utils.h:102-136 only times kernels). */
+int souffle_l2_stream_probe(const void *src, size_t src_bytes, int iters, double *bytes, souffle_stream_t stream);
 
 /* Zero a workspace, all workspace_bytes of it (stream-ordered fill kernel, no allocation, capturable).
  * Once before the first use, and again after a launch that reported a failed wait.

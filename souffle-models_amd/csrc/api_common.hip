@@ -212,6 +212,43 @@ extern "C" int souffle_mfma_probe(float *out, size_t out_bytes, int iters, doubl
   return SOUFFLE_OK;
 }
 
+// L2-to-LDS streaming rate: every workgroup does nothing but pull an L2-resident region into LDS with
+// wave-wide 16-byte direct loads (1 KB contiguous each, 8 to 12 in flight per wave), the way the GEMM
+// kernels take in their operands.  All workgroups walk the same region from different starting points.
+namespace souffle {
+__global__ void __launch_bounds__(256) k_l2_stream_probe(const unsigned char *src, unsigned span, int iters) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds[65536];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned ring = lds_address(lds);
+  unsigned o = ((blockIdx.x % 16u) * 65536u + wave * 1024u + lane * 16u) % span;   // span is a multiple of 4096
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      load_lds16(src + o, ring + (((it & 1) * 8 + u) * 4096) + wave * 1024);
+      o += 4096u;
+      if (o >= span) o -= span;
+    }
+    wait_vmcnt<4>();
+  }
+  wait_vmcnt<0>();
+}
+}  // namespace souffle
+
+extern "C" int souffle_l2_stream_probe(const void *src, size_t src_bytes, int iters, double *bytes, souffle_stream_t stream) {
+  if (!src) return fail(SOUFFLE_ERR_NULL, "src is NULL");
+  if (!aligned16(src)) return fail(SOUFFLE_ERR_ALIGN, "src must be 16-byte aligned");
+  if (src_bytes < 65536 || src_bytes > ((size_t)1 << 30)) return fail(SOUFFLE_ERR_SHAPE, "src_bytes must be in 64 KiB..1 GiB (got %zu)", src_bytes);
+  if (iters <= 0 || iters > (1 << 20)) return fail(SOUFFLE_ERR_SHAPE, "iters must be in 1..2^20 (got %d)", iters);
+  DeviceFacts df;
+  if (int rc = device_facts(&df)) return rc;
+  const unsigned span = (unsigned)(src_bytes & ~(size_t)4095);
+  const unsigned char *p = static_cast<const unsigned char *>(src);
+  hipLaunchKernelGGL(souffle::k_l2_stream_probe, dim3(df.num_cus), dim3(256), 0, static_cast<hipStream_t>(stream), p, span, iters);
+  SOUFFLE_HIP_TRY(hipGetLastError());
+  if (bytes) *bytes = (double)df.num_cus * 4 * iters * 8 * 1024.0;
+  return SOUFFLE_OK;
+}
+
 // The floor of a chain of dependent grid-wide stages on this device: `n` stages that do nothing but
 // hand a value on.  mode 0: the grid barrier alone.  mode 1: every workgroup writes 16 bytes through,
 // passes the barrier, and reads the 16 bytes another workgroup (on another XCD) wrote; what it reads

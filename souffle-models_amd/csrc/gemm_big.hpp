@@ -24,15 +24,15 @@
 // W is row-major [K][N] as the reference stores it (cpp/bert/kernels/gemm_three_stages.h:95-131);
 // the MFMA takes W as operand A and X as operand B, so a lane ends up with 4 consecutive output
 // columns of one row.
-// Tried and dropped: X straight from global memory into registers (a wave's 64 rows are its own, and
-// a lane's 16 operand bytes are contiguous in the row-major X), which takes X out of LDS altogether.
-// Same results, 2 % slower (12 layers at M = 4096: 1421 us against 1393): a K step without any X
-// traffic is 16-18 % shorter, so the step is bound by the number of wave-wide loads the CU's load
-// unit takes, and a load that returns to registers costs it no less than one that lands in LDS.
-// Also dropped: X staged two K steps at a time ([256][64 k] stages, a ring of three, so that a wave-wide
-// load takes 8 rows x 128 bytes, whole cache lines, instead of 16 rows x 64 bytes; alone in a kernel the
-// former costs a CU 51 cycles per KB, the latter 60).  Same results, 2 % slower (1421 us against 1393 on
-// one box).
+// Tried and dropped, all with the same results: X straight from global memory into registers (a wave's
+// 64 rows are its own, and a lane's 16 operand bytes are contiguous in the row-major X), which takes X
+// out of LDS altogether: 2 % slower (12 layers at M = 4096: 1421 us against 1393).  X staged two K
+// steps at a time ([256][64 k] stages, a ring of three, so that a wave-wide load takes 8 rows x 128
+// bytes, whole cache lines, instead of 16 rows x 64 bytes): 2 % slower.  Eight waves of 32 x BN (two
+// per SIMD): 3 % less per K step in an isolated loop.  A K step without any X traffic is 16-18 %
+// shorter, and the costs of a step add up (MFMAs + X + W) whichever way the operands travel, while the
+// same loads alone in a kernel run three times faster than inside the loop: fewer operand bytes per
+// MAC is what helps (hence BM).
 #pragma once
 #include <type_traits>
 #include "common.hpp"

@@ -78,6 +78,7 @@ SIGNATURES = {
     "souffle_device_info": (C.c_int, [C.POINTER(DevInfo)]),
     "souffle_stage_floor_probe": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]),
     "souffle_mfma_probe": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double), C.c_void_p]),
+    "souffle_l2_stream_probe": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double), C.c_void_p]),
     "souffle_set_stage_trace": (C.c_int, [C.c_void_p, C.c_size_t]),
     "souffle_set_cooperative_launch": (C.c_int, [C.c_int]),
     "souffle_workspace_init": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
@@ -253,6 +254,19 @@ def measured_ceilings(device="cuda:0"):
         check(lib().souffle_mfma_probe(out.data_ptr(), out.numel() * 4, iters, C.byref(flops), current_stream()))
     mn, _ = bench_us(probe, warmup=2, rounds=3, repeat=3)
     return copy_gbs, flops.value / (mn * 1e-6) / 1e12
+
+
+def measured_l2_stream_gbs(region_bytes=1 << 20, device="cuda:0"):
+    """Device-wide rate (GB/s) at which all CUs together stream an L2-resident region into LDS.  Synchronises."""
+    import torch
+    src = torch.ones(region_bytes, dtype=torch.uint8, device=device)
+    moved = C.c_double()
+    iters = 512
+
+    def probe():
+        check(lib().souffle_l2_stream_probe(src.data_ptr(), src.numel(), iters, C.byref(moved), current_stream()))
+    mn, _ = bench_us(probe, warmup=2, rounds=3, repeat=3)
+    return moved.value / (mn * 1e-6) / 1e9
 
 
 def bench_us(launch, warmup=20, rounds=10, repeat=100, stream=None):

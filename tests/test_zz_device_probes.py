@@ -14,6 +14,10 @@ def test_device_probes_report_plausible_ceilings():
     import souffle_hip as sh
     copy_gbs, mfma_tflops = sh.measured_ceilings()
     assert 500 < copy_gbs < 8000 and 200 < mfma_tflops < 2600
+    l2_gbs = sh.measured_l2_stream_gbs()
+    assert 1000 < l2_gbs < 40000
+    with pytest.raises(sh.SouffleError):
+        sh.check(sh.lib().souffle_l2_stream_probe(None, 1 << 20, 10, None, None))
     bar_us, floor_us = sh.stage_floor_us(24)
     assert 5 < bar_us < floor_us < 400
     with pytest.raises(sh.SouffleError):
