@@ -1500,6 +1500,9 @@ __global__ void __launch_bounds__(256) k_encoder_flow(Args args) {
     const unsigned err = __hip_atomic_load(args.ctl + kCtlErrWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __hip_atomic_store(args.ctl + kCtlFlowWord, err ? 0u : args.flow_marker, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  // (the refill is acknowledged before the wave ends: a pattern store still on its way when the next launch
+  // writes the same word would put that word back into the "not written" state for good)
+  __builtin_amdgcn_s_waitcnt(0);
   grid_barrier_end(bar);
 }
 

@@ -123,6 +123,9 @@ __global__ void __launch_bounds__(256) k_lstm(Args a) {
     const int t = i / UNITS_PER_WG, u = g * UNITS_PER_WG + i % UNITS_PER_WG;
     st8_atomic(own + (size_t)t * HID + u, u2{0u, 0u});
   }
+  // (acknowledged before the wave ends: a clearing store that were still on its way when the next
+  // launch publishes into the same slot would wipe that value out)
+  __builtin_amdgcn_s_waitcnt(0);
   grid_barrier_end(bar);
 }
 
