@@ -96,21 +96,11 @@ int souffle_set_cooperative_launch(int on);
 
 /* Reads (and optionally clears) the sticky failure flags of a workspace after waiting for
  * `stream`: 0 = every launch that used it ran to completion; bit 0 = an LSTM wait, bit 1 = a
- * grid barrier, bit 2 = a dataflow wait of the encoder gave up (bounded spins; the output of
+ * grid barrier or a hand-over of the encoder gave up (bounded spins; the output of
  * that launch is invalid).  Replaces the reference's abort on a CUDA error after its blocking
  * cudaDeviceSynchronize (cpp/bert/bert_binding.cu:532, cpp/souffle_utils/cuda_utils.h:10-19).
  * This is the one entry point that synchronises. */
 int souffle_workspace_status(void *workspace, souffle_stream_t stream, unsigned *flags, int clear);
-
-/* How the stages of the fused encoder at batch*seq_len < 1024 hand their results on.
- * SOUFFLE_SYNC_BARRIER (default): a grid barrier after every stage, as the reference's
- * cooperative kernels do (cpp/bert/kernels/fused_sqq_bert.cu:2768,3331,3688 grid.sync()).
- * SOUFFLE_SYNC_DATAFLOW: no barrier between stages; consumers poll the data itself (buffers
- * start in a "not written" bit pattern).  Same arithmetic, same results; on MI355X it measures
- * 7 % slower than the barrier, so it is an option, not the default.  Calls that ask for the
- * per-stage tensors always use barriers.  SOUFFLE_BERT_SYNC=dataflow sets the initial value. */
-enum { SOUFFLE_SYNC_DATAFLOW = 0, SOUFFLE_SYNC_BARRIER = 1 };
-int souffle_set_bert_sync(int mode);
 
 /* ------------------------------------------------------------------ BERT ---- */
 enum { SOUFFLE_ACT_GELU_TANH = 0, SOUFFLE_ACT_RELU = 1 };

@@ -61,16 +61,6 @@ int swin_split_mode() {
   }
   return v;
 }
-static std::atomic<int> g_bert_sync{-1};
-int bert_sync_mode() {
-  int v = g_bert_sync.load();
-  if (v < 0) {
-    const char *e = getenv("SOUFFLE_BERT_SYNC");
-    v = (e && (e[0] == 'd' || e[0] == 'D')) ? SOUFFLE_SYNC_DATAFLOW : SOUFFLE_SYNC_BARRIER;
-    g_bert_sync.store(v);
-  }
-  return v;
-}
 static std::atomic<int> g_cooperative{-1};
 static bool cooperative_mode() {
   int v = g_cooperative.load();
@@ -296,12 +286,6 @@ extern "C" int souffle_set_cooperative_launch(int on) {
 
 extern "C" int souffle_set_swin_split(int on) {
   souffle::g_swin_split.store(on ? 1 : 0);
-  return SOUFFLE_OK;
-}
-
-extern "C" int souffle_set_bert_sync(int mode) {
-  if (mode != SOUFFLE_SYNC_DATAFLOW && mode != SOUFFLE_SYNC_BARRIER) return fail(SOUFFLE_ERR_SHAPE, "unknown synchronisation mode %d", mode);
-  souffle::g_bert_sync.store(mode);
   return SOUFFLE_OK;
 }
 

@@ -1,0 +1,942 @@
+// BERT-base encoder, few rows (batch * seq_len < 1024): the weight-stream-bound shapes.
+//
+// A layer is six phases, each a set of independent items dealt to the workgroups of one persistent launch:
+//   QKV  (m-tile, 64 of the 2304 q/k/v columns)   X = layer input (layer 0) or LN2 of the previous layer's sum
+//   ATT  (head, 16 queries)                       scores, softmax and P.V; keys split over the waves
+//   OUT  (m-tile, 64 of 768 columns)              z1 = ctx.Wo + b + x, fp16, plus row statistics of its 64 columns
+//   FC1  (m-tile, 64 of 3072 columns)             h = act(LN1(z1).W1 + b)
+//   FC2  (m-tile, 64 of 768 columns, K quarter)   fp32 partial sums
+//   RED  (the same item, 8 of its 32 rows)        z2 = sum of the 4 partials + b + LN1(z1), fp16, plus row statistics
+// and after the last layer FIN (m-tile, 64 columns): y = LN2(z2).
+//
+// There is no grid barrier.  A workgroup that has finished its items of a phase waits for the acknowledgement of
+// its write-through stores and publishes the number of that phase in its flag word; a consumer polls the flag
+// words of exactly the workgroups that produce what its items read (9 to 48 of them; which ones follows from the
+// item numbering and is worked out once per launch).  Flag words exist in eight copies, one per XCD, so that a
+// line is polled by the 32 workgroups of one XCD only: measured 1.65 us per hand-over against 2.25 us for the
+// grid barrier with per-XCD counters, 3.8 us with a single copy.
+//
+// Memory model of a hand-over (gfx950, one L2 per XCD, one L1 per CU):
+//   producer: data stores with sc1 (write-through to the memory side, which invalidates the copies other L2s hold),
+//             s_waitcnt vmcnt(0) = all of them are acknowledged, workgroup barrier, then the flag store (sc1);
+//   consumer: flag loads with sc1 until the value is there, workgroup barrier, then data loads with sc1.
+// sc1 loads are served by the L2 when it holds the line (same latency as a plain load) but never by the L1 of the
+// CU, which nothing keeps coherent: in a test of 163840 lines a plain load returned the old value in 85 % of the
+// cases where the CU had read the line before, an sc1 load never, and no L2 ever served an old value, neither to
+// plain nor to sc1 loads, within a launch or across launches.  Every load of data that another workgroup of the
+// launch wrote is therefore an sc1 load here.  The release and acquire fences of the compiler's memory model
+// (buffer_wbl2 sc1 / buffer_inv sc1) are not needed on top of that and were measured at 14 us per hand-over.
+//
+// LayerNorm never runs as a pass of its own: producers publish, per row, mean and sum of squared deviations of
+// the 64 columns they wrote; a consumer combines the twelve partials of a row (exact pairwise update, no
+// cancellation) and normalises the operand registers on their way into the MFMA.
+#pragma once
+#include <type_traits>
+#include "bert_defs.hpp"
+
+namespace souffle {
+namespace bert {
+namespace sk {
+
+enum { PH_QKV = 0, PH_ATT, PH_OUT, PH_FC1, PH_FC2, PH_RED, PH_FIN, PH_SLOTS = 8 };
+
+// ---- LDS map (bytes) ----
+constexpr int kXPart = 12288;                 // per wave: its K quarter of the X tile, 12 operand blocks of 1 KB
+constexpr int kWOff = 4 * kXPart;             // weight slice [768][64] fp16
+constexpr int kWBytes = 768 * 128;
+constexpr int kGamOff = kWOff + kWBytes;      // gamma and beta of the LayerNorm applied on load: 768 B per wave (its K quarter of each)
+constexpr int kBiasOff = kGamOff + 4 * 768;   // bias of the item's 64 columns
+constexpr int kAuxOff = kBiasOff + 512;       // LN GEMMs: the row statistics, one copy per wave (4 x 3 KB);
+constexpr int kStatBytes = 32 * 12 * 8;       // OUT: residual patch (4 KB) + one copy of the statistics
+constexpr int kLdsBytes = kAuxOff + 4 * kStatBytes;
+static_assert(kLdsBytes <= 160 * 1024, "LDS of a CU");
+constexpr int kRedLd = 68;                    // floats per row of a wave's partial tile
+static_assert(32 * kRedLd * 4 <= kXPart, "a wave's partial tile reuses its X part");
+
+// ---- flag words ----
+constexpr int kFlagCopies = 8, kFlagStride = 256;
+constexpr int kFlagBaseWord = kFlagCopies * kFlagStride;       // number the flags of this launch start from
+constexpr int kFlagDoneWord = kFlagBaseWord + 1;               // workgroups of the launch that have ended
+constexpr int kFlagWords = kFlagBaseWord + 64;
+constexpr int kMaxFlagSpin = 1 << 21;                          // about a second of polling
+
+struct Shape {
+  int B, S, M, m_tiles, G;
+};
+
+struct Sync {
+  unsigned *flags;       // kFlagWords words, zeroed with the workspace
+  unsigned *err;         // sticky failure word of the control block
+  unsigned base;         // flag value of (layer l, phase p) = base + 1 + l * PH_SLOTS + p
+  bool failed;
+  unsigned long long *trace;   // optional: entry to / exit from every wait, trace[(2 i + {0,1}) * G + block]
+  int trace_cap, trace_idx;
+};
+
+__device__ __forceinline__ unsigned phase_seq(const Sync &s, int l, int ph) { return s.base + 1u + (unsigned)(l * PH_SLOTS + ph); }
+
+// One wave-wide direct-to-LDS load: lane L's 16 bytes at sbase + voff land at LDS byte lds_addr + 16 L.
+// sbase and lds_addr are wave-uniform.  The wait is the caller's (wait_vmcnt<N>).
+template <bool SC1>
+__device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned lds_addr) {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+  if constexpr (SC1)
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 sc1" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+#pragma clang diagnostic pop
+}
+__device__ __forceinline__ unsigned uni(unsigned v) { return __builtin_amdgcn_readfirstlane(v); }
+// Bit patterns of scalars, passed by value.  (__builtin_bit_cast applied directly to an element of a vector,
+// bit_cast(float, v[1]), reads element 0 with this compiler: the element reference decays to the vector's address.)
+__device__ __forceinline__ float f32_of(unsigned v) { return __builtin_bit_cast(float, v); }
+__device__ __forceinline__ unsigned u32_of(float v) { return __builtin_bit_cast(unsigned, v); }
+
+// ---- item numbering ----
+// Workgroup b runs on XCD b % 8 (each XCD has its own L2).  The m-tiles that share one weight slice are dealt to
+// workgroups of ONE XCD in the same pass, so the slice crosses the fabric once per XCD.
+__device__ __forceinline__ bool xcd_item(int G, int it, int m_tiles, int w_slices, int *mt, int *ws) {
+  if ((G & 7) != 0) { *mt = it % m_tiles; *ws = it / m_tiles; return it < m_tiles * w_slices; }
+  const int xcd = it & 7, j = it >> 3;
+  *mt = j % m_tiles;
+  *ws = (j / m_tiles) * 8 + xcd;
+  return *ws < w_slices;
+}
+__device__ __forceinline__ int xcd_item_span(int G, int m_tiles, int w_slices) {   // exclusive upper bound of valid `it`
+  return (G & 7) != 0 ? m_tiles * w_slices : ((w_slices + 7) >> 3) * m_tiles * 8;
+}
+struct It { int a, b; };     // GEMM phases: (m-tile, slice); ATT: (16-query block, batch * 12 + head)
+__device__ __forceinline__ int ph_slices(int ph) { return ph == PH_QKV ? 36 : (ph == PH_OUT || ph == PH_FIN) ? 12 : 48; }
+__device__ __forceinline__ int ph_span(const Shape &s, int ph) {
+  return ph == PH_ATT ? xcd_item_span(s.G, s.S / 16, s.B * 12) : xcd_item_span(s.G, s.m_tiles, ph_slices(ph));
+}
+// Attention items go to workgroups 64.. when there is room, so that the workgroups of the out-projection
+// (the first ones) have their LDS free for the weight slice meanwhile.
+__device__ __forceinline__ int ph_off(const Shape &s, int ph) { return (ph == PH_ATT && ph_span(s, ph) + 64 <= s.G) ? 64 : 0; }
+__device__ __forceinline__ bool ph_item(const Shape &s, int ph, int it, It &d) {
+  if (ph == PH_ATT) return xcd_item(s.G, it, s.S / 16, s.B * 12, &d.a, &d.b);
+  return xcd_item(s.G, it, s.m_tiles, ph_slices(ph), &d.a, &d.b);
+}
+// items of workgroup b: it = b - off, b - off + G, ... below the span
+__device__ __forceinline__ bool has_items(const Shape &s, int ph, int b) {
+  It d;
+  for (int it = b - ph_off(s, ph); it < ph_span(s, ph); it += s.G)
+    if (it >= 0 && ph_item(s, ph, it, d)) return true;
+  return false;
+}
+// Does producer item p (of the phase that feeds phase cph) write something that consumer item c reads?
+__device__ __forceinline__ bool feeds(const Shape &s, int cph, const It &c, const It &p) {
+  switch (cph) {
+    case PH_ATT: {        // p = QKV (m-tile, q/k/v * 12 + head); c = (query block, batch * 12 + head)
+      const int b = c.b / 12, h = c.b % 12, j = p.b / 12, head = p.b % 12;
+      return head == h && (32 * p.a) / s.S == b && (j != 0 || (b * s.S + 16 * c.a) / 32 == p.a);
+    }
+    case PH_OUT: return ((p.b / 12) * s.S + 16 * p.a) / 32 == c.a;                 // p = ATT
+    case PH_FC2: return p.a == c.a && p.b / 12 == (c.b & 3);                       // p = FC1 slice, c = n-slice * 4 + K quarter
+    case PH_RED: return p.a == c.a && (p.b >> 2) == (c.b >> 2);                    // the four K quarters of one tile
+    default: return p.a == c.a;                                                    // QKV <- RED, FC1 <- OUT, FIN <- RED
+  }
+}
+__device__ __forceinline__ int producer_phase(int cph) { return cph == PH_QKV ? PH_RED : cph == PH_FIN ? PH_RED : cph - 1; }
+
+// Which of the workgroups 4 lane .. 4 lane + 3 must have published the producer phase before this workgroup may
+// start its items of phase cph (4 bits).  Exact where both phases are a single pass over the grid; otherwise every
+// workgroup that has an item of the producer phase.
+__device__ unsigned wait_mask(const Shape &s, int cph, int b, int lane) {
+  const int pph = producer_phase(cph);
+  const bool fine = ph_span(s, pph) + ph_off(s, pph) <= s.G && ph_span(s, cph) + ph_off(s, cph) <= s.G;
+  It c{0, 0};
+  bool mine = false;
+  if (fine) {
+    const int cit = b - ph_off(s, cph);
+    mine = cit >= 0 && cit < ph_span(s, cph) && ph_item(s, cph, cit, c);
+  } else mine = has_items(s, cph, b);
+  unsigned m = 0;
+  if (!mine) return 0;
+  for (int t = 0; t < 4; ++t) {
+    const int pb = 4 * lane + t;
+    if (pb >= s.G) break;
+    bool need;
+    if (fine) {
+      It p;
+      const int pit = pb - ph_off(s, pph);
+      need = pit >= 0 && pit < ph_span(s, pph) && ph_item(s, pph, pit, p) && feeds(s, cph, c, p);
+    } else need = has_items(s, pph, pb);
+    m |= (need ? 1u : 0u) << t;
+  }
+  return m;
+}
+
+// ---- hand-over ----
+__device__ __forceinline__ void sync_begin(Sync &sy, unsigned *flags, unsigned *err, unsigned long long *trace, int trace_cap) {
+  sy.flags = flags;
+  sy.err = err;
+  sy.failed = false;
+  sy.trace = trace;
+  sy.trace_cap = trace_cap;
+  sy.trace_idx = 0;
+  sy.base = __hip_atomic_load(flags + kFlagBaseWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Every workgroup of the launch calls this last.  The one that ends last moves the base past every value this
+// launch has published, so that the next launch on this workspace starts from flags that all read "not yet".
+__device__ __forceinline__ void sync_end(Sync &sy, int num_layers) {
+  if (threadIdx.x == 0) {
+    const unsigned old = __hip_atomic_fetch_add(sy.flags + kFlagDoneWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old + 1 == gridDim.x) {
+      __hip_atomic_store(sy.flags + kFlagDoneWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(sy.flags + kFlagBaseWord, sy.base + (unsigned)((num_layers + 1) * PH_SLOTS), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    wait_vmcnt<0>();
+  }
+}
+// This workgroup's items of a phase are written: publish.
+__device__ __forceinline__ void publish(const Sync &sy, unsigned seq) {
+  wait_vmcnt<0>();                               // this wave's write-through stores are acknowledged
+  __builtin_amdgcn_s_barrier();                  // ... and every wave's
+  if (threadIdx.x < kFlagCopies)
+    __hip_atomic_store(sy.flags + threadIdx.x * kFlagStride + blockIdx.x, seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Wait until the workgroups named by `mask` (wave 0: 4 bits per lane) have published `seq` or something later.
+// Bounded: a wait that gives up flags the control block and ends all waiting of the launch.
+__device__ __forceinline__ void await(Sync &sy, unsigned mask, unsigned seq) {
+  const bool tr = sy.trace && sy.trace_idx < sy.trace_cap && threadIdx.x == 0;
+  if (tr) sy.trace[(size_t)(2 * sy.trace_idx) * gridDim.x + blockIdx.x] = wall_clock64();
+  if (threadIdx.x < 64 && !sy.failed) {
+    const unsigned *copy = sy.flags + (blockIdx.x & (kFlagCopies - 1)) * kFlagStride;
+    for (int spin = 0;; ++spin) {
+      const u4 f = ld16<true>(copy, (int)threadIdx.x * 16);
+      bool ok = true;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) ok &= !((mask >> t) & 1u) || (int)(f[t] - seq) >= 0;
+      if (__all(ok)) break;
+      if (spin >= kMaxFlagSpin) {
+        sy.failed = true;
+        if (threadIdx.x == 0) (void)__hip_atomic_fetch_or(sy.err, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+    }
+  }
+  if (tr) sy.trace[(size_t)(2 * sy.trace_idx + 1) * gridDim.x + blockIdx.x] = wall_clock64();
+  sy.trace_idx++;
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// ---- row statistics ----
+// st[m][12][2]: per row and per 64-column slice (mean, sum of squared deviations from that mean) of the fp16 values.
+// Combination of the twelve slices of a row (equal counts): mean = average of the means,
+// M2 = sum M2_i + 64 sum (mean_i - mean)^2.
+struct RowStat { float mean, rstd; };
+
+// 8 consecutive lanes share row m: lane t of the group reads slices t and t + 8.
+__device__ __forceinline__ RowStat row_stat8(const float *st, int m, int t8, float eps) {
+  const u2 p0 = ld8<true>(st, (m * 12 + t8) * 8);
+  u2 p1 = {0u, 0u};
+  if (t8 < 4) p1 = ld8<true>(st, (m * 12 + 8 + t8) * 8);
+  const float m0 = f32_of(p0[0]), q0 = f32_of(p0[1]);
+  const float m1 = f32_of(p1[0]), q1 = f32_of(p1[1]);
+  float s = m0 + (t8 < 4 ? m1 : 0.f);
+  s += wave_xor(s, 1); s += wave_xor(s, 2); s += wave_xor(s, 4);
+  const float mean = s * (1.0f / 12.0f);
+  float q = q0 + 64.0f * (m0 - mean) * (m0 - mean);
+  if (t8 < 4) q += q1 + 64.0f * (m1 - mean) * (m1 - mean);
+  q += wave_xor(q, 1); q += wave_xor(q, 2); q += wave_xor(q, 4);
+  return RowStat{mean, rsqrtf(q * (1.0f / 768.0f) + eps)};
+}
+// Publish the statistics of 64 values of a row held by `n` consecutive lanes (v: this lane's values, already
+// rounded to fp16 and widened again); lane 0 of the group stores.
+template <int PER, int LANES>
+__device__ __forceinline__ void put_stat(float *st, int m, int slice, const float (&v)[PER], int lane_in_group) {
+  static_assert(PER * LANES == 64, "a slice is 64 columns");
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) s += v[i];
+#pragma unroll
+  for (int k = 1; k < LANES; k <<= 1) s += wave_xor(s, k);
+  const float mean = s * (1.0f / 64.0f);
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) { const float d = v[i] - mean; q += d * d; }
+#pragma unroll
+  for (int k = 1; k < LANES; k <<= 1) q += wave_xor(q, k);
+  if (lane_in_group == 0) st8<true>(st, (m * 12 + slice) * 8, u2{u32_of(mean), u32_of(q)});
+}
+
+// ---- GEMM item: 32 rows x 64 columns over a K slice of 768 ----
+// Wave w owns the K quarter [192 w, 192 w + 192): it loads exactly the operand bytes it multiplies, so nothing
+// but its own loads stands between a wave and its MFMAs, and a k-step starts as soon as its two X blocks are
+// there.  X blocks are stored in operand order (block (s, i): lane L's 16 bytes are X[16 i + L % 16][32 s + 8 (L / 16) ..]),
+// W rows as [k][64] with the 16-byte slot index XORed with (k & 2) for the transposing read.
+struct GemmItem {
+  const half_t *X; int ldx, kx0;      // activation rows start at column kx0
+  const half_t *W; int ldw, kw0, n0;  // weight rows kw0 .. kw0 + 767, columns n0 .. n0 + 63
+  int m0;
+};
+
+__device__ __forceinline__ void issue_w(unsigned char *lds, const GemmItem &g) {
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
+  const half_t *sb = uniform_ptr(g.W + (size_t)(g.kw0 + 192 * w) * g.ldw + g.n0);
+  const int rl = lane >> 3;
+  unsigned voff = (unsigned)(rl * g.ldw * 2 + (((lane & 7) ^ (rl & 2)) * 16));
+  const unsigned step = (unsigned)(8 * g.ldw * 2);
+  const unsigned base = uni(lds_address(lds) + kWOff + 24 * 1024 * w);
+#pragma unroll
+  for (int q = 0; q < 24; ++q) {
+    dma16<false>(sb, voff, base + q * 1024);
+    voff += step;
+  }
+}
+// gamma and beta of the LayerNorm applied on load: every wave fetches the 192 values of its own K quarter
+// (wave w: [gamma quarter 384 B][beta quarter 384 B] at kGamOff + 768 w; a missing vector is written as ones /
+// zeros), so that like its operands they are its own loads.  The bias of the item's 64 columns is fetched by wave 3.
+__device__ __forceinline__ void issue_params(unsigned char *lds, const half_t *gam, const half_t *bet, bool ln_affine,
+                                             const half_t *bias, int n0) {
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
+  if (ln_affine) {
+    unsigned char *dst = lds + kGamOff + 768 * w;
+    if (lane < 24) {
+      if (gam) dma16<false>(uniform_ptr(gam + 192 * w), (unsigned)lane * 16, uni(lds_address(dst)));
+      else { const half_t c = (half_t)1.0f; *reinterpret_cast<h8 *>(dst + lane * 16) = h8{c, c, c, c, c, c, c, c}; }
+      if (bet) dma16<false>(uniform_ptr(bet + 192 * w), (unsigned)lane * 16, uni(lds_address(dst + 384)));
+      else { const half_t c = (half_t)0.0f; *reinterpret_cast<h8 *>(dst + 384 + lane * 16) = h8{c, c, c, c, c, c, c, c}; }
+    }
+  }
+  if (bias && w == 3 && lane < 8) dma16<false>(uniform_ptr(bias + n0), (unsigned)lane * 16, uni(lds_address(lds) + kBiasOff));
+}
+// this wave's twelve X blocks, in k-step order
+template <bool SC1>
+__device__ __forceinline__ void issue_x(unsigned char *lds, const GemmItem &g) {
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6, l16 = lane & 15, gq = lane >> 4;
+  const half_t *sb = uniform_ptr(g.X + (size_t)g.m0 * g.ldx + g.kx0 + 192 * w);
+  unsigned v0 = (unsigned)((l16 * g.ldx + gq * 8) * 2);
+  unsigned v1 = v0 + (unsigned)(16 * g.ldx * 2);
+  const unsigned base = uni(lds_address(lds) + kXPart * w);
+#pragma unroll
+  for (int s = 0; s < 6; ++s) {
+    dma16<SC1>(sb, v0, base + (2 * s) * 1024);
+    dma16<SC1>(sb, v1, base + (2 * s + 1) * 1024);
+    v0 += 64;
+    v1 += 64;
+  }
+}
+// the statistics of rows m0 .. m0 + 31 (3 KB, contiguous), one copy per wave (COPIES = 4) or one for the workgroup
+template <int COPIES>
+__device__ __forceinline__ void issue_stats(unsigned char *lds, const float *st, int m0) {
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
+  const float *sb = uniform_ptr(st + (size_t)m0 * 24);
+  if constexpr (COPIES == 4) {
+    const unsigned base = uni(lds_address(lds) + kAuxOff + kStatBytes * w);
+#pragma unroll
+    for (int q = 0; q < 3; ++q) dma16<true>(sb, (unsigned)(q * 1024 + lane * 16), base + q * 1024);
+  } else {
+    if (w < 3) dma16<true>(sb, (unsigned)(w * 1024 + lane * 16), uni(lds_address(lds) + kAuxOff + 4096 + w * 1024));
+  }
+}
+
+enum { LN_NONE = 0, LN_PLAIN = 1, LN_AFFINE = 2 };
+
+// f(integral_constant<int, I>) for I = BEGIN .. END - 1: a loop whose index is a compile-time constant (s_waitcnt
+// takes its count as an immediate).
+template <int BEGIN, int END, class F>
+__device__ __forceinline__ void static_for(F f) {
+  if constexpr (BEGIN < END) {
+    f(std::integral_constant<int, BEGIN>{});
+    static_for<BEGIN + 1, END>(f);
+  }
+}
+
+// The operand registers of one k-step.
+struct KOps { h8 x[2], w[4]; };
+__device__ __forceinline__ void read_ops(const unsigned char *lds, int w, int lane, int s, KOps &o) {
+  const int l16 = lane & 15, gq = lane >> 4;
+  const unsigned char *xb = lds + kXPart * w + (2 * s) * 1024 + lane * 16;
+  o.x[0] = *reinterpret_cast<const h8 *>(xb);
+  o.x[1] = *reinterpret_cast<const h8 *>(xb + 1024);
+  const half_t *ws = reinterpret_cast<const half_t *>(lds + kWOff);
+  const int k = 192 * w + 32 * s + gq * 8 + (l16 >> 2);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = j * 2 + ((l16 & 3) >> 1);
+    const half_t *p = ws + (k * 8 + (c ^ (k & 2))) * 8 + (l16 & 1) * 4;
+    const h4 lo = lds_read_tr16(p), hi = lds_read_tr16(p + 4 * 64);
+    o.w[j] = h8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  }
+}
+
+// acc[i][j]: rows 16 i + lane % 16, columns 16 j + 4 (lane / 16) .. + 3, summed over this wave's K quarter.
+// LN: the X operand is normalised in registers, (x - mean) * rstd [* gamma + beta], in packed fp16 arithmetic: the
+// fp16 part of the mean is subtracted first (a difference of neighbouring values, rounded relative to itself), what
+// rounding the mean to fp16 left over enters through the addend of the multiply-add, so that it does not shift the row.
+template <int LN>
+__device__ __forceinline__ void mfma_quarter(const unsigned char *lds, f4 (&acc)[2][4], float eps) {
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6, l16 = lane & 15, gq = lane >> 4;
+  h8 nmh[2], off[2], rs[2];     // -mean (its fp16 part), -(mean - that part) * rstd, rstd
+  if constexpr (LN != LN_NONE) {
+    // Lane L combines row L / 2: slices 6 (L % 2) .. + 5 from this wave's copy of the statistics, then its partner's.
+    wait_vmcnt<12>();                    // the three statistics loads are older than the twelve X blocks
+    const int row = lane >> 1, half = lane & 1;
+    const float *sp = reinterpret_cast<const float *>(lds + kAuxOff + kStatBytes * w) + (row * 12 + 6 * half) * 2;
+    float mi[6], qi[6];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      const f4 v = *reinterpret_cast<const f4 *>(sp + 4 * i);
+      mi[2 * i] = v[0]; qi[2 * i] = v[1]; mi[2 * i + 1] = v[2]; qi[2 * i + 1] = v[3];
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 6; ++i) s += mi[i];
+    s += wave_xor(s, 1);
+    const float mean = s * (1.0f / 12.0f);
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < 6; ++i) q += qi[i] + 64.0f * (mi[i] - mean) * (mi[i] - mean);
+    q += wave_xor(q, 1);
+    const float rstd = rsqrtf(q * (1.0f / 768.0f) + eps);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const float mu = __shfl(mean, 2 * (16 * i + l16), kWave), r = __shfl(rstd, 2 * (16 * i + l16), kWave);
+      const half_t a = (half_t)mu, c = (half_t)fminf(r, 65504.0f), b2 = (half_t)(((float)a - mu) * (float)c), na = -a;
+      nmh[i] = h8{na, na, na, na, na, na, na, na};
+      off[i] = h8{b2, b2, b2, b2, b2, b2, b2, b2};
+      rs[i] = h8{c, c, c, c, c, c, c, c};
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+  KOps cur, nxt;
+  wait_vmcnt<10>();
+  read_ops(lds, w, lane, 0, cur);
+  static_for<0, 6>([&](auto sc) {
+    constexpr int s = decltype(sc)::value;
+    if constexpr (s + 1 < 6) {
+      wait_vmcnt<10 - 2 * (s + 1)>();
+      read_ops(lds, w, lane, s + 1, nxt);
+    }
+    if constexpr (LN != LN_NONE) {
+      h8 gm, bt;
+      if constexpr (LN == LN_AFFINE) {
+        gm = *reinterpret_cast<const h8 *>(lds + kGamOff + 768 * w + (32 * s + 8 * gq) * 2);
+        bt = *reinterpret_cast<const h8 *>(lds + kGamOff + 768 * w + 384 + (32 * s + 8 * gq) * 2);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        h8 t = (cur.x[i] + nmh[i]) * rs[i] + off[i];     // (x - mean) * rstd: the first difference is all but exact
+        if constexpr (LN == LN_AFFINE) t = t * gm + bt;
+        cur.x[i] = t;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = mfma_16x16x32(cur.w[j], cur.x[i], acc[i][j]);
+    if constexpr (s + 1 < 6) cur = nxt;
+  });
+}
+
+// The four partial tiles are summed through LDS (each wave parks its own in its X part, which only it reads);
+// epi(row, col0, lo, hi) then receives 8 consecutive columns of a row per thread (row = tid / 8, col0 = 8 (tid % 8)).
+template <class Epi>
+__device__ __forceinline__ void reduce_tile(unsigned char *lds, const f4 (&acc)[2][4], Epi epi) {
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6, l16 = lane & 15, gq = lane >> 4;
+  float *mine = reinterpret_cast<float *>(lds + kXPart * w);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<f4 *>(mine + (i * 16 + l16) * kRedLd + j * 16 + gq * 4) = acc[i][j];
+  __syncthreads();
+  const int row = tid >> 3, col0 = (tid & 7) * 8;
+  const float *src = reinterpret_cast<const float *>(lds) + row * kRedLd + col0;
+  f4 lo = *reinterpret_cast<const f4 *>(src), hi = *reinterpret_cast<const f4 *>(src + 4);
+#pragma unroll
+  for (int k = 1; k < 4; ++k) {
+    lo += *reinterpret_cast<const f4 *>(src + k * (kXPart / 4));
+    hi += *reinterpret_cast<const f4 *>(src + k * (kXPart / 4) + 4);
+  }
+  epi(row, col0, lo, hi);
+}
+
+
+// ------------------------------------------------------------------ attention ----
+// One item = one head x 16 queries.  Each wave handles a quarter of the keys for the same 16 queries and loads
+// exactly the K/V rows it multiplies (no workgroup barrier before the MFMAs); the four partial results are
+// merged through LDS the flash-attention way (running maximum, rescaled sums).
+// [reference: cpp/bert/kernels/fused_sqq_bert.cu:2772-3329]
+constexpr int kAttnCombLd = 68;                                   // floats per row of a wave's partial context
+constexpr int attn_lds_bytes(int S) { return 2 * S * 128 + 4 * 2048 + 4 * 16 * kAttnCombLd * 4 + 512; }
+
+// Rows row0 .. row0 + rows - 1 of a [*][64] fp16 tile into LDS (128-byte rows = 8 slots of 16 bytes), swizzled for
+// its reader: MODE 0 for b128 operand reads of 16 consecutive rows (slot ^= (row >> 1) & 7), MODE 1 for the
+// transposing read of 4 consecutive rows (slot ^= row & 2).  sc1 loads: the tile was written by other workgroups.
+template <int MODE>
+__device__ __forceinline__ void issue_rows64_wave(unsigned char *lds_tile, const half_t *src, int row0, int rows) {
+  typedef __attribute__((address_space(1))) const void *gptr_t;
+  typedef __attribute__((address_space(3))) void *lptr_t;
+  const int lane = threadIdx.x & 63;
+  for (int inst = 0; inst < rows / 8; ++inst) {
+    const int r = row0 + inst * 8 + (lane >> 3), c = (lane & 7) ^ (MODE == 0 ? ((r >> 1) & 7) : (r & 2));
+    __builtin_amdgcn_global_load_lds((gptr_t)(src + (size_t)r * HD + c * 8), (lptr_t)(lds_tile + (row0 + inst * 8) * 128), 16, 0, kAuxSc1);
+  }
+}
+
+struct AttnArgs {
+  int B, S;
+  float scale;
+  const half_t *qkv, *mask;
+  half_t *ctx, *probs;
+};
+
+template <int NKT>
+__device__ __forceinline__ void attn_item_split(unsigned char *lds, const AttnArgs &a, int bh, int qb) {
+  constexpr int S = NKT * 16, TPW = NKT / 4;                       // key tiles per wave
+  static_assert(NKT % 4 == 0, "keys split evenly over four waves");
+  unsigned char *ks_ = lds, *vs_ = lds + S * 128, *qs_ = lds + 2 * S * 128;
+  float *comb = reinterpret_cast<float *>(lds + 2 * S * 128 + 4 * 2048);
+  float *stats = comb + 4 * 16 * kAttnCombLd;                      // [wave][query][max, sum]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+  const int b = bh / NH, hh = bh % NH;
+  const int head_off = ((b * NH + hh) * S) * HD;                   // halves, within one of q/k/v
+  const size_t plane = (size_t)a.B * NH * S * HD;
+  const half_t *Q = a.qkv + head_off + (size_t)qb * 16 * HD, *K = a.qkv + plane + head_off, *V = a.qkv + 2 * plane + head_off;
+
+  __syncthreads();   // LDS reuse
+  issue_rows64_wave<0>(qs_ + wave * 2048, Q, 0, 16);               // every wave its own copy of the queries
+  issue_rows64_wave<0>(ks_, K, wave * TPW * 16, TPW * 16);
+  issue_rows64_wave<1>(vs_, V, wave * TPW * 16, TPW * 16);
+  __builtin_amdgcn_s_waitcnt(0);                                   // this wave's rows only: no barrier needed
+
+  const half_t *kh = reinterpret_cast<const half_t *>(ks_), *vh = reinterpret_cast<const half_t *>(vs_),
+               *qh = reinterpret_cast<const half_t *>(qs_ + wave * 2048);
+  const int q = qb * 16 + l16;
+  h8 qop[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) qop[ks] = *reinterpret_cast<const h8 *>(qh + (l16 * 8 + ((ks * 4 + g) ^ ((l16 >> 1) & 7))) * 8);
+  f4 sc[TPW];
+  float mx = -1e30f;                                               // finite: a fully masked quarter contributes nothing
+#pragma unroll
+  for (int tt = 0; tt < TPW; ++tt) {
+    const int t = wave * TPW + tt, r = t * 16 + l16, sw = (r >> 1) & 7;
+    const h8 k0 = *reinterpret_cast<const h8 *>(kh + (r * 8 + (g ^ sw)) * 8);
+    const h8 k1 = *reinterpret_cast<const h8 *>(kh + (r * 8 + ((4 + g) ^ sw)) * 8);
+    f4 sv = mfma_16x16x32(k1, qop[1], mfma_16x16x32(k0, qop[0], f4{0.f, 0.f, 0.f, 0.f})) * a.scale;
+    // sv[v] = score(key = 16t + 4g + v, query = q)
+    if (a.mask) {
+      const h4 mk = ldg<h4>(a.mask + ((size_t)b * S + q) * S + t * 16 + g * 4);
+      sv += f4{(float)mk[0], (float)mk[1], (float)mk[2], (float)mk[3]};
+    }
+    sc[tt] = sv;
+    mx = fmaxf(mx, fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
+  }
+  mx = fmaxf(mx, wave_xor(mx, 16));
+  mx = fmaxf(mx, wave_xor(mx, 32));
+  float sum = 0.f;
+  h4 p[TPW];
+#pragma unroll
+  for (int tt = 0; tt < TPW; ++tt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { sc[tt][i] = __expf(sc[tt][i] - mx); sum += sc[tt][i]; }
+    p[tt] = h4{(half_t)sc[tt][0], (half_t)sc[tt][1], (half_t)sc[tt][2], (half_t)sc[tt][3]};
+  }
+  sum += wave_xor(sum, 16);
+  sum += wave_xor(sum, 32);
+  f4 o[HD / 16];
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt) o[dt] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int tt = 0; tt < TPW; ++tt) {
+    const int kr = (wave * TPW + tt) * 16 + g * 4 + (l16 >> 2);
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) {
+      const int c = dt * 2 + ((l16 & 3) >> 1);
+      const h4 vop = lds_read_tr16(vh + (kr * 8 + (c ^ (kr & 2))) * 8 + (l16 & 1) * 4);
+      o[dt] = mfma_16x16x16(vop, p[tt], o[dt]);
+    }
+  }
+  // o[dt][v] = sum over this wave's keys of exp(score - mx) * V[key][16dt + 4g + v], query q
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt)
+    *reinterpret_cast<f4 *>(comb + (wave * 16 + l16) * kAttnCombLd + dt * 16 + g * 4) = o[dt];
+  if (g == 0) { stats[(wave * 16 + l16) * 2] = mx; stats[(wave * 16 + l16) * 2 + 1] = sum; }
+  __syncthreads();
+  float wmx[4], wsum[4];
+  auto merged = [&](int qq, float *scale) {                        // scale[w] = exp(mx_w - max) / total
+    float m = -1e30f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) { wmx[w] = stats[(w * 16 + qq) * 2]; wsum[w] = stats[(w * 16 + qq) * 2 + 1]; m = fmaxf(m, wmx[w]); }
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) { scale[w] = __expf(wmx[w] - m); total += wsum[w] * scale[w]; }
+    const float inv = 1.0f / total;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) scale[w] *= inv;
+  };
+  {
+    const int qq = tid >> 4, d0 = (tid & 15) * 4;
+    float scale[4];
+    merged(qq, scale);
+    f4 r = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) r += *reinterpret_cast<const f4 *>(comb + (w * 16 + qq) * kAttnCombLd + d0) * scale[w];
+    st8<true>(a.ctx, ((b * S + qb * 16 + qq) * H + hh * HD + d0) * 2, pack_h4(r));
+  }
+  if (a.probs) {
+    float scale[4];
+    merged(l16, scale);
+#pragma unroll
+    for (int tt = 0; tt < TPW; ++tt) {
+      const f4 pr = sc[tt] * scale[wave];
+      const h4 ph = {(half_t)pr[0], (half_t)pr[1], (half_t)pr[2], (half_t)pr[3]};
+      st8<false>(a.probs, (int)((((size_t)(b * NH + hh) * S + q) * S + (wave * TPW + tt) * 16 + g * 4) * 2), as_u2(ph));
+    }
+  }
+}
+
+// ------------------------------------------------------------------ phases ----
+// Kernel arguments.  The inter-phase buffers exist once per layer (layer l at + l * layer_stride bytes): inside a
+// launch every address is written by one item of one phase and read only afterwards.
+struct Args {
+  int B, S, M, act, num_layers;
+  float scale, eps;
+  const half_t *x, *mask;
+  half_t *y;
+  half_t *qkv, *ctx, *z1, *h, *z2;     // [3][B][12][S][64], [M][768], [M][768] (pre-LN1 sum), [M][3072], [M][768] (pre-LN2 sum)
+  float *st1, *st2, *part;             // row statistics of z1 / z2 [M][12][2], FC2 partial sums [4][M][768]
+  half_t *probs, *ln1_out;             // optional per-stage outputs (single layer only)
+  size_t layer_stride;
+  unsigned *ctl, *flags;
+  unsigned long long *trace;
+  int trace_cap;
+  LayerW layers[kMaxLayers];
+};
+struct Bufs { half_t *qkv, *ctx, *z1, *h, *z2; float *st1, *st2, *part; };
+__device__ __forceinline__ Bufs layer_bufs(const Args &a, int l) {
+  const size_t off = (size_t)l * a.layer_stride;
+  auto adv = [&](auto *q) { return uniform_ptr(reinterpret_cast<decltype(q)>(reinterpret_cast<char *>(q) + off)); };
+  return Bufs{adv(a.qkv), adv(a.ctx), adv(a.z1), adv(a.h), adv(a.z2), adv(a.st1), adv(a.st2), adv(a.part)};
+}
+
+// What a GEMM item of (layer l, phase ph) multiplies, and what travels with its weight slice.
+struct Job {
+  GemmItem g;
+  int ln;                              // LN_* applied to X on load
+  const float *stats;                  // statistics of the X rows (ln != LN_NONE)
+  const half_t *gam, *bet;             // of that LayerNorm
+  const half_t *bias;                  // of the item's columns (LDS copy at kBiasOff), or null
+  const half_t *rgam, *rbet;           // OUT: gamma / beta of the LayerNorm that produces the residual (LDS copies), or null
+  bool x_sc1;
+};
+__device__ __forceinline__ Job make_job(const Args &a, int l, int ph, const It &d) {
+  const LayerW &w = a.layers[l];
+  const Bufs cur = layer_bufs(a, l);
+  Job j{};
+  j.g.m0 = d.a * 32;
+  j.ln = LN_NONE;
+  j.x_sc1 = true;
+  if (ph == PH_QKV) {
+    const int which = d.b / 12, head = d.b % 12;
+    j.g.W = w.w_qkv + (size_t)which * H * H; j.g.ldw = H; j.g.kw0 = 0; j.g.n0 = head * HD;
+    j.g.ldx = H; j.g.kx0 = 0;
+    if (l == 0) { j.g.X = a.x; j.x_sc1 = false; }
+    else {
+      const LayerW &pw = a.layers[l - 1];
+      const Bufs prev = layer_bufs(a, l - 1);
+      j.g.X = prev.z2; j.stats = prev.st2; j.gam = pw.ln2_g; j.bet = pw.ln2_b;
+      j.ln = (pw.ln2_g || pw.ln2_b) ? LN_AFFINE : LN_PLAIN;
+    }
+    j.bias = w.b_qkv ? w.b_qkv + which * H : nullptr;
+  } else if (ph == PH_OUT) {
+    j.g.W = w.w_o; j.g.ldw = H; j.g.kw0 = 0; j.g.n0 = d.b * 64;
+    j.g.X = cur.ctx; j.g.ldx = H; j.g.kx0 = 0;
+    j.bias = w.b_o;
+    if (l > 0) { j.rgam = a.layers[l - 1].ln2_g; j.rbet = a.layers[l - 1].ln2_b; }
+  } else if (ph == PH_FC1) {
+    j.g.W = w.w_fc1; j.g.ldw = F; j.g.kw0 = 0; j.g.n0 = d.b * 64;
+    j.g.X = cur.z1; j.g.ldx = H; j.g.kx0 = 0;
+    j.stats = cur.st1; j.gam = w.ln1_g; j.bet = w.ln1_b;
+    j.ln = (w.ln1_g || w.ln1_b) ? LN_AFFINE : LN_PLAIN;
+    j.bias = w.b_fc1;
+  } else {   // PH_FC2: slice = n-slice * 4 + K quarter
+    const int ks = d.b & 3, ns = d.b >> 2;
+    j.g.W = w.w_fc2; j.g.ldw = H; j.g.kw0 = ks * 768; j.g.n0 = ns * 64;
+    j.g.X = cur.h; j.g.ldx = F; j.g.kx0 = ks * 768;
+  }
+  return j;
+}
+// The loads of an item that depend on no other workgroup: weight slice, LayerNorm vectors, bias.
+__device__ __forceinline__ void issue_weights(unsigned char *lds, const Job &j) {
+  issue_w(lds, j.g);
+  issue_params(lds, j.gam, j.bet, j.ln == LN_AFFINE, j.bias, j.g.n0);
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
+  if (w == 2 && lane < 8) {      // the residual's LayerNorm vectors for the item's 64 columns (OUT)
+    if (j.rgam) dma16<false>(uniform_ptr(j.rgam + j.g.n0), (unsigned)lane * 16, uni(lds_address(lds) + kGamOff));
+    if (j.rbet) dma16<false>(uniform_ptr(j.rbet + j.g.n0), (unsigned)lane * 16, uni(lds_address(lds) + kGamOff + 128));
+  }
+}
+
+__device__ __forceinline__ f4 widen(h4 v) { return f4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]}; }
+
+// One GEMM item from operand fetch to the stores of its epilogue.
+__device__ __forceinline__ void run_gemm_item(unsigned char *lds, const Args &a, int l, int ph, const It &d, bool w_ready) {
+  const Job j = make_job(a, l, ph, d);
+  const Bufs cur = layer_bufs(a, l);
+  if (!w_ready) issue_weights(lds, j);
+  // what the item reads of other workgroups' results, statistics first (they are needed first)
+  if (j.ln != LN_NONE) issue_stats<4>(lds, j.stats, j.g.m0);
+  if (ph == PH_OUT) {
+    const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
+    const half_t *res = l == 0 ? a.x : layer_bufs(a, l - 1).z2;
+    // residual patch: rows m0 .. m0 + 31, columns n0 .. n0 + 63 -> [32][128 B] at kAuxOff
+    dma16<true>(uniform_ptr(res + (size_t)(j.g.m0 + 8 * w) * H + j.g.n0), (unsigned)((lane >> 3) * H * 2 + (lane & 7) * 16),
+                uni(lds_address(lds) + kAuxOff + w * 1024));
+    if (l > 0) issue_stats<1>(lds, layer_bufs(a, l - 1).st2, j.g.m0);
+  }
+  if (j.x_sc1) issue_x<true>(lds, j.g); else issue_x<false>(lds, j.g);
+  f4 acc[2][4];
+  if (j.ln == LN_NONE) mfma_quarter<LN_NONE>(lds, acc, a.eps);
+  else if (j.ln == LN_PLAIN) mfma_quarter<LN_PLAIN>(lds, acc, a.eps);
+  else mfma_quarter<LN_AFFINE>(lds, acc, a.eps);
+  const half_t *bias_lds = j.bias ? reinterpret_cast<const half_t *>(lds + kBiasOff) : nullptr;
+  auto add_bias = [&](int col0, f4 &lo, f4 &hi) {
+    if (bias_lds) {
+      const h8 bb = *reinterpret_cast<const h8 *>(bias_lds + col0);
+      lo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+      hi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]};
+    }
+  };
+  if (ph == PH_QKV) {
+    const int which = d.b / 12, head = d.b % 12;
+    reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
+      add_bias(col0, lo, hi);
+      const int m = j.g.m0 + row, b = m / a.S, s = m % a.S;
+      st16<true>(cur.qkv, ((((which * a.B + b) * NH + head) * a.S + s) * HD + col0) * 2, pack_h8(lo, hi));
+    });
+  } else if (ph == PH_OUT) {
+    reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
+      add_bias(col0, lo, hi);
+      const h8 rv = *reinterpret_cast<const h8 *>(lds + kAuxOff + row * 128 + col0 * 2);
+      f4 rlo = f4{(float)rv[0], (float)rv[1], (float)rv[2], (float)rv[3]}, rhi = f4{(float)rv[4], (float)rv[5], (float)rv[6], (float)rv[7]};
+      if (l > 0) {   // the residual is LN2 of the previous layer's sum: normalise the patch
+        const float *sp = reinterpret_cast<const float *>(lds + kAuxOff + 4096) + row * 24;
+        float mean = 0.f;
+#pragma unroll
+        for (int i = 0; i < 12; ++i) mean += sp[2 * i];
+        mean *= (1.0f / 12.0f);
+        float q = 0.f;
+#pragma unroll
+        for (int i = 0; i < 12; ++i) q += sp[2 * i + 1] + 64.0f * (sp[2 * i] - mean) * (sp[2 * i] - mean);
+        const float rstd = rsqrtf(q * (1.0f / 768.0f) + a.eps);
+        rlo = (rlo - mean) * rstd; rhi = (rhi - mean) * rstd;
+        if (j.rgam) { const h8 gg = *reinterpret_cast<const h8 *>(lds + kGamOff + col0 * 2); rlo *= f4{(float)gg[0], (float)gg[1], (float)gg[2], (float)gg[3]}; rhi *= f4{(float)gg[4], (float)gg[5], (float)gg[6], (float)gg[7]}; }
+        if (j.rbet) { const h8 bb = *reinterpret_cast<const h8 *>(lds + kGamOff + 128 + col0 * 2); rlo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]}; rhi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]}; }
+      }
+      lo += rlo; hi += rhi;
+      const int m = j.g.m0 + row;
+      const u4 packed = pack_h8(lo, hi);
+      st16<true>(cur.z1, (m * H + j.g.n0 + col0) * 2, packed);
+      const h8 r8 = as_h8(packed);
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = (float)r8[i];
+      put_stat<8, 8>(cur.st1, m, d.b, v, opaque_thread_id() & 7);
+    });
+  } else if (ph == PH_FC1) {
+    reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
+      add_bias(col0, lo, hi);
+      if (a.act == SOUFFLE_ACT_RELU) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { lo[i] = fmaxf(lo[i], 0.f); hi[i] = fmaxf(hi[i], 0.f); }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { lo[i] = gelu_tanh(lo[i]); hi[i] = gelu_tanh(hi[i]); }
+      }
+      st16<true>(cur.h, ((j.g.m0 + row) * F + j.g.n0 + col0) * 2, pack_h8(lo, hi));
+    });
+  } else {
+    const int ks = d.b & 3;
+    reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
+      const int off = ((ks * a.M + j.g.m0 + row) * H + j.g.n0 + col0) * 4;
+      st16<true>(cur.part, off, __builtin_bit_cast(u4, lo));
+      st16<true>(cur.part, off + 16, __builtin_bit_cast(u4, hi));
+    });
+  }
+}
+
+// RED: rows 8 ks .. 8 ks + 7 of the tile of FC2 item (m-tile, n-slice * 4 + ks): z2 = sum of the four partial sums
+// (in order) + bias + LN1(z1), rounded to fp16, and the statistics of those 64 values per row.
+// `pre` runs between the loads that need no sibling and those that do (the wait for the siblings).
+template <class Pre>
+__device__ __forceinline__ void run_red_item(const Args &a, int l, const It &d, Pre pre) {
+  const LayerW &w = a.layers[l];
+  const Bufs cur = layer_bufs(a, l);
+  const int tid = opaque_thread_id(), row = tid >> 5, cp = tid & 31;
+  const int ks = d.b & 3, ns = d.b >> 2, m = d.a * 32 + ks * 8 + row, n = ns * 64 + 2 * cp;
+  // LN1 of the residual
+  u2 part_stat = {0u, 0u};
+  if (cp < 12) part_stat = ld8<true>(cur.st1, (m * 12 + cp) * 8);
+  const unsigned zraw = ld4<true>(cur.z1, (m * H + n) * 2);
+  float g0 = 1.f, g1 = 1.f, e0 = 0.f, e1 = 0.f, c0 = 0.f, c1 = 0.f;
+  if (w.ln1_g) { const h2 t = ldg<h2>(w.ln1_g + n); g0 = (float)t[0]; g1 = (float)t[1]; }
+  if (w.ln1_b) { const h2 t = ldg<h2>(w.ln1_b + n); e0 = (float)t[0]; e1 = (float)t[1]; }
+  if (w.b_fc2) { const h2 t = ldg<h2>(w.b_fc2 + n); c0 = (float)t[0]; c1 = (float)t[1]; }
+  const float pm = cp < 12 ? f32_of(part_stat[0]) : 0.f, pq = f32_of(part_stat[1]);
+  float s = pm;
+#pragma unroll
+  for (int k = 1; k < 32; k <<= 1) s += wave_xor(s, k);
+  const float mean = s * (1.0f / 12.0f);
+  float q = cp < 12 ? pq + 64.0f * (pm - mean) * (pm - mean) : 0.f;
+#pragma unroll
+  for (int k = 1; k < 32; k <<= 1) q += wave_xor(q, k);
+  const float rstd = rsqrtf(q * (1.0f / 768.0f) + a.eps);
+  const h2 z = __builtin_bit_cast(h2, zraw);
+  const float y0 = ((float)z[0] - mean) * rstd * g0 + e0, y1 = ((float)z[1] - mean) * rstd * g1 + e1;
+  if (a.ln1_out) *reinterpret_cast<h2 *>(a.ln1_out + (size_t)m * H + n) = h2{(half_t)y0, (half_t)y1};
+  pre();
+  float v0 = 0.f, v1 = 0.f;
+  u2 pr[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) pr[k] = ld8<true>(cur.part, ((k * a.M + m) * H + n) * 4);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) { v0 += f32_of(pr[k][0]); v1 += f32_of(pr[k][1]); }
+  v0 += c0 + y0; v1 += c1 + y1;
+  const h2 out = {(half_t)v0, (half_t)v1};
+  st4<true>(cur.z2, (m * H + n) * 2, __builtin_bit_cast(unsigned, out));
+  float vv[2] = {(float)out[0], (float)out[1]};
+  put_stat<2, 32>(cur.st2, m, ns, vv, cp);
+}
+
+// FIN: y = LN2 of the last layer's sum, a 32 x 64 patch per item.
+__device__ __forceinline__ void run_fin_item(const Args &a, const It &d) {
+  const int l = a.num_layers - 1;
+  const LayerW &w = a.layers[l];
+  const Bufs cur = layer_bufs(a, l);
+  const int tid = opaque_thread_id(), row = tid >> 3, t8 = tid & 7, m = d.a * 32 + row, n = d.b * 64 + t8 * 8;
+  const h8 z = as_h8(ld16<true>(cur.z2, (m * H + n) * 2));
+  const RowStat rs = row_stat8(cur.st2, m, t8, a.eps);
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = ((float)z[i] - rs.mean) * rs.rstd;
+  if (w.ln2_g) { const h8 g8 = ldg<h8>(w.ln2_g + n);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] *= (float)g8[i]; }
+  if (w.ln2_b) { const h8 b8 = ldg<h8>(w.ln2_b + n);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] += (float)b8[i]; }
+  const h8 o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3], (half_t)v[4], (half_t)v[5], (half_t)v[6], (half_t)v[7]};
+  st16<false>(a.y, (m * H + n) * 2, as_u4(o));
+}
+
+// for every item of phase ph that belongs to workgroup b: fn(item, first)
+template <class Fn>
+__device__ __forceinline__ void for_items(const Shape &sh, int ph, int b, Fn fn) {
+  const int span = ph_span(sh, ph);
+  bool first = true;
+  for (int it = b - ph_off(sh, ph); it < span; it += sh.G) {
+    It d;
+    if (it < 0 || !ph_item(sh, ph, it, d)) continue;
+    fn(d, first);
+    first = false;
+  }
+}
+__device__ __forceinline__ AttnArgs attn_args(const Args &a, int l) {
+  const Bufs cur = layer_bufs(a, l);
+  return AttnArgs{a.B, a.S, a.scale, cur.qkv, a.mask, cur.ctx, a.probs};
+}
+
+// ------------------------------------------------------------------ fused kernel ----
+template <int NKT>
+__global__ void __launch_bounds__(256) k_encoder_small(Args args) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const Shape sh{args.B, args.S, args.M, args.M / 32, (int)gridDim.x};
+  Sync sy;
+  sync_begin(sy, args.flags, args.ctl + kCtlErrWord, args.trace, args.trace_cap);
+  const int L = args.num_layers;
+  // Who feeds whom (wave 0: 4 workgroups per lane, one nibble per phase) and in which phases this workgroup
+  // has items (one bit per phase); packed into words so that the phase loop indexes no register array.
+  unsigned wm_all = 0, mine_bits = 0;
+  for (int ph = 0; ph <= PH_FIN; ++ph) {
+    if (tid < 64) wm_all |= wait_mask(sh, ph, b, tid) << (4 * ph);
+    mine_bits |= (has_items(sh, ph, b) ? 1u : 0u) << ph;
+  }
+  auto mine = [&](int ph) { return ((mine_bits >> ph) & 1u) != 0; };
+  auto wm = [&](int ph) { return (wm_all >> (4 * ph)) & 15u; };
+  // Weight slices are fetched one GEMM phase ahead, as soon as the W region of the LDS is free: pf names the
+  // (layer, phase) whose first item's slice has been requested, -1 = none.
+  int pf = -1;
+  auto prefetch_after = [&](int l, int ph) {
+    for (int step = 1; step <= 6; ++step) {
+      const int q = ph + step, ll = l + q / 6, pp = q % 6;
+      if (ll >= L) return;
+      if (pp == PH_ATT) { if (mine(PH_ATT)) return; continue; }    // the attention tiles overlap the W region
+      if (pp == PH_RED || !mine(pp)) continue;
+      for_items(sh, pp, b, [&](const It &d, bool first) { if (first) issue_weights(lds, make_job(args, ll, pp, d)); });
+      pf = ll * 8 + pp;
+      return;
+    }
+  };
+  int l = 0, ph = -1;          // (the request in front of the first phase shares the call below)
+#pragma unroll 1
+  for (;;) {
+    if (pf < 0) prefetch_after(l, ph);
+    // next phase
+    if (++ph > PH_RED) { ph = PH_QKV; if (++l >= L) break; }
+    if (!mine(ph)) continue;
+    if (ph == PH_RED) {
+      bool waited = false;
+      for_items(sh, PH_RED, b, [&](const It &d, bool) {
+        run_red_item(args, l, d, [&]() {
+          if (!waited) await(sy, wm(PH_RED), phase_seq(sy, l, PH_FC2));
+          waited = true;
+        });
+      });
+    } else {
+      if (l > 0 || ph > PH_QKV) await(sy, wm(ph), phase_seq(sy, ph == PH_QKV ? l - 1 : l, producer_phase(ph)));
+      if (ph == PH_ATT) {
+        const AttnArgs aa = attn_args(args, l);
+        for_items(sh, ph, b, [&](const It &d, bool) { attn_item_split<NKT>(lds, aa, d.b, d.a); });
+      } else {
+        const bool ready = pf == l * 8 + ph;
+        pf = -1;
+        for_items(sh, ph, b, [&](const It &d, bool first) {
+          if (!first) __syncthreads();                        // the partial tiles of the previous item have been read
+          run_gemm_item(lds, args, l, ph, d, first && ready);
+        });
+      }
+    }
+    publish(sy, phase_seq(sy, l, ph));
+    if (ph == PH_ATT) __syncthreads();                        // every wave is done with the attention tiles
+  }
+  if (mine(PH_FIN)) {
+    await(sy, wm(PH_FIN), phase_seq(sy, L - 1, PH_RED));
+    for_items(sh, PH_FIN, b, [&](const It &d, bool) { run_fin_item(args, d); });
+  }
+  sync_end(sy, L);
+}
+
+// ------------------------------------------------------------------ per-op kernels ----
+// The same items as separate launches (the unfused baseline): one kernel per phase and layer.
+template <int NKT>
+__global__ void __launch_bounds__(256) k_small_phase(Args args, int l, int ph) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int b = blockIdx.x;
+  const Shape sh{args.B, args.S, args.M, args.M / 32, (int)gridDim.x};
+  if (ph == PH_ATT) {
+    const AttnArgs aa = attn_args(args, l);
+    for_items(sh, ph, b, [&](const It &d, bool) { attn_item_split<NKT>(lds, aa, d.b, d.a); });
+  } else if (ph == PH_RED) {
+    for_items(sh, ph, b, [&](const It &d, bool) { run_red_item(args, l, d, []() {}); });
+  } else if (ph == PH_FIN) {
+    for_items(sh, ph, b, [&](const It &d, bool) { run_fin_item(args, d); });
+  } else {
+    for_items(sh, ph, b, [&](const It &d, bool first) {
+      if (!first) __syncthreads();
+      run_gemm_item(lds, args, l, ph, d, false);
+    });
+  }
+}
+
+}  // namespace sk
+}  // namespace bert
+}  // namespace souffle

@@ -220,14 +220,11 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 //                 rewritten by grid_barrier_end() (all workgroups read them before their first
 //                 arrival, nobody writes them before the last barrier of the launch has completed)
 //   [kCtlErrWord] sticky error flag for kernels with bounded spin loops (bit 0: LSTM wait,
-//                 bit 1: grid barrier, bit 2: dataflow wait of the encoder)
-//   [kCtlFlowWord] layout marker of the dataflow encoder kernel: non-zero while every inter-stage
-//                 buffer of that layout holds the "not written yet" pattern
+//                 bit 1: grid barrier or hand-over of the encoder)
 // Data exchanged across a barrier must be written with st*<true> (write-through); the barrier
 // itself carries no cache write-back or invalidate.
 constexpr int kCtlWords = 512;
 constexpr int kCtlErrWord = 400;
-constexpr int kCtlFlowWord = 401;
 constexpr int kMaxBarrierSpin = 1 << 20;       // about a second of polling; a barrier normally completes in microseconds
 
 struct GridBarrier {

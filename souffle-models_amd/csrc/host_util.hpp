@@ -26,9 +26,6 @@ int device_facts(DeviceFacts *out);
 // 1: the Swin block pair runs four workgroups per window (souffle_set_swin_split / SOUFFLE_SWIN_SPLIT).
 int swin_split_mode();
 
-// SOUFFLE_SYNC_* selected by souffle_set_bert_sync / SOUFFLE_BERT_SYNC.
-int bert_sync_mode();
-
 // Process-wide stage-trace buffer set by souffle_set_stage_trace (NULL = tracing off).
 void stage_trace(unsigned long long **buf, int *max_barriers, int nblk);
 

@@ -83,7 +83,6 @@ SIGNATURES = {
     "souffle_set_cooperative_launch": (C.c_int, [C.c_int]),
     "souffle_workspace_init": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "souffle_workspace_status": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_uint), C.c_int]),
-    "souffle_set_bert_sync": (C.c_int, [C.c_int]),
     "souffle_bert_workspace_bytes": (C.c_size_t, [C.POINTER(BertCfg)]),
     "souffle_bert_layer_fused": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
                                            C.c_void_p, C.POINTER(BertDump), C.c_void_p, C.c_size_t, C.c_void_p]),
@@ -194,15 +193,6 @@ def set_stage_trace(tensor):
         check(lib().souffle_set_stage_trace(None, 0))
     else:
         check(lib().souffle_set_stage_trace(tensor.data_ptr(), tensor.numel() * tensor.element_size()))
-
-
-SYNC_DATAFLOW, SYNC_BARRIER = 0, 1
-
-
-def set_bert_sync(mode):
-    """Hand-over between the stages of the skinny fused encoder: "barrier" (default) or "dataflow"."""
-    modes = {"dataflow": SYNC_DATAFLOW, "barrier": SYNC_BARRIER, SYNC_DATAFLOW: SYNC_DATAFLOW, SYNC_BARRIER: SYNC_BARRIER}
-    check(lib().souffle_set_bert_sync(modes[mode]))
 
 
 def set_swin_split(on):

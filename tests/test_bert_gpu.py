@@ -168,30 +168,79 @@ def test_many_rows_encoder_in_a_workspace_of_unknown_content():
     assert torch.equal(y_a, y_u) and torch.equal(y_b, y_u)
 
 
-@pytest.mark.parametrize("B,S,layers", [(1, 128, 12), (1, 384, 2), (2, 64, 3), (1, 128, 1)])
-def test_dataflow_sync_equals_barrier_sync(B, S, layers):
-    """The dataflow hand-over (consumers poll the data) runs the same arithmetic as the grid-barrier
-    one: bit-identical results, also on a second launch (buffers put back into the unwritten state by
-    the first) and after the per-op chain has left data in the shared workspace."""
-    announce("bert encoder dataflow sync B=%d S=%d L=%d" % (B, S, layers))
+@pytest.mark.parametrize("B,S,layers", [(1, 128, 12), (1, 384, 2), (2, 64, 3), (1, 128, 1), (3, 256, 2)])
+def test_few_rows_handovers_on_repeated_launches(B, S, layers):
+    """The flag hand-overs of the few-rows encoder: launch after launch on one workspace, with another input
+    in between (a value that survived from an earlier launch, in a cache or in a flag word, would show), fused
+    and per-op launches give the same bits, all LayerNorm vectors and biases present, and no bounded wait gives up."""
+    announce("bert encoder few rows, repeated launches B=%d S=%d L=%d" % (B, S, layers))
+    import bert_binding
+    ws = [synth.bert_layer_weights(2, l, with_bias=True) for l in range(layers)]
+    x0, x1 = synth.bert_input(2, B, S), synth.bert_input(3, B, S)
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    y_u = enc(dev(x0), fused=False).clone()
+    y_1 = enc(dev(x0)).clone()
+    z_1 = enc(dev(x1)).clone()
+    y_2 = enc(dev(x0)).clone()
+    z_u = enc(dev(x1), fused=False).clone()
+    y_3 = enc(dev(x0)).clone()
+    flags = enc.ws.status()
+    assert flags == 0, "a bounded wait gave up (flags %d)" % flags
+    assert torch.equal(y_1, y_u) and torch.equal(y_2, y_u) and torch.equal(y_3, y_u) and torch.equal(z_1, z_u)
+    assert_close("encoder x0", y_1, oracle.bert_encoder(x0, ws, B, S))
+    assert_close("encoder x1", z_1, oracle.bert_encoder(x1, ws, B, S))
+
+
+def test_layernorm_of_rows_far_from_zero():
+    """Rows whose mean is far larger than their spread, and feature columns of large magnitude: the LayerNorm
+    statistics (per-slice mean and squared deviations, combined pairwise) and the normalisation in the operand
+    registers must not lose the spread to cancellation.  Checked against the oracle on the few-rows path, at both
+    places where a LayerNorm is applied on load (LN1 inside FC1, LN2 inside the next layer's QKV and at the end)."""
+    announce("bert encoder few rows, rows with a large mean")
+    import bert_binding
+    B, S, layers = 1, 128, 2
+    ws = [synth.bert_layer_weights(2, l, with_bias=True) for l in range(layers)]
+    x = synth.bert_input(5, B, S)
+    # The biases of both sublayers carry the offsets, so that the pre-LayerNorm sums (not the attention inputs,
+    # whose fp16 rounding a near one-hot softmax would amplify) are what is far from zero: every row of z1 has
+    # mean 25 and two columns of magnitude 300, every row of z2 mean -30 and a column of magnitude 1000.
+    for w in ws:
+        b1 = w["attn_fc_bias"].astype(np.float32) + 25.0
+        b1[17] += 300.0
+        b1[500] -= 250.0
+        w["attn_fc_bias"] = b1.astype(np.float16)
+        b2 = w["fc2_bias"].astype(np.float32) - 30.0
+        b2[3] += 1000.0
+        w["fc2_bias"] = b2.astype(np.float16)
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    y_f = enc(dev(x))
+    y_u = enc(dev(x), fused=False)
+    assert enc.ws.status() == 0
+    assert torch.equal(y_f, y_u)
+    assert_close("encoder, rows far from zero", y_f, oracle.bert_encoder(x, ws, B, S))
+
+
+def test_cooperative_launch_matches_oracle():
+    """The persistent encoder launched with hipLaunchCooperativeKernel (the runtime's co-residency guarantee)
+    instead of the plain launch: same results, checked against the oracle."""
+    announce("bert encoder, cooperative launch")
     import bert_binding
     import souffle_hip as sh
+    B, S, layers = 1, 128, 3
     ws = [synth.bert_layer_weights(2, l) for l in range(layers)]
-    x = dev(synth.bert_input(2, B, S))
+    x = synth.bert_input(2, B, S)
     enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
-    y_b = enc(x).clone()
-    sh.set_bert_sync("dataflow")
+    y_plain = enc(dev(x)).clone()
+    sh.set_cooperative_launch(True)
     try:
-        y_1 = enc(x).clone()
-        y_2 = enc(x).clone()
-        y_u = enc(x, fused=False).clone()
-        y_3 = enc(x).clone()
+        y_coop = enc(dev(x)).clone()
+        y_coop2 = enc(dev(x)).clone()
         flags = enc.ws.status()
     finally:
-        sh.set_bert_sync("barrier")
-    assert flags == 0, "a bounded wait gave up (flags %d)" % flags
-    assert torch.equal(y_1, y_b) and torch.equal(y_2, y_b) and torch.equal(y_3, y_b) and torch.equal(y_u, y_b)
-    assert_close("encoder dataflow", y_1, oracle.bert_encoder(synth.bert_input(2, B, S), ws, B, S))
+        sh.set_cooperative_launch(False)
+    assert flags == 0
+    assert torch.equal(y_coop, y_plain) and torch.equal(y_coop2, y_plain)
+    assert_close("encoder cooperative", y_coop, oracle.bert_encoder(x, ws, B, S))
 
 
 @pytest.mark.parametrize("B,S,layers,masked", [(1, 100, 2, False), (2, 77, 1, True), (1, 200, 1, False), (3, 5, 1, False)])
