@@ -69,9 +69,18 @@ struct Sync {
   unsigned *err;         // sticky failure word of the control block
   unsigned base;         // flag value of (layer l, phase p) = base + 1 + l * PH_SLOTS + p
   bool failed;
-  unsigned long long *trace;   // optional: entry to / exit from every wait, trace[(2 i + {0,1}) * G + block]
-  int trace_cap, trace_idx;
+  // optional stamps of the 100 MHz clock, slot i = layer * PH_SLOTS + phase: trace[(2 i + {0,1}) * G + block] = entry to /
+  // exit from the wait in front of the phase, trace[(2 cap + 8 i + id) * G + block] = marks inside it (0 operands of the
+  // first k-step there, 1 MFMAs done, 2 stores issued, 3 published)
+  unsigned long long *trace;
+  int trace_cap;
 };
+__device__ __forceinline__ void stamp_wait(const Sync &sy, int slot, int which) {
+  if (sy.trace && slot < sy.trace_cap && threadIdx.x == 0) sy.trace[(size_t)(2 * slot + which) * gridDim.x + blockIdx.x] = wall_clock64();
+}
+__device__ __forceinline__ void stamp_mark(const Sync &sy, int slot, int id) {
+  if (sy.trace && slot < sy.trace_cap && threadIdx.x == 0) sy.trace[(size_t)(2 * sy.trace_cap + 8 * slot + id) * gridDim.x + blockIdx.x] = wall_clock64();
+}
 
 __device__ __forceinline__ unsigned phase_seq(const Sync &s, int l, int ph) { return s.base + 1u + (unsigned)(l * PH_SLOTS + ph); }
 
@@ -140,32 +149,18 @@ __device__ __forceinline__ bool feeds(const Shape &s, int cph, const It &c, cons
 }
 __device__ __forceinline__ int producer_phase(int cph) { return cph == PH_QKV ? PH_RED : cph == PH_FIN ? PH_RED : cph - 1; }
 
-// Which of the workgroups 4 lane .. 4 lane + 3 must have published the producer phase before this workgroup may
-// start its items of phase cph (4 bits).  Exact where both phases are a single pass over the grid; otherwise every
-// workgroup that has an item of the producer phase.
-__device__ unsigned wait_mask(const Shape &s, int cph, int b, int lane) {
+// Must workgroup pb have published the producer phase before workgroup b may start its items of phase cph?
+// Exact where both phases are a single pass over the grid; otherwise every workgroup that has an item of the
+// producer phase.
+__device__ bool wait_needs(const Shape &s, int cph, int b, int pb) {
   const int pph = producer_phase(cph);
   const bool fine = ph_span(s, pph) + ph_off(s, pph) <= s.G && ph_span(s, cph) + ph_off(s, cph) <= s.G;
-  It c{0, 0};
-  bool mine = false;
-  if (fine) {
-    const int cit = b - ph_off(s, cph);
-    mine = cit >= 0 && cit < ph_span(s, cph) && ph_item(s, cph, cit, c);
-  } else mine = has_items(s, cph, b);
-  unsigned m = 0;
-  if (!mine) return 0;
-  for (int t = 0; t < 4; ++t) {
-    const int pb = 4 * lane + t;
-    if (pb >= s.G) break;
-    bool need;
-    if (fine) {
-      It p;
-      const int pit = pb - ph_off(s, pph);
-      need = pit >= 0 && pit < ph_span(s, pph) && ph_item(s, pph, pit, p) && feeds(s, cph, c, p);
-    } else need = has_items(s, pph, pb);
-    m |= (need ? 1u : 0u) << t;
-  }
-  return m;
+  if (pb >= s.G) return false;
+  if (!fine) return has_items(s, cph, b) && has_items(s, pph, pb);
+  It c, p;
+  const int cit = b - ph_off(s, cph), pit = pb - ph_off(s, pph);
+  if (!(cit >= 0 && cit < ph_span(s, cph) && ph_item(s, cph, cit, c))) return false;
+  return pit >= 0 && pit < ph_span(s, pph) && ph_item(s, pph, pit, p) && feeds(s, cph, c, p);
 }
 
 // ---- hand-over ----
@@ -175,7 +170,6 @@ __device__ __forceinline__ void sync_begin(Sync &sy, unsigned *flags, unsigned *
   sy.failed = false;
   sy.trace = trace;
   sy.trace_cap = trace_cap;
-  sy.trace_idx = 0;
   sy.base = __hip_atomic_load(flags + kFlagBaseWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 // Every workgroup of the launch calls this last.  The one that ends last moves the base past every value this
@@ -199,9 +193,8 @@ __device__ __forceinline__ void publish(const Sync &sy, unsigned seq) {
 }
 // Wait until the workgroups named by `mask` (wave 0: 4 bits per lane) have published `seq` or something later.
 // Bounded: a wait that gives up flags the control block and ends all waiting of the launch.
-__device__ __forceinline__ void await(Sync &sy, unsigned mask, unsigned seq) {
-  const bool tr = sy.trace && sy.trace_idx < sy.trace_cap && threadIdx.x == 0;
-  if (tr) sy.trace[(size_t)(2 * sy.trace_idx) * gridDim.x + blockIdx.x] = wall_clock64();
+__device__ __forceinline__ void await(Sync &sy, unsigned mask, unsigned seq, int slot) {
+  stamp_wait(sy, slot, 0);
   if (threadIdx.x < 64 && !sy.failed) {
     const unsigned *copy = sy.flags + (blockIdx.x & (kFlagCopies - 1)) * kFlagStride;
     for (int spin = 0;; ++spin) {
@@ -217,10 +210,45 @@ __device__ __forceinline__ void await(Sync &sy, unsigned mask, unsigned seq) {
       }
     }
   }
-  if (tr) sy.trace[(size_t)(2 * sy.trace_idx + 1) * gridDim.x + blockIdx.x] = wall_clock64();
-  sy.trace_idx++;
+  stamp_wait(sy, slot, 1);
+  if (threadIdx.x >= 64) wait_vmcnt<0>();         // a weight slice requested ahead (issue_w_ahead) has landed: wave 0 may read its part
+#ifdef SOUFFLE_STAGE_MARKS
+  if (sy.trace && slot < sy.trace_cap && threadIdx.x == 64) sy.trace[(size_t)(2 * sy.trace_cap + 8 * slot + 5) * gridDim.x + blockIdx.x] = wall_clock64();
+#endif
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+}
+
+// Sums over groups of neighbouring lanes with DPP moves (a few cycles each; a shuffle through the LDS crossbar
+// costs a round trip of a hundred): after the call every lane of the group holds the group's sum.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float sum4(float v) {            // the four lanes of a quad
+  v += dpp_move<0xB1>(v);                                   // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E>(v);                                   // quad_perm [2,3,0,1]
+  return v;
+}
+__device__ __forceinline__ float sum8(float v) {            // 8 consecutive lanes
+  v = sum4(v);
+  v += dpp_move<0x141>(v);                                  // row_half_mirror: lane i <- lane 7 - i, the other quad
+  return v;
+}
+__device__ __forceinline__ float sum16(float v) {           // the 16 lanes of a row
+  v = sum8(v);
+  v += dpp_move<0x128>(v);                                  // row_ror:8: lane i <- lane (i + 8) % 16
+  return v;
+}
+__device__ __forceinline__ float sum32(float v) {           // 32 consecutive lanes (two rows)
+  v = sum16(v);
+  v += wave_xor(v, 16);
+  return v;
+}
+template <int LANES>
+__device__ __forceinline__ float sum_lanes(float v) {
+  static_assert(LANES == 8 || LANES == 32, "group sizes in use");
+  if constexpr (LANES == 8) return sum8(v); else return sum32(v);
 }
 
 // ---- row statistics ----
@@ -236,12 +264,11 @@ __device__ __forceinline__ RowStat row_stat8(const float *st, int m, int t8, flo
   if (t8 < 4) p1 = ld8<true>(st, (m * 12 + 8 + t8) * 8);
   const float m0 = f32_of(p0[0]), q0 = f32_of(p0[1]);
   const float m1 = f32_of(p1[0]), q1 = f32_of(p1[1]);
-  float s = m0 + (t8 < 4 ? m1 : 0.f);
-  s += wave_xor(s, 1); s += wave_xor(s, 2); s += wave_xor(s, 4);
+  const float s = sum8(m0 + (t8 < 4 ? m1 : 0.f));
   const float mean = s * (1.0f / 12.0f);
   float q = q0 + 64.0f * (m0 - mean) * (m0 - mean);
   if (t8 < 4) q += q1 + 64.0f * (m1 - mean) * (m1 - mean);
-  q += wave_xor(q, 1); q += wave_xor(q, 2); q += wave_xor(q, 4);
+  q = sum8(q);
   return RowStat{mean, rsqrtf(q * (1.0f / 768.0f) + eps)};
 }
 // Publish the statistics of 64 values of a row held by `n` consecutive lanes (v: this lane's values, already
@@ -252,72 +279,90 @@ __device__ __forceinline__ void put_stat(float *st, int m, int slice, const floa
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < PER; ++i) s += v[i];
-#pragma unroll
-  for (int k = 1; k < LANES; k <<= 1) s += wave_xor(s, k);
+  s = sum_lanes<LANES>(s);
   const float mean = s * (1.0f / 64.0f);
   float q = 0.f;
 #pragma unroll
   for (int i = 0; i < PER; ++i) { const float d = v[i] - mean; q += d * d; }
-#pragma unroll
-  for (int k = 1; k < LANES; k <<= 1) q += wave_xor(q, k);
+  q = sum_lanes<LANES>(q);
   if (lane_in_group == 0) st8<true>(st, (m * 12 + slice) * 8, u2{u32_of(mean), u32_of(q)});
 }
 
 // ---- GEMM item: 32 rows x 64 columns over a K slice of 768 ----
-// Wave w owns the K quarter [192 w, 192 w + 192): it loads exactly the operand bytes it multiplies, so nothing
-// but its own loads stands between a wave and its MFMAs, and a k-step starts as soon as its two X blocks are
-// there.  X blocks are stored in operand order (block (s, i): lane L's 16 bytes are X[16 i + L % 16][32 s + 8 (L / 16) ..]),
-// W rows as [k][64] with the 16-byte slot index XORed with (k & 2) for the transposing read.
+// Wave w multiplies the K quarter [192 w, 192 w + 192), three pairs of k-steps (a pair = 64 columns of X = one
+// 128-byte line per row).  Every wave-wide load asks for whole lines: 8 rows x 128 bytes, the eight lanes of a row
+// next to each other (requests for half lines moved half the bytes in the same time: what limits a CU's intake from
+// beyond its L2 is the number of requests in flight).  X block (c, h) = rows 8 h .. 8 h + 7 of pair c, its 16-byte slots
+// XORed with (row >> 1) & 7 for the 16-row operand read; W rows [k][64] with the slot index XORed with (k & 2) for
+// the transposing read.  A wave starts a pair as soon as its four X blocks are there.
 struct GemmItem {
   const half_t *X; int ldx, kx0;      // activation rows start at column kx0
   const half_t *W; int ldw, kw0, n0;  // weight rows kw0 .. kw0 + 767, columns n0 .. n0 + 63
   int m0;
+  int rot;                            // a wave takes the three pairs of its quarter in the order rot, rot + 1, ... (mod 3)
 };
+// The workgroups of an XCD that share an operand (the m-tiles of a weight slice, the slices of an m-tile) start at
+// different pairs, so that each of them is the first to ask for another part and finds the rest in the L2.
+__device__ __forceinline__ int pair_of(int i, int rot) { const int t = i + rot; return t >= 3 ? t - 3 : t; }
 
+// The eight wave-wide loads of rows [64 c, 64 c + 64) of K quarter `quarter` (pair c of that quarter).
+__device__ __forceinline__ void issue_w_pair(unsigned char *lds, const GemmItem &g, int quarter, int c, int lane) {
+  const half_t *sb = uniform_ptr(g.W + (size_t)(g.kw0 + 192 * quarter + 64 * c) * g.ldw + g.n0);
+  const int rl = lane >> 3;
+  const unsigned voff = (unsigned)(rl * g.ldw * 2 + (((lane & 7) ^ (rl & 2)) * 16));
+  const unsigned step = (unsigned)(8 * g.ldw * 2);
+  const unsigned base = uni(lds_address(lds) + kWOff + (24 * quarter + 8 * c) * 1024);
+#pragma unroll
+  for (int u = 0; u < 8; ++u) dma16<false>(sb, voff + (unsigned)u * step, base + u * 1024);
+}
+// Every wave its own quarter (24 loads), in the order of its pairs.
 __device__ __forceinline__ void issue_w(unsigned char *lds, const GemmItem &g) {
   const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
-  const half_t *sb = uniform_ptr(g.W + (size_t)(g.kw0 + 192 * w) * g.ldw + g.n0);
-  const int rl = lane >> 3;
-  unsigned voff = (unsigned)(rl * g.ldw * 2 + (((lane & 7) ^ (rl & 2)) * 16));
-  const unsigned step = (unsigned)(8 * g.ldw * 2);
-  const unsigned base = uni(lds_address(lds) + kWOff + 24 * 1024 * w);
 #pragma unroll
-  for (int q = 0; q < 24; ++q) {
-    dma16<false>(sb, voff, base + q * 1024);
-    voff += step;
-  }
+  for (int i = 0; i < 3; ++i) issue_w_pair(lds, g, w, pair_of(i, g.rot), lane);
 }
-// gamma and beta of the LayerNorm applied on load: every wave fetches the 192 values of its own K quarter
-// (wave w: [gamma quarter 384 B][beta quarter 384 B] at kGamOff + 768 w; a missing vector is written as ones /
-// zeros), so that like its operands they are its own loads.  The bias of the item's 64 columns is fetched by wave 3.
-__device__ __forceinline__ void issue_params(unsigned char *lds, const half_t *gam, const half_t *bet, bool ln_affine,
-                                             const half_t *bias, int n0) {
+// The same slice requested ahead of time by waves 1..3 alone (32 loads each: their own quarter and one pair of
+// wave 0's): wave 0 polls the flag words meanwhile, and a wave that issues loads faster than they are served is
+// held at the load instruction.  Wave 0 may read its quarter once waves 1..3 have seen their loads land (await).
+__device__ __forceinline__ void issue_w_ahead(unsigned char *lds, const GemmItem &g) {
   const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
-  if (ln_affine) {
-    unsigned char *dst = lds + kGamOff + 768 * w;
-    if (lane < 24) {
-      if (gam) dma16<false>(uniform_ptr(gam + 192 * w), (unsigned)lane * 16, uni(lds_address(dst)));
+  if (w == 0) return;
+#pragma unroll
+  for (int i = 0; i < 3; ++i) issue_w_pair(lds, g, w, pair_of(i, g.rot), lane);
+  issue_w_pair(lds, g, 0, w - 1, lane);
+}
+// gamma and beta of the LayerNorm applied on load, per K quarter q: [gamma quarter 384 B][beta quarter 384 B] at
+// kGamOff + 768 q (a missing vector is written as ones / zeros).  Fetched by the wave that multiplies the quarter, or
+// (ahead = true) quarter 0 by wave 1.  The bias of the item's 64 columns is fetched by wave 3.
+__device__ __forceinline__ void issue_params(unsigned char *lds, const half_t *gam, const half_t *bet, bool ln_affine,
+                                             const half_t *bias, int n0, bool ahead) {
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
+  if (ln_affine && lane < 24 && !(ahead && w == 0)) {
+    for (int q = (ahead && w == 1) ? 0 : w; q <= w; ++q) {
+      unsigned char *dst = lds + kGamOff + 768 * q;
+      if (gam) dma16<false>(uniform_ptr(gam + 192 * q), (unsigned)lane * 16, uni(lds_address(lds) + kGamOff + 768 * q));
       else { const half_t c = (half_t)1.0f; *reinterpret_cast<h8 *>(dst + lane * 16) = h8{c, c, c, c, c, c, c, c}; }
-      if (bet) dma16<false>(uniform_ptr(bet + 192 * w), (unsigned)lane * 16, uni(lds_address(dst + 384)));
+      if (bet) dma16<false>(uniform_ptr(bet + 192 * q), (unsigned)lane * 16, uni(lds_address(lds) + kGamOff + 768 * q + 384));
       else { const half_t c = (half_t)0.0f; *reinterpret_cast<h8 *>(dst + 384 + lane * 16) = h8{c, c, c, c, c, c, c, c}; }
     }
   }
   if (bias && w == 3 && lane < 8) dma16<false>(uniform_ptr(bias + n0), (unsigned)lane * 16, uni(lds_address(lds) + kBiasOff));
 }
-// this wave's twelve X blocks, in k-step order
+// this wave's twelve X blocks, pair after pair
 template <bool SC1>
 __device__ __forceinline__ void issue_x(unsigned char *lds, const GemmItem &g) {
-  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6, l16 = lane & 15, gq = lane >> 4;
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
   const half_t *sb = uniform_ptr(g.X + (size_t)g.m0 * g.ldx + g.kx0 + 192 * w);
-  unsigned v0 = (unsigned)((l16 * g.ldx + gq * 8) * 2);
-  unsigned v1 = v0 + (unsigned)(16 * g.ldx * 2);
+  const int rl = lane >> 3;                                          // row within a block; (8 h + rl) >> 1 & 7 = 4 (h & 1) + (rl >> 1)
   const unsigned base = uni(lds_address(lds) + kXPart * w);
 #pragma unroll
-  for (int s = 0; s < 6; ++s) {
-    dma16<SC1>(sb, v0, base + (2 * s) * 1024);
-    dma16<SC1>(sb, v1, base + (2 * s + 1) * 1024);
-    v0 += 64;
-    v1 += 64;
+  for (int i = 0; i < 3; ++i) {
+    const int c = pair_of(i, g.rot);
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      const int slot = (lane & 7) ^ (4 * (h & 1) + (rl >> 1));
+      dma16<SC1>(sb, (unsigned)(((8 * h + rl) * g.ldx + 64 * c + 8 * slot) * 2), uni(base + (4 * c + h) * 1024));
+    }
   }
 }
 // the statistics of rows m0 .. m0 + 31 (3 KB, contiguous), one copy per wave (COPIES = 4) or one for the workgroup
@@ -346,20 +391,21 @@ __device__ __forceinline__ void static_for(F f) {
   }
 }
 
-// The operand registers of one k-step.
+// The operand registers of one k-step (s = 2 pair + parity).
 struct KOps { h8 x[2], w[4]; };
 __device__ __forceinline__ void read_ops(const unsigned char *lds, int w, int lane, int s, KOps &o) {
-  const int l16 = lane & 15, gq = lane >> 4;
-  const unsigned char *xb = lds + kXPart * w + (2 * s) * 1024 + lane * 16;
+  const int l16 = lane & 15, gq = lane >> 4, c = s >> 1, p = s & 1;
+  // row 16 i + l16 of pair c: block (c, 2 i + l16 / 8), row l16 % 8 of it, slot (4 p + gq) ^ ((l16 >> 1) & 7)
+  const unsigned char *xb = lds + kXPart * w + (4 * c + (l16 >> 3)) * 1024 + (l16 & 7) * 128 + (((4 * p + gq) ^ ((l16 >> 1) & 7)) * 16);
   o.x[0] = *reinterpret_cast<const h8 *>(xb);
-  o.x[1] = *reinterpret_cast<const h8 *>(xb + 1024);
+  o.x[1] = *reinterpret_cast<const h8 *>(xb + 2048);
   const half_t *ws = reinterpret_cast<const half_t *>(lds + kWOff);
   const int k = 192 * w + 32 * s + gq * 8 + (l16 >> 2);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int c = j * 2 + ((l16 & 3) >> 1);
-    const half_t *p = ws + (k * 8 + (c ^ (k & 2))) * 8 + (l16 & 1) * 4;
-    const h4 lo = lds_read_tr16(p), hi = lds_read_tr16(p + 4 * 64);
+    const int cc = j * 2 + ((l16 & 3) >> 1);
+    const half_t *pp = ws + (k * 8 + (cc ^ (k & 2))) * 8 + (l16 & 1) * 4;
+    const h4 lo = lds_read_tr16(pp), hi = lds_read_tr16(pp + 4 * 64);
     o.w[j] = h8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   }
 }
@@ -369,7 +415,7 @@ __device__ __forceinline__ void read_ops(const unsigned char *lds, int w, int la
 // fp16 part of the mean is subtracted first (a difference of neighbouring values, rounded relative to itself), what
 // rounding the mean to fp16 left over enters through the addend of the multiply-add, so that it does not shift the row.
 template <int LN>
-__device__ __forceinline__ void mfma_quarter(const unsigned char *lds, f4 (&acc)[2][4], float eps) {
+__device__ __forceinline__ void mfma_quarter(const unsigned char *lds, f4 (&acc)[2][4], float eps, int rot) {
   const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6, l16 = lane & 15, gq = lane >> 4;
   h8 nmh[2], off[2], rs[2];     // -mean (its fp16 part), -(mean - that part) * rstd, rstd
   if constexpr (LN != LN_NONE) {
@@ -386,12 +432,12 @@ __device__ __forceinline__ void mfma_quarter(const unsigned char *lds, f4 (&acc)
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < 6; ++i) s += mi[i];
-    s += wave_xor(s, 1);
+    s += dpp_move<0xB1>(s);             // the partner lane (quad_perm [1,0,3,2])
     const float mean = s * (1.0f / 12.0f);
     float q = 0.f;
 #pragma unroll
     for (int i = 0; i < 6; ++i) q += qi[i] + 64.0f * (mi[i] - mean) * (mi[i] - mean);
-    q += wave_xor(q, 1);
+    q += dpp_move<0xB1>(q);
     const float rstd = rsqrtf(q * (1.0f / 768.0f) + eps);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -407,25 +453,26 @@ __device__ __forceinline__ void mfma_quarter(const unsigned char *lds, f4 (&acc)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
   KOps cur, nxt;
-  wait_vmcnt<10>();
-  read_ops(lds, w, lane, 0, cur);
+  wait_vmcnt<8>();                                      // the four X blocks of the first pair
+  read_ops(lds, w, lane, 2 * pair_of(0, rot), cur);
   static_for<0, 6>([&](auto sc) {
-    constexpr int s = decltype(sc)::value;
+    constexpr int s = decltype(sc)::value;               // turn s multiplies k-step 2 pair_of(s / 2) + s % 2
+    [[maybe_unused]] const int t = 2 * pair_of(s / 2, rot) + (s & 1);
     if constexpr (s + 1 < 6) {
-      wait_vmcnt<10 - 2 * (s + 1)>();
-      read_ops(lds, w, lane, s + 1, nxt);
+      if constexpr ((s & 1) == 1) wait_vmcnt<8 - 4 * ((s + 1) / 2)>();     // the next pair's blocks
+      read_ops(lds, w, lane, 2 * pair_of((s + 1) / 2, rot) + ((s + 1) & 1), nxt);
     }
     if constexpr (LN != LN_NONE) {
       h8 gm, bt;
       if constexpr (LN == LN_AFFINE) {
-        gm = *reinterpret_cast<const h8 *>(lds + kGamOff + 768 * w + (32 * s + 8 * gq) * 2);
-        bt = *reinterpret_cast<const h8 *>(lds + kGamOff + 768 * w + 384 + (32 * s + 8 * gq) * 2);
+        gm = *reinterpret_cast<const h8 *>(lds + kGamOff + 768 * w + (32 * t + 8 * gq) * 2);
+        bt = *reinterpret_cast<const h8 *>(lds + kGamOff + 768 * w + 384 + (32 * t + 8 * gq) * 2);
       }
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        h8 t = (cur.x[i] + nmh[i]) * rs[i] + off[i];     // (x - mean) * rstd: the first difference is all but exact
-        if constexpr (LN == LN_AFFINE) t = t * gm + bt;
-        cur.x[i] = t;
+        h8 y = (cur.x[i] + nmh[i]) * rs[i] + off[i];     // (x - mean) * rstd: the first difference is all but exact
+        if constexpr (LN == LN_AFFINE) y = y * gm + bt;
+        cur.x[i] = y;
       }
     }
 #pragma unroll
@@ -617,7 +664,7 @@ __device__ __forceinline__ Bufs layer_bufs(const Args &a, int l) {
   return Bufs{adv(a.qkv), adv(a.ctx), adv(a.z1), adv(a.h), adv(a.z2), adv(a.st1), adv(a.st2), adv(a.part)};
 }
 
-// What a GEMM item of (layer l, phase ph) multiplies, and what travels with its weight slice.
+// What a GEMM item of (layer l, phase ph) multiplies, what travels with its weight slice, and where its results go.
 struct Job {
   GemmItem g;
   int ln;                              // LN_* applied to X on load
@@ -625,17 +672,25 @@ struct Job {
   const half_t *gam, *bet;             // of that LayerNorm
   const half_t *bias;                  // of the item's columns (LDS copy at kBiasOff), or null
   const half_t *rgam, *rbet;           // OUT: gamma / beta of the LayerNorm that produces the residual (LDS copies), or null
+  const half_t *res;                   // OUT: the residual rows [M][768] before that LayerNorm
+  const float *rstats;                 // OUT: their statistics, null = the residual is taken as it is (layer 0)
+  half_t *out;                         // qkv / z1 / h of the layer
+  float *aux;                          // OUT: st1; FC2: the partial sums
+  int which, head;                     // QKV: q, k or v and the head; FC2: which = K quarter
   bool x_sc1;
 };
-__device__ __forceinline__ Job make_job(const Args &a, int l, int ph, const It &d) {
+template <int PH>
+__device__ __forceinline__ Job make_job_t(const Args &a, int l, const It &d) {
   const LayerW &w = a.layers[l];
   const Bufs cur = layer_bufs(a, l);
   Job j{};
   j.g.m0 = d.a * 32;
+  j.g.rot = (d.a + (d.b >> 3)) % 3;
   j.ln = LN_NONE;
   j.x_sc1 = true;
-  if (ph == PH_QKV) {
+  if constexpr (PH == PH_QKV) {
     const int which = d.b / 12, head = d.b % 12;
+    j.which = which; j.head = head;
     j.g.W = w.w_qkv + (size_t)which * H * H; j.g.ldw = H; j.g.kw0 = 0; j.g.n0 = head * HD;
     j.g.ldx = H; j.g.kx0 = 0;
     if (l == 0) { j.g.X = a.x; j.x_sc1 = false; }
@@ -646,28 +701,50 @@ __device__ __forceinline__ Job make_job(const Args &a, int l, int ph, const It &
       j.ln = (pw.ln2_g || pw.ln2_b) ? LN_AFFINE : LN_PLAIN;
     }
     j.bias = w.b_qkv ? w.b_qkv + which * H : nullptr;
-  } else if (ph == PH_OUT) {
+    j.out = cur.qkv;
+  } else if constexpr (PH == PH_OUT) {
     j.g.W = w.w_o; j.g.ldw = H; j.g.kw0 = 0; j.g.n0 = d.b * 64;
     j.g.X = cur.ctx; j.g.ldx = H; j.g.kx0 = 0;
     j.bias = w.b_o;
-    if (l > 0) { j.rgam = a.layers[l - 1].ln2_g; j.rbet = a.layers[l - 1].ln2_b; }
-  } else if (ph == PH_FC1) {
+    if (l > 0) {
+      const Bufs prev = layer_bufs(a, l - 1);
+      j.rgam = a.layers[l - 1].ln2_g; j.rbet = a.layers[l - 1].ln2_b;
+      j.res = prev.z2; j.rstats = prev.st2;
+    } else j.res = a.x;
+    j.out = cur.z1; j.aux = cur.st1;
+  } else if constexpr (PH == PH_FC1) {
     j.g.W = w.w_fc1; j.g.ldw = F; j.g.kw0 = 0; j.g.n0 = d.b * 64;
     j.g.X = cur.z1; j.g.ldx = H; j.g.kx0 = 0;
     j.stats = cur.st1; j.gam = w.ln1_g; j.bet = w.ln1_b;
     j.ln = (w.ln1_g || w.ln1_b) ? LN_AFFINE : LN_PLAIN;
     j.bias = w.b_fc1;
+    j.out = cur.h;
   } else {   // PH_FC2: slice = n-slice * 4 + K quarter
+    static_assert(PH == PH_FC2, "a GEMM phase");
     const int ks = d.b & 3, ns = d.b >> 2;
+    j.which = ks;
     j.g.W = w.w_fc2; j.g.ldw = H; j.g.kw0 = ks * 768; j.g.n0 = ns * 64;
     j.g.X = cur.h; j.g.ldx = F; j.g.kx0 = ks * 768;
+    j.aux = cur.part;
   }
   return j;
 }
+__device__ __forceinline__ Job make_job(const Args &a, int l, int ph, const It &d) {
+  return ph == PH_QKV ? make_job_t<PH_QKV>(a, l, d) : ph == PH_OUT ? make_job_t<PH_OUT>(a, l, d)
+       : ph == PH_FC1 ? make_job_t<PH_FC1>(a, l, d) : make_job_t<PH_FC2>(a, l, d);
+}
+// Holds the addresses an item needs after its wait in registers from here on: what is computed in front of the
+// wait stays there, instead of being recomputed (or fetched from the kernel arguments) between the wait and the
+// first load.
+template <class T>
+__device__ __forceinline__ void keep_scalar(T *&p) { asm volatile("" : "+s"(p)); }
+__device__ __forceinline__ void pin(Job &j) {
+  keep_scalar(j.g.X); keep_scalar(j.stats); keep_scalar(j.res); keep_scalar(j.rstats); keep_scalar(j.out); keep_scalar(j.aux);
+}
 // The loads of an item that depend on no other workgroup: weight slice, LayerNorm vectors, bias.
-__device__ __forceinline__ void issue_weights(unsigned char *lds, const Job &j) {
-  issue_w(lds, j.g);
-  issue_params(lds, j.gam, j.bet, j.ln == LN_AFFINE, j.bias, j.g.n0);
+__device__ __forceinline__ void issue_weights(unsigned char *lds, const Job &j, bool ahead) {
+  if (ahead) issue_w_ahead(lds, j.g); else issue_w(lds, j.g);
+  issue_params(lds, j.gam, j.bet, j.ln == LN_AFFINE, j.bias, j.g.n0, ahead);
   const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
   if (w == 2 && lane < 8) {      // the residual's LayerNorm vectors for the item's 64 columns (OUT)
     if (j.rgam) dma16<false>(uniform_ptr(j.rgam + j.g.n0), (unsigned)lane * 16, uni(lds_address(lds) + kGamOff));
@@ -678,25 +755,35 @@ __device__ __forceinline__ void issue_weights(unsigned char *lds, const Job &j) 
 __device__ __forceinline__ f4 widen(h4 v) { return f4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]}; }
 
 // One GEMM item from operand fetch to the stores of its epilogue.
-__device__ __forceinline__ void run_gemm_item(unsigned char *lds, const Args &a, int l, int ph, const It &d, bool w_ready) {
-  const Job j = make_job(a, l, ph, d);
-  const Bufs cur = layer_bufs(a, l);
-  if (!w_ready) issue_weights(lds, j);
+template <int PH>
+__device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &a, int l, const It &d, const Job &j, bool w_ready, const Sync *sy = nullptr) {
+  constexpr int ph = PH;
+  if (!w_ready) issue_weights(lds, j, false);
   // what the item reads of other workgroups' results, statistics first (they are needed first)
   if (j.ln != LN_NONE) issue_stats<4>(lds, j.stats, j.g.m0);
-  if (ph == PH_OUT) {
+  if constexpr (ph == PH_OUT) {
     const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
-    const half_t *res = l == 0 ? a.x : layer_bufs(a, l - 1).z2;
     // residual patch: rows m0 .. m0 + 31, columns n0 .. n0 + 63 -> [32][128 B] at kAuxOff
-    dma16<true>(uniform_ptr(res + (size_t)(j.g.m0 + 8 * w) * H + j.g.n0), (unsigned)((lane >> 3) * H * 2 + (lane & 7) * 16),
+    dma16<true>(uniform_ptr(j.res + (size_t)(j.g.m0 + 8 * w) * H + j.g.n0), (unsigned)((lane >> 3) * H * 2 + (lane & 7) * 16),
                 uni(lds_address(lds) + kAuxOff + w * 1024));
-    if (l > 0) issue_stats<1>(lds, layer_bufs(a, l - 1).st2, j.g.m0);
+    if (j.rstats) issue_stats<1>(lds, j.rstats, j.g.m0);
   }
+#ifdef SOUFFLE_STAGE_MARKS      // development build: serialises the weight slice and the X tile to time them apart
+  if (sy) stamp_mark(*sy, l * PH_SLOTS + ph, 4);
+#endif
   if (j.x_sc1) issue_x<true>(lds, j.g); else issue_x<false>(lds, j.g);
+#ifdef SOUFFLE_STAGE_MARKS
+  if (sy) stamp_mark(*sy, l * PH_SLOTS + ph, 6);
+#endif
   f4 acc[2][4];
-  if (j.ln == LN_NONE) mfma_quarter<LN_NONE>(lds, acc, a.eps);
-  else if (j.ln == LN_PLAIN) mfma_quarter<LN_PLAIN>(lds, acc, a.eps);
-  else mfma_quarter<LN_AFFINE>(lds, acc, a.eps);
+  if (sy && sy->trace) { wait_vmcnt<8>(); stamp_mark(*sy, l * PH_SLOTS + ph, 0); }
+#ifdef SOUFFLE_STAGE_MARKS
+  if (sy) { wait_vmcnt<0>(); stamp_mark(*sy, l * PH_SLOTS + ph, 7); }
+#endif
+  if (j.ln == LN_NONE) mfma_quarter<LN_NONE>(lds, acc, a.eps, j.g.rot);
+  else if (j.ln == LN_PLAIN) mfma_quarter<LN_PLAIN>(lds, acc, a.eps, j.g.rot);
+  else mfma_quarter<LN_AFFINE>(lds, acc, a.eps, j.g.rot);
+  if (sy) stamp_mark(*sy, l * PH_SLOTS + ph, 1);
   const half_t *bias_lds = j.bias ? reinterpret_cast<const half_t *>(lds + kBiasOff) : nullptr;
   auto add_bias = [&](int col0, f4 &lo, f4 &hi) {
     if (bias_lds) {
@@ -705,19 +792,19 @@ __device__ __forceinline__ void run_gemm_item(unsigned char *lds, const Args &a,
       hi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]};
     }
   };
-  if (ph == PH_QKV) {
-    const int which = d.b / 12, head = d.b % 12;
+  if constexpr (ph == PH_QKV) {
+    const int which = j.which, head = j.head;
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
       add_bias(col0, lo, hi);
       const int m = j.g.m0 + row, b = m / a.S, s = m % a.S;
-      st16<true>(cur.qkv, ((((which * a.B + b) * NH + head) * a.S + s) * HD + col0) * 2, pack_h8(lo, hi));
+      st16<true>(j.out, ((((which * a.B + b) * NH + head) * a.S + s) * HD + col0) * 2, pack_h8(lo, hi));
     });
-  } else if (ph == PH_OUT) {
+  } else if constexpr (ph == PH_OUT) {
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
       add_bias(col0, lo, hi);
       const h8 rv = *reinterpret_cast<const h8 *>(lds + kAuxOff + row * 128 + col0 * 2);
       f4 rlo = f4{(float)rv[0], (float)rv[1], (float)rv[2], (float)rv[3]}, rhi = f4{(float)rv[4], (float)rv[5], (float)rv[6], (float)rv[7]};
-      if (l > 0) {   // the residual is LN2 of the previous layer's sum: normalise the patch
+      if (j.rstats) {   // the residual is LN2 of the previous layer's sum: normalise the patch
         const float *sp = reinterpret_cast<const float *>(lds + kAuxOff + 4096) + row * 24;
         float mean = 0.f;
 #pragma unroll
@@ -734,14 +821,14 @@ __device__ __forceinline__ void run_gemm_item(unsigned char *lds, const Args &a,
       lo += rlo; hi += rhi;
       const int m = j.g.m0 + row;
       const u4 packed = pack_h8(lo, hi);
-      st16<true>(cur.z1, (m * H + j.g.n0 + col0) * 2, packed);
+      st16<true>(j.out, (m * H + j.g.n0 + col0) * 2, packed);
       const h8 r8 = as_h8(packed);
       float v[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[i] = (float)r8[i];
-      put_stat<8, 8>(cur.st1, m, d.b, v, opaque_thread_id() & 7);
+      put_stat<8, 8>(j.aux, m, d.b, v, opaque_thread_id() & 7);
     });
-  } else if (ph == PH_FC1) {
+  } else if constexpr (ph == PH_FC1) {
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
       add_bias(col0, lo, hi);
       if (a.act == SOUFFLE_ACT_RELU) {
@@ -751,55 +838,56 @@ __device__ __forceinline__ void run_gemm_item(unsigned char *lds, const Args &a,
 #pragma unroll
         for (int i = 0; i < 4; ++i) { lo[i] = gelu_tanh(lo[i]); hi[i] = gelu_tanh(hi[i]); }
       }
-      st16<true>(cur.h, ((j.g.m0 + row) * F + j.g.n0 + col0) * 2, pack_h8(lo, hi));
+      st16<true>(j.out, ((j.g.m0 + row) * F + j.g.n0 + col0) * 2, pack_h8(lo, hi));
     });
   } else {
-    const int ks = d.b & 3;
+    const int ks = j.which;
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
       const int off = ((ks * a.M + j.g.m0 + row) * H + j.g.n0 + col0) * 4;
-      st16<true>(cur.part, off, __builtin_bit_cast(u4, lo));
-      st16<true>(cur.part, off + 16, __builtin_bit_cast(u4, hi));
+      st16<true>(j.aux, off, __builtin_bit_cast(u4, lo));
+      st16<true>(j.aux, off + 16, __builtin_bit_cast(u4, hi));
     });
   }
+}
+__device__ __forceinline__ void run_gemm_item(unsigned char *lds, const Args &a, int l, int ph, const It &d, const Job &j, bool w_ready, const Sync *sy = nullptr) {
+  if (ph == PH_QKV) run_gemm_item_t<PH_QKV>(lds, a, l, d, j, w_ready, sy);
+  else if (ph == PH_OUT) run_gemm_item_t<PH_OUT>(lds, a, l, d, j, w_ready, sy);
+  else if (ph == PH_FC1) run_gemm_item_t<PH_FC1>(lds, a, l, d, j, w_ready, sy);
+  else run_gemm_item_t<PH_FC2>(lds, a, l, d, j, w_ready, sy);
 }
 
 // RED: rows 8 ks .. 8 ks + 7 of the tile of FC2 item (m-tile, n-slice * 4 + ks): z2 = sum of the four partial sums
 // (in order) + bias + LN1(z1), rounded to fp16, and the statistics of those 64 values per row.
-// `pre` runs between the loads that need no sibling and those that do (the wait for the siblings).
+// `pre` (the wait for the three sibling items) runs after the loads that need no sibling have been requested and
+// before anything is computed from them: they travel while the workgroup polls.
 template <class Pre>
 __device__ __forceinline__ void run_red_item(const Args &a, int l, const It &d, Pre pre) {
   const LayerW &w = a.layers[l];
   const Bufs cur = layer_bufs(a, l);
   const int tid = opaque_thread_id(), row = tid >> 5, cp = tid & 31;
   const int ks = d.b & 3, ns = d.b >> 2, m = d.a * 32 + ks * 8 + row, n = ns * 64 + 2 * cp;
-  // LN1 of the residual
+  // LN1 of the residual: twelve lanes of the row's 32 read one slice of its statistics each
   u2 part_stat = {0u, 0u};
   if (cp < 12) part_stat = ld8<true>(cur.st1, (m * 12 + cp) * 8);
   const unsigned zraw = ld4<true>(cur.z1, (m * H + n) * 2);
-  float g0 = 1.f, g1 = 1.f, e0 = 0.f, e1 = 0.f, c0 = 0.f, c1 = 0.f;
-  if (w.ln1_g) { const h2 t = ldg<h2>(w.ln1_g + n); g0 = (float)t[0]; g1 = (float)t[1]; }
-  if (w.ln1_b) { const h2 t = ldg<h2>(w.ln1_b + n); e0 = (float)t[0]; e1 = (float)t[1]; }
-  if (w.b_fc2) { const h2 t = ldg<h2>(w.b_fc2 + n); c0 = (float)t[0]; c1 = (float)t[1]; }
-  const float pm = cp < 12 ? f32_of(part_stat[0]) : 0.f, pq = f32_of(part_stat[1]);
-  float s = pm;
-#pragma unroll
-  for (int k = 1; k < 32; k <<= 1) s += wave_xor(s, k);
-  const float mean = s * (1.0f / 12.0f);
-  float q = cp < 12 ? pq + 64.0f * (pm - mean) * (pm - mean) : 0.f;
-#pragma unroll
-  for (int k = 1; k < 32; k <<= 1) q += wave_xor(q, k);
-  const float rstd = rsqrtf(q * (1.0f / 768.0f) + a.eps);
-  const h2 z = __builtin_bit_cast(h2, zraw);
-  const float y0 = ((float)z[0] - mean) * rstd * g0 + e0, y1 = ((float)z[1] - mean) * rstd * g1 + e1;
-  if (a.ln1_out) *reinterpret_cast<h2 *>(a.ln1_out + (size_t)m * H + n) = h2{(half_t)y0, (half_t)y1};
+  h2 gv = {(half_t)1.f, (half_t)1.f}, ev = {(half_t)0.f, (half_t)0.f}, cv = {(half_t)0.f, (half_t)0.f};
+  if (w.ln1_g) gv = ldg<h2>(w.ln1_g + n);
+  if (w.ln1_b) ev = ldg<h2>(w.ln1_b + n);
+  if (w.b_fc2) cv = ldg<h2>(w.b_fc2 + n);
   pre();
-  float v0 = 0.f, v1 = 0.f;
   u2 pr[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) pr[k] = ld8<true>(cur.part, ((k * a.M + m) * H + n) * 4);
+  const float pm = cp < 12 ? f32_of(part_stat[0]) : 0.f, pq = f32_of(part_stat[1]);
+  const float mean = sum32(pm) * (1.0f / 12.0f);
+  const float rstd = rsqrtf(sum32(cp < 12 ? pq + 64.0f * (pm - mean) * (pm - mean) : 0.f) * (1.0f / 768.0f) + a.eps);
+  const h2 z = __builtin_bit_cast(h2, zraw);
+  const float y0 = ((float)z[0] - mean) * rstd * (float)gv[0] + (float)ev[0], y1 = ((float)z[1] - mean) * rstd * (float)gv[1] + (float)ev[1];
+  if (a.ln1_out) *reinterpret_cast<h2 *>(a.ln1_out + (size_t)m * H + n) = h2{(half_t)y0, (half_t)y1};
+  float v0 = 0.f, v1 = 0.f;
 #pragma unroll
   for (int k = 0; k < 4; ++k) { v0 += f32_of(pr[k][0]); v1 += f32_of(pr[k][1]); }
-  v0 += c0 + y0; v1 += c1 + y1;
+  v0 += (float)cv[0] + y0; v1 += (float)cv[1] + y1;
   const h2 out = {(half_t)v0, (half_t)v1};
   st4<true>(cur.z2, (m * H + n) * 2, __builtin_bit_cast(unsigned, out));
   float vv[2] = {(float)out[0], (float)out[1]};
@@ -839,6 +927,27 @@ __device__ __forceinline__ void for_items(const Shape &sh, int ph, int b, Fn fn)
     first = false;
   }
 }
+// the items of workgroup b in phase ph from item number `it` on (it + G, it + 2 G, ...): fn(item)
+template <class Fn>
+__device__ __forceinline__ void for_items_from(const Shape &sh, int ph, int it, Fn fn) {
+  const int span = ph_span(sh, ph);
+  for (; it < span; it += sh.G) {
+    It d;
+    if (it < 0 || !ph_item(sh, ph, it, d)) continue;
+    fn(d);
+  }
+}
+// the number of workgroup b's first item in phase ph (for_items_from continues behind it), -1 = none
+struct FirstItem { int it; It d; };
+__device__ __forceinline__ FirstItem first_item(const Shape &sh, int ph, int b) {
+  const int span = ph_span(sh, ph);
+  FirstItem f{-1, It{0, 0}};
+  for (int it = b - ph_off(sh, ph); it < span && f.it < 0; it += sh.G) {
+    It d;
+    if (it >= 0 && ph_item(sh, ph, it, d)) { f.it = it; f.d = d; }
+  }
+  return f;
+}
 __device__ __forceinline__ AttnArgs attn_args(const Args &a, int l) {
   const Bufs cur = layer_bufs(a, l);
   return AttnArgs{a.B, a.S, a.scale, cur.qkv, a.mask, cur.ctx, a.probs};
@@ -853,63 +962,149 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
   Sync sy;
   sync_begin(sy, args.flags, args.ctl + kCtlErrWord, args.trace, args.trace_cap);
   const int L = args.num_layers;
+  stamp_wait(sy, PH_SLOTS - 1, 0);          // (slot 7 of layer 0 is no phase: start of the kernel, end of its set-up)
   // Who feeds whom (wave 0: 4 workgroups per lane, one nibble per phase) and in which phases this workgroup
   // has items (one bit per phase); packed into words so that the phase loop indexes no register array.
+  // Thread t answers for producer workgroup t; the answers travel through LDS to the lanes of wave 0.
   unsigned wm_all = 0, mine_bits = 0;
-  for (int ph = 0; ph <= PH_FIN; ++ph) {
-    if (tid < 64) wm_all |= wait_mask(sh, ph, b, tid) << (4 * ph);
-    mine_bits |= (has_items(sh, ph, b) ? 1u : 0u) << ph;
+  {
+    unsigned needs = 0;
+    for (int ph = 0; ph <= PH_FIN; ++ph) {
+      needs |= (wait_needs(sh, ph, b, tid) ? 1u : 0u) << ph;
+      mine_bits |= (has_items(sh, ph, b) ? 1u : 0u) << ph;
+    }
+    lds[tid] = (unsigned char)needs;
+    __syncthreads();
+    if (tid < 64) {
+      const unsigned four = *reinterpret_cast<const unsigned *>(lds + 4 * tid);
+      for (int ph = 0; ph <= PH_FIN; ++ph)
+        for (int t = 0; t < 4; ++t) wm_all |= ((four >> (8 * t + ph)) & 1u) << (4 * ph + t);
+    }
+    __syncthreads();
   }
+  stamp_wait(sy, PH_SLOTS - 1, 1);
   auto mine = [&](int ph) { return ((mine_bits >> ph) & 1u) != 0; };
   auto wm = [&](int ph) { return (wm_all >> (4 * ph)) & 15u; };
+  // The first item of each GEMM phase (at up to 256 rows there is no second one): found once, not per layer.
+  const FirstItem f_qkv = first_item(sh, PH_QKV, b), f_out = first_item(sh, PH_OUT, b), f_fc1 = first_item(sh, PH_FC1, b), f_fc2 = first_item(sh, PH_FC2, b);
+  auto first_of = [&](auto phc) -> const FirstItem & {
+    constexpr int ph = decltype(phc)::value;
+    if constexpr (ph == PH_QKV) return f_qkv; else if constexpr (ph == PH_OUT) return f_out; else if constexpr (ph == PH_FC1) return f_fc1; else return f_fc2;
+  };
   // Weight slices are fetched one GEMM phase ahead, as soon as the W region of the LDS is free: pf names the
   // (layer, phase) whose first item's slice has been requested, -1 = none.
   int pf = -1;
-  auto prefetch_after = [&](int l, int ph) {
-    for (int step = 1; step <= 6; ++step) {
-      const int q = ph + step, ll = l + q / 6, pp = q % 6;
-      if (ll >= L) return;
-      if (pp == PH_ATT) { if (mine(PH_ATT)) return; continue; }    // the attention tiles overlap the W region
-      if (pp == PH_RED || !mine(pp)) continue;
-      for_items(sh, pp, b, [&](const It &d, bool first) { if (first) issue_weights(lds, make_job(args, ll, pp, d)); });
-      pf = ll * 8 + pp;
-      return;
-    }
+  auto prefetch_after = [&](int l, auto phc) {
+    constexpr int ph = decltype(phc)::value;
+    bool done = false;
+    static_for<1, 7>([&](auto sc) {
+      constexpr int q = ph + decltype(sc)::value, dl = q / 6, pp = q % 6;
+      if (done) return;
+      if (l + dl >= L) { done = true; return; }
+      if constexpr (pp == PH_ATT) {
+        if (mine(PH_ATT)) done = true;                  // the attention tiles overlap the W region
+      } else if constexpr (pp != PH_RED) {
+        if (mine(pp)) {
+          issue_weights(lds, make_job_t<pp>(args, l + dl, first_of(std::integral_constant<int, pp>{}).d), true);
+          pf = (l + dl) * 8 + pp;
+          done = true;
+        }
+      }
+    });
   };
-  int l = 0, ph = -1;          // (the request in front of the first phase shares the call below)
+  // A workgroup without any item (at 128 rows: a quarter of the grid) fetches weight slices ahead of the workgroups
+  // of its XCD that will multiply them: a CU takes data from beyond its L2 at a third of the rate at which it
+  // takes it from the L2 (the requests it can have in flight are few), and 96 KB of weights per phase are more than
+  // the hand-over in front of the phase covers.  The slices land in this workgroup's own LDS, which nobody reads:
+  // what counts is that they have passed through the L2.  It stays two GEMM phases ahead of workgroup 0, which has
+  // an item in every GEMM phase, so that no more than a few slices wait in the L2 at a time.
+  if (mine_bits == 0) {
+    int rank = 0, peers = 0;                       // among the idle workgroups of this XCD
+    for (int ob = b & 7; ob < sh.G; ob += 8) {
+      bool idle = true;
+      for (int ph = 0; ph <= PH_FIN; ++ph) idle = idle && !has_items(sh, ph, ob);
+      if (idle) { if (ob < b) ++rank; ++peers; }
+    }
+    int turn = 0;
 #pragma unroll 1
-  for (;;) {
-    if (pf < 0) prefetch_after(l, ph);
-    // next phase
-    if (++ph > PH_RED) { ph = PH_QKV; if (++l >= L) break; }
-    if (!mine(ph)) continue;
-    if (ph == PH_RED) {
+    for (int ll = 0; ll < L; ++ll) {
+      static_for<0, 4>([&](auto kc) {                // GEMM phase number g = 4 ll + k: QKV, OUT, FC1 or FC2 of layer ll
+        constexpr int k = decltype(kc)::value, pph = k == 0 ? PH_QKV : k == 1 ? PH_OUT : k == 2 ? PH_FC1 : PH_FC2;
+        const int g = 4 * ll + k;
+        if (g >= 2) {
+          constexpr int ppp = k == 0 ? PH_FC1 : k == 1 ? PH_FC2 : k == 2 ? PH_QKV : PH_OUT;      // two GEMM phases back
+          await(sy, tid == 0 ? 1u : 0u, phase_seq(sy, k < 2 ? ll - 1 : ll, ppp), PH_SLOTS * L);   // (workgroup 0's flag word; no trace slot)
+        }
+        const int slices = ph_slices(pph);
+        for (int ws = b & 7; ws < slices; ws += 8, ++turn) {
+          if (turn % peers != rank) continue;
+          const Job j = make_job_t<pph>(args, ll, It{0, ws});
+          __syncthreads();
+          issue_w(lds, j.g);
+          wait_vmcnt<0>();
+        }
+      });
+    }
+    sync_end(sy, L);
+    return;
+  }
+  auto gemm_phase = [&](int l, auto phc) {
+    constexpr int ph = decltype(phc)::value;
+    if (!mine(ph)) return;
+    const FirstItem &f0 = first_of(phc);
+    // what the first item multiplies is worked out before the wait, not between the wait and its loads
+    Job j0 = make_job_t<ph>(args, l, f0.d);
+    pin(j0);
+    const bool ready = pf == l * 8 + ph;
+    pf = -1;
+    if (l > 0 || ph > PH_QKV) await(sy, wm(ph), phase_seq(sy, ph == PH_QKV ? l - 1 : l, producer_phase(ph)), l * PH_SLOTS + ph);
+    else if (ready) {                                         // (no wait in front of the very first phase)
+      if (tid >= 64) wait_vmcnt<0>();
+      __syncthreads();
+    }
+    run_gemm_item_t<ph>(lds, args, l, f0.d, j0, ready, &sy);
+    for_items_from(sh, ph, f0.it + sh.G, [&](const It &d) {
+      __syncthreads();                                        // the partial tiles of the previous item have been read
+      run_gemm_item_t<ph>(lds, args, l, d, make_job_t<ph>(args, l, d), false, &sy);
+    });
+    stamp_mark(sy, l * PH_SLOTS + ph, 2);
+    publish(sy, phase_seq(sy, l, ph));
+    stamp_mark(sy, l * PH_SLOTS + ph, 3);
+    if (!(ph == PH_FC2 && mine(PH_RED))) prefetch_after(l, phc);   // (RED follows FC2 at once: the request waits until after it)
+  };
+  prefetch_after(0, std::integral_constant<int, -1>{});
+#pragma unroll 1
+  for (int l = 0; l < L; ++l) {
+    gemm_phase(l, std::integral_constant<int, PH_QKV>{});
+    if (mine(PH_ATT)) {
+      await(sy, wm(PH_ATT), phase_seq(sy, l, PH_QKV), l * PH_SLOTS + PH_ATT);
+      const AttnArgs aa = attn_args(args, l);
+      for_items(sh, PH_ATT, b, [&](const It &d, bool) { attn_item_split<NKT>(lds, aa, d.b, d.a); });
+      stamp_mark(sy, l * PH_SLOTS + PH_ATT, 2);
+      publish(sy, phase_seq(sy, l, PH_ATT));
+      stamp_mark(sy, l * PH_SLOTS + PH_ATT, 3);
+      __syncthreads();                                        // every wave is done with the attention tiles
+      if (pf < 0) prefetch_after(l, std::integral_constant<int, PH_ATT>{});
+    }
+    gemm_phase(l, std::integral_constant<int, PH_OUT>{});
+    gemm_phase(l, std::integral_constant<int, PH_FC1>{});
+    gemm_phase(l, std::integral_constant<int, PH_FC2>{});
+    if (mine(PH_RED)) {
       bool waited = false;
       for_items(sh, PH_RED, b, [&](const It &d, bool) {
         run_red_item(args, l, d, [&]() {
-          if (!waited) await(sy, wm(PH_RED), phase_seq(sy, l, PH_FC2));
+          if (!waited) await(sy, wm(PH_RED), phase_seq(sy, l, PH_FC2), l * PH_SLOTS + PH_RED);
           waited = true;
         });
       });
-    } else {
-      if (l > 0 || ph > PH_QKV) await(sy, wm(ph), phase_seq(sy, ph == PH_QKV ? l - 1 : l, producer_phase(ph)));
-      if (ph == PH_ATT) {
-        const AttnArgs aa = attn_args(args, l);
-        for_items(sh, ph, b, [&](const It &d, bool) { attn_item_split<NKT>(lds, aa, d.b, d.a); });
-      } else {
-        const bool ready = pf == l * 8 + ph;
-        pf = -1;
-        for_items(sh, ph, b, [&](const It &d, bool first) {
-          if (!first) __syncthreads();                        // the partial tiles of the previous item have been read
-          run_gemm_item(lds, args, l, ph, d, first && ready);
-        });
-      }
+      stamp_mark(sy, l * PH_SLOTS + PH_RED, 2);
+      publish(sy, phase_seq(sy, l, PH_RED));
+      stamp_mark(sy, l * PH_SLOTS + PH_RED, 3);
+      if (pf < 0) prefetch_after(l, std::integral_constant<int, PH_RED>{});
     }
-    publish(sy, phase_seq(sy, l, ph));
-    if (ph == PH_ATT) __syncthreads();                        // every wave is done with the attention tiles
   }
   if (mine(PH_FIN)) {
-    await(sy, wm(PH_FIN), phase_seq(sy, L - 1, PH_RED));
+    await(sy, wm(PH_FIN), phase_seq(sy, L - 1, PH_RED), (L - 1) * PH_SLOTS + PH_FIN);
     for_items(sh, PH_FIN, b, [&](const It &d, bool) { run_fin_item(args, d); });
   }
   sync_end(sy, L);
@@ -932,7 +1127,7 @@ __global__ void __launch_bounds__(256) k_small_phase(Args args, int l, int ph) {
   } else {
     for_items(sh, ph, b, [&](const It &d, bool first) {
       if (!first) __syncthreads();
-      run_gemm_item(lds, args, l, ph, d, false);
+      run_gemm_item(lds, args, l, ph, d, make_job(args, l, ph, d), false);
     });
   }
 }
