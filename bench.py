@@ -38,20 +38,26 @@ def parse():
     p.add_argument("--workload", default="encoder")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU-baseline sample")
     p.add_argument("--no-cpu", action="store_true")
+    p.add_argument("--no-sub", action="store_true", help="skip the S=384 and B=32 sub-results of the default workload")
     p.add_argument("--weight-sets", type=int, default=4)
     return p.parse_args()
+
+
+def host_threads():
+    """The cores this process may run on (its affinity mask; every one of them is used)."""
+    try:
+        return len(os.sched_getaffinity(0))
+    except Exception:
+        return os.cpu_count() or 1
 
 
 def cpu_baseline_encoder(layers_np, x_np, B, S, budget_s):
     """The CPU oracle (a port: the reference has no CPU path) timed on the host cores."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import oracle
-    threads = os.cpu_count() or 1
-    try:
-        threads = len(os.sched_getaffinity(0))
-    except Exception:
-        pass
-    threads = min(threads, 16)
+    threads = host_threads()
+    print("cpu_baseline: %d cores in the affinity mask (os.cpu_count() = %s), %d OpenMP threads" % (threads, os.cpu_count(), threads),
+          file=sys.stderr)
     os.environ.setdefault("OMP_NUM_THREADS", str(threads))
     oracle.bert_encoder(x_np, layers_np[:1], B, S, threads=threads)       # warm up
     n, t0 = 0, time.perf_counter()
@@ -64,6 +70,49 @@ def cpu_baseline_encoder(layers_np, x_np, B, S, budget_s):
     dt = (time.perf_counter() - t0) / n
     return ref, {"value": dt * 1e6, "unit": "us", "cores": threads, "kind": "port",
                  "sample": "%d passes of the %d-layer encoder B=%d S=%d through oracle/bert_oracle.c (OpenMP fp32)" % (n, len(layers_np), B, S)}
+
+
+def traffic_from_profile(name):
+    """HBM bytes per launch from the tracked counter summary profiles/<name> (a line
+    'traffic_bytes_per_launch: <number>' written when the summary was made), None if there is none."""
+    import re
+    try:
+        with open(os.path.join(ROOT, "profiles", name)) as f:
+            m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", f.read(), re.M)
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def encoder_sub_result(args, B, S, L=12):
+    """One more shape of the same encoder for the default line: parity against the oracle (unless --no-cpu), then
+    the event-timed launch and its place under the roofline that bounds it."""
+    import numpy as np
+    import torch
+    import bert_binding
+    import synth
+    dev = torch.device("cuda:0")
+    layers_np = [synth.bert_layer_weights(2, l) for l in range(L)]
+    x_np = synth.bert_input(2, B, S)
+    enc = bert_binding.Encoder([{k: torch.from_numpy(v).to(dev) for k, v in w.items()} for w in layers_np], B, S)
+    x = torch.from_numpy(x_np).to(dev)
+    out = torch.empty((B * S, 768), dtype=torch.float16, device=dev)
+    y = enc(x, out=out).float().cpu().numpy()
+    parity = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle
+        ref = oracle.bert_encoder(x_np, layers_np, B, S, threads=host_threads())
+        d = np.abs(y - ref)
+        if not (np.isfinite(y).all() and d.max() <= 2e-2 and d.mean() <= 2e-3):
+            print("PARITY FAILURE (B=%d S=%d): max-abs %.4g mean-abs %.4g" % (B, S, d.max(), d.mean()), file=sys.stderr)
+            sys.exit(1)
+        parity = {"max_abs": float(d.max()), "mean_abs": float(d.mean())}
+    _, ev = time_steps(lambda i: enc(x, out=out), max(20, args.steps // 4), 5)
+    flops, bytes_alg = L * layer_flops(B, S), L * layer_bytes(B * S)
+    tf, gbs = flops / (ev * 1e-3) / 1e12, bytes_alg / (ev * 1e-3) / 1e9
+    return {"us": ev * 1e3, "parity": parity, "TFLOPs": tf, "mfma_frac": tf / MFMA_F16_PEAK_TFLOPS, "GBps": gbs,
+            "hbm_frac": gbs / HBM_PEAK_GBS, "bound": "mfma" if flops / (MFMA_F16_PEAK_TFLOPS * 1e12) > bytes_alg / (HBM_PEAK_GBS * 1e9) else "hbm"}
 
 
 def time_steps(launch, steps, warmup):
@@ -145,11 +194,12 @@ def bench_encoder(args, B, S, L, name):
         ach = bytes_alg / (cold_ev * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS,
                 "traffic": None}
+    few_rows = M < 1024
     if (B, S, L) == (1, 128, 12):
-        # L2<->fabric bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a device
-        # copy of known size (profiles/k_encoder_mega_bert_encoder_b1_s128_hbm_traffic.txt)
-        roof["traffic"] = 339.6e6
-    roof["kernel"] = "k_encoder_mega (one launch = %d layers)" % L
+        # L2<->fabric bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a device copy of
+        # known size: read from the tracked summary, so the figure cannot outlive the kernel it was measured on
+        roof["traffic"] = traffic_from_profile("k_encoder_small_bert_encoder_b1_s128_hbm_traffic.txt")
+    roof["kernel"] = "%s (one launch = %d layers)" % ("k_encoder_small" if few_rows else "k_encoder_mega", L)
     roof["algorithmic_bytes_per_launch"] = bytes_alg
     roof["algorithmic_flops_per_launch"] = flops
     roof["avg_launch_us"] = cold_ev * 1e3
@@ -175,16 +225,29 @@ def bench_encoder(args, B, S, L, name):
         roof["frac_of_measured"] = ach / (mfma_tflops if mfma_bound else copy_gbs)
         if (B, S) == (1, 384):            # mixed shape: both fractions
             roof["mfma_frac"] = flops / (cold_ev * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS
-        if M < 1024:
-            # what a chain of this many dependent grid-wide stages costs with no arithmetic at all
-            nst = 6 * L
+        if few_rows:
+            # Six phases per layer (QKV, attention, out-projection, FC1, FC2, split-K reduction) and the final
+            # LayerNorm follow one another through flag hand-overs among the workgroups that exchange data; no grid
+            # barrier.  The yardstick beside it: a chain of as many grid-wide stages with no arithmetic at all.
+            nst = 6 * L + 1
             bar_us, floor_us = sh.stage_floor_us(nst)
             res["extra"]["stages_per_launch"] = nst
+            res["extra"]["grid_barriers_per_launch"] = 0
             res["extra"]["barriers_only_us"] = bar_us
             res["extra"]["stage_chain_floor_us"] = floor_us
             res["extra"]["frac_of_stage_chain_floor"] = floor_us / (cold_ev * 1e3)
     except sh.SouffleError as e:
         roof["measured_ceilings_error"] = str(e)
+    # the same launch as a cooperative one (hipLaunchCooperativeKernel): the co-residency the hand-overs need is then
+    # guaranteed by the runtime instead of checked with the occupancy query
+    try:
+        sh.set_cooperative_launch(1)
+        _, coop_ev = time_steps(lambda i: encs[i % len(encs)](x, out=out), max(20, args.steps // 2), 5)
+        res["extra"]["cooperative_launch_us"] = coop_ev * 1e3
+    except sh.SouffleError as e:
+        res["extra"]["cooperative_launch_error"] = str(e)
+    finally:
+        sh.set_cooperative_launch(0)
     if cpu:
         res["cpu_baseline"] = cpu
         res["extra"]["gpu_speedup_vs_cpu"] = cpu["value"] / (cold_ev * 1e3)
@@ -202,6 +265,9 @@ def main():
         sys.exit(3)
     if args.workload == "encoder":
         res = bench_encoder(args, 1, 128, 12, "BERT-base 12-layer encoder, B=1, S=128, fp16 (BASELINE configs[2], first shape)")
+        if not args.no_sub:
+            res["extra"]["encoder_s384"] = encoder_sub_result(args, 1, 384)
+            res["extra"]["encoder_b32"] = encoder_sub_result(args, 32, 128)
     elif args.workload == "layer":
         res = bench_encoder(args, 1, 128, 1, "single BERT-base encoder layer, B=1, S=128, fp16 (BASELINE configs[0])")
     elif args.workload == "encoder_s384":

@@ -21,10 +21,26 @@ def _cpu_time(fn, budget_s):
 
 
 def _threads():
+    from bench import host_threads
+    return host_threads()
+
+
+def _kernel_us(launch):
+    """(min over rounds of the mean, median) of `launch()` in us, HIP events on the launch stream, the reference's
+    timing rule (cpp/souffle_utils/cuda_utils.h:102-136).  `launch` is a bare C-ABI call on preallocated buffers."""
+    import souffle_hip as sh
+    return sh.bench_us(launch, warmup=20, rounds=5, repeat=100)
+
+
+def _floor(extra, stages, launch_us):
+    """What `stages` dependent grid-wide stages cost with no arithmetic at all, beside the measured launch."""
+    import souffle_hip as sh
     try:
-        return min(len(os.sched_getaffinity(0)), 16)
-    except Exception:
-        return min(os.cpu_count() or 1, 16)
+        bar_us, floor_us = sh.stage_floor_us(stages)
+        extra.update({"stages_per_launch": stages, "barriers_only_us": bar_us, "stage_chain_floor_us": floor_us,
+                      "frac_of_stage_chain_floor": floor_us / launch_us})
+    except sh.SouffleError as e:
+        extra["stage_floor_error"] = str(e)
 
 
 def _base(metric, value_us, args, workload, dtype, roof, extra):
@@ -61,8 +77,10 @@ def bench_lstm(args):
     roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
             "kernel": "k_lstm", "algorithmic_bytes_per_launch": bytes_alg, "avg_launch_us": ev * 1e3,
             "note": "109 dependent wavefront steps bound the latency, not the one-time 10.5 MB weight stream"}
+    extra = {"us_per_wavefront_step": ev * 1e3 / 109}
+    _floor(extra, 109, ev * 1e3)
     res = _base("lstm_stack_latency_us", wall * 1e3, args, "stacked LSTM 10x256, T=100, batch 1 (BASELINE configs[1])", "f16",
-                roof, {"us_per_wavefront_step": ev * 1e3 / 109})
+                roof, extra)
     if res_cpu:
         res["cpu_baseline"] = res_cpu
     return res
@@ -92,13 +110,17 @@ def bench_swin(args):
         us, n = _cpu_time(lambda: oracle.swin_block_pair(x, ws, threads=thr), min(args.cpu_seconds, 8.0))
         res_cpu = {"value": us, "unit": "us", "cores": thr, "kind": "port",
                    "sample": "%d passes of the 56x56x128 block pair through oracle/swin_oracle.c (OpenMP fp32)" % n}
-    wall, ev = time_steps(lambda i: sb.swin_block_pair(dx, dw[0], dw[1]), args.steps, args.warmup)
+    launch = sb.block_pair_launcher(dx, dw[0], dw[1], torch.empty_like(dx))       # bare C-ABI call, output preallocated
+    wall, ev = time_steps(lambda i: launch(), args.steps, args.warmup)
+    mn, med = _kernel_us(launch)
     flops = 2 * (2.0 * 3136 * 196608 + 4.0 * 64 * 4 * 49 * 49 * 32)
     ach = flops / (ev * 1e-3) / 1e12
     roof = {"bound": "mfma", "achieved": ach, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": ach / MFMA_F16_PEAK_TFLOPS,
             "traffic": None, "kernel": "k_block_pair", "algorithmic_flops_per_launch": flops, "avg_launch_us": ev * 1e3}
+    extra = {"kernel_us_min_of_means": mn, "kernel_us_median": med}
+    _floor(extra, sb.BLOCK_PAIR_GRID_STAGES, ev * 1e3)
     res = _base("swin_block_pair_latency_us", wall * 1e3, args,
-                "Swin-Base stage-1 block pair 56x56, C=128, 4 heads, window 7, shift 3 (BASELINE configs[3])", "f16", roof, {})
+                "Swin-Base stage-1 block pair 56x56, C=128, 4 heads, window 7, shift 3 (BASELINE configs[3])", "f16", roof, extra)
     if res_cpu:
         res["cpu_baseline"] = res_cpu
     return res
@@ -115,17 +137,20 @@ def bench_se(args):
     for (Cc, Hh, R), ref_us in zip(shapes, a100):
         x = torch.rand((1, Cc, Hh, Hh), device="cuda:0")
         wr, we = torch.randn((R, Cc), device="cuda:0") * 0.3, torch.randn((Cc, R), device="cuda:0") * 0.3
-        wall, ev = time_steps(lambda i: eb.torch_dispatch_efficientnet_se_module_v2_short_cut_fused(x, wr, we, 2, combine="add"),
-                              args.steps, args.warmup)
-        rows.append({"C": Cc, "H": Hh, "R": R, "us": ev * 1e3, "reference_a100_us": ref_us,
-                     "GBps": 2.0 * Cc * Hh * Hh * 4 / (ev * 1e-3) / 1e9})
+        launch = eb.se_launcher(x, wr, we, torch.empty_like(x), torch.empty((1, Cc), device="cuda:0"), combine="add")
+        wall, ev = time_steps(lambda i: launch(), args.steps, args.warmup)
+        mn, med = _kernel_us(launch)
+        rows.append({"C": Cc, "H": Hh, "R": R, "us": ev * 1e3, "kernel_us_min_of_means": mn, "reference_a100_us": ref_us,
+                     "vs_reference_a100": ref_us / mn, "GBps": 2.0 * Cc * Hh * Hh * 4 / (mn * 1e-6) / 1e9})
     tot = sum(r["us"] for r in rows)
     byt = sum(2.0 * r["C"] * r["H"] ** 2 * 4 for r in rows)
     ach = byt / (tot * 1e-6) / 1e9
     roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
             "kernel": "k_se", "avg_launch_us": tot / len(rows)}
+    extra = {"per_shape": rows, "reference_a100_sum_us": sum(a100), "kernel_us_min_of_means_sum": sum(r["kernel_us_min_of_means"] for r in rows)}
+    _floor(extra, 2, tot / len(rows))          # pool -> (grid barrier) -> gate and combine
     return _base("se_module_latency_us_sum_of_10_shapes", tot, args, "EfficientNet-B0 SE module, the reference's 10 shapes, fp32", "f32",
-                 roof, {"per_shape": rows, "reference_a100_sum_us": sum(a100)})
+                 roof, extra)
 
 
 def bench_mbconv(args):
@@ -171,9 +196,11 @@ def bench_mbconv(args):
             "kernel": "k_mbconv", "algorithmic_bytes_per_launch": bytes_alg, "algorithmic_flops_per_launch": flops,
             "avg_launch_us": ev * 1e3,
             "note": "%d dependent stages bound the latency, not the %.1f MB of weights and activations" % (stages, bytes_alg / 1e6)}
+    extra = {"unfused_per_op_us": ev_u * 1e3, "stages": stages, "us_per_stage": ev * 1e3 / stages}
+    _floor(extra, stages, ev * 1e3)
     res = _base("mbconv_stack_latency_us", wall * 1e3, args,
                 "EfficientNet-B0 MBConv stack (16 blocks), 112x112x32 -> 7x7x320, batch 1, fp16 (BASELINE configs[4])", "f16", roof,
-                {"unfused_per_op_us": ev_u * 1e3, "stages": stages, "us_per_stage": ev * 1e3 / stages})
+                extra)
     if res_cpu:
         res["cpu_baseline"] = res_cpu
     return res
@@ -206,14 +233,17 @@ def bench_swin_merge(args):
         us, n = _cpu_time(lambda: oracle.swin_patch_merge(x, H, W, g, b, w, threads=thr), min(args.cpu_seconds, 5.0))
         res_cpu = {"value": us, "unit": "us", "cores": thr, "kind": "port",
                    "sample": "%d passes of the 56x56x128 patch merge through oracle/swin_oracle.c (OpenMP fp32)" % n}
-    wall, ev = time_steps(lambda i: sb.patch_merging(dx, H, W, dg, db, dw), args.steps, args.warmup)
+    launch = sb.patch_merge_launcher(dx, H, W, dg, db, dw, torch.empty((H // 2 * (W // 2), 2 * Cc), dtype=torch.float16, device="cuda:0"))
+    wall, ev = time_steps(lambda i: launch(), args.steps, args.warmup)
+    mn, med = _kernel_us(launch)
     bytes_alg = x.nbytes + w.nbytes + g.nbytes + b.nbytes + y.size * 2
     ach = bytes_alg / (ev * 1e-3) / 1e9
     roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
             "kernel": "k_patch_merge", "algorithmic_bytes_per_launch": bytes_alg,
             "algorithmic_flops_per_launch": 2.0 * 784 * 512 * 256, "avg_launch_us": ev * 1e3,
             "note": "one launch of 1.5 MB and 0.2 GFLOP: launch and memory latency, not bandwidth"}
-    res = _base("swin_patch_merge_latency_us", wall * 1e3, args, "Swin patch merging 56x56x128 -> 28x28x256, fp16", "f16", roof, {})
+    res = _base("swin_patch_merge_latency_us", wall * 1e3, args, "Swin patch merging 56x56x128 -> 28x28x256, fp16", "f16", roof,
+                {"kernel_us_min_of_means": mn, "kernel_us_median": med})
     if res_cpu:
         res["cpu_baseline"] = res_cpu
     return res

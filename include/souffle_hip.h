@@ -173,11 +173,16 @@ int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert
  * HuggingFace embedding module the reference feeds its layer with
  * (cpp/bert/test_souffle_bert_layer.py:186-189; python/models/bert/relay_bert.py:12-13 starts
  * from its [1,384,768] output).  token_ids / segment_ids: int32 device arrays [B*S]
- * (segment_ids and type_emb may be NULL); tables fp16 [rows][768]; ids are not range-checked. */
+ * (segment_ids and type_emb may be NULL); tables fp16 [rows][768] with vocab_size, max_positions
+ * (>= seq_len, else SOUFFLE_ERR_SHAPE) and type_vocab_size rows.  The ids live on the device, so the
+ * call cannot refuse them: an id outside its table is clamped into it, never read out of bounds, and
+ * counted in the device word *bad_ids (may be NULL; the caller zeroes it and reads it after the stream
+ * has finished: a non-zero count means those rows of `out` are wrong). */
 int souffle_bert_embed(const int32_t *token_ids, const int32_t *segment_ids,
-                       const void *word_emb, const void *pos_emb, const void *type_emb,
+                       const void *word_emb, int vocab_size, const void *pos_emb, int max_positions,
+                       const void *type_emb, int type_vocab_size,
                        const void *ln_g, const void *ln_b, float ln_eps,
-                       int batch, int seq_len, int hidden, void *out, souffle_stream_t stream);
+                       int batch, int seq_len, int hidden, void *out, uint32_t *bad_ids, souffle_stream_t stream);
 /* The stage behind the encoder: out[b] = tanh(x[b*S + 0] . W + bias), W fp16 [768][768] stored
  * [K][N] like every weight here (transposition rule: cpp/bert/test_souffle_bert_layer.py:139-143);
  * out fp16 [B][768].  The reference stops at the last encoder layer. */

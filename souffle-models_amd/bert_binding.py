@@ -42,7 +42,11 @@ def _check_f16_cuda(name, t, shape=None):
 
 
 def make_cfg(batch, seq_len, act="gelu_tanh", scale=0.125, ln_eps=1e-12, num_layers=1):
-    acts = {"gelu_tanh": sh.ACT_GELU_TANH, "gelu": sh.ACT_GELU_TANH, "relu": sh.ACT_RELU}
+    acts = {"gelu_tanh": sh.ACT_GELU_TANH, "relu": sh.ACT_RELU}
+    if act == "gelu":
+        # HuggingFace's "gelu" is the erf form; the reference kernel (and this one) computes the tanh form.  The two
+        # differ by up to 5e-4 per activation, so the name is not taken as an alias.
+        raise ValueError("act='gelu' (the erf form) is not built: the reference computes the tanh form, pass act='gelu_tanh'")
     if act not in acts:
         raise ValueError("act must be one of %s" % sorted(acts))
     return sh.BertCfg(batch, seq_len, HIDDEN, HEADS, FFN, acts[act], float(scale), float(ln_eps), num_layers, 0)
@@ -160,11 +164,14 @@ class Encoder:
         return out
 
 
-def embed(token_ids, word_emb, pos_emb, type_emb=None, segment_ids=None, ln_gamma=None, ln_beta=None, ln_eps=1e-12):
+def embed(token_ids, word_emb, pos_emb, type_emb=None, segment_ids=None, ln_gamma=None, ln_beta=None, ln_eps=1e-12,
+          check_ids=True):
     """The stage in front of the encoder: LayerNorm(word[token] + pos[position] + type[segment]).
     Stands in for the HuggingFace embedding module the reference feeds its layer with
     (cpp/bert/test_souffle_bert_layer.py:186-189).  token_ids: int32 CUDA tensor [B, S];
-    returns fp16 [B*S, 768]."""
+    returns fp16 [B*S, 768].  An id outside its table is never read out of bounds (the kernel clamps
+    it); with check_ids the call then waits for the kernel and raises IndexError, as indexing the
+    table on the host would."""
     if not isinstance(token_ids, torch.Tensor) or not token_ids.is_cuda or token_ids.dtype != torch.int32 or token_ids.dim() != 2:
         raise TypeError("token_ids must be an int32 CUDA tensor [B, S]")
     B, S = token_ids.shape
@@ -179,10 +186,20 @@ def embed(token_ids, word_emb, pos_emb, type_emb=None, segment_ids=None, ln_gamm
         raise ValueError("pos_emb has %d rows, sequence length is %d" % (pos_emb.shape[0], S))
     tok = token_ids.contiguous()
     seg = None if segment_ids is None else segment_ids.contiguous()
+    for name, t in (("word_emb", word_emb), ("pos_emb", pos_emb), ("type_emb", type_emb)):
+        if t is not None and (t.dim() != 2 or not t.is_contiguous()):
+            raise ValueError("%s must be a contiguous [rows, %d] table" % (name, HIDDEN))
     out = torch.empty((B * S, HIDDEN), dtype=torch.float16, device=token_ids.device)
-    sh.check(sh.lib().souffle_bert_embed(tok.data_ptr(), sh.ptr(seg), word_emb.data_ptr(), pos_emb.data_ptr(), sh.ptr(type_emb),
+    bad = torch.zeros(1, dtype=torch.int32, device=token_ids.device) if check_ids else None
+    sh.check(sh.lib().souffle_bert_embed(tok.data_ptr(), sh.ptr(seg), word_emb.data_ptr(), word_emb.shape[0], pos_emb.data_ptr(),
+                                         pos_emb.shape[0], sh.ptr(type_emb), 0 if type_emb is None else type_emb.shape[0],
                                          sh.ptr(ln_gamma), sh.ptr(ln_beta), float(ln_eps), B, S, HIDDEN, out.data_ptr(),
-                                         sh.current_stream()))
+                                         sh.ptr(bad), sh.current_stream()))
+    if check_ids:
+        n_bad = int(bad.item())
+        if n_bad:
+            raise IndexError("%d token or segment ids lie outside their embedding tables (%d / %d rows)"
+                             % (n_bad, word_emb.shape[0], 0 if type_emb is None else type_emb.shape[0]))
     return out
 
 

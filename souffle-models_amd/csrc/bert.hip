@@ -426,7 +426,7 @@ __device__ __forceinline__ void rowblock_sync(const Params &a, GridBarrier &bar,
   const int m_tiles = a.M / 256;
   const bool tr = bar.trace && bar.trace_idx < bar.trace_cap && threadIdx.x == 0;
   if (tr) bar.trace[(size_t)(2 * bar.trace_idx) * bar.nblk + blockIdx.x] = wall_clock64();
-  __builtin_amdgcn_s_waitcnt(0);                 // this wave's write-through stores are acknowledged
+  wait_all_memory();                             // this wave's write-through stores are acknowledged
   __syncthreads();
   if (threadIdx.x == 0)
     for (int it = first; it < m_tiles * 16; it += stride) {
@@ -456,6 +456,7 @@ __device__ __forceinline__ void rowblock_sync(const Params &a, GridBarrier &bar,
   if (tr) bar.trace[(size_t)(2 * bar.trace_idx + 1) * bar.nblk + blockIdx.x] = wall_clock64();
   bar.trace_idx++;
   __syncthreads();
+  compiler_fence();                              // no load of the other tiles' results is scheduled above the poll
 }
 template <bool COH, int NZ>
 __device__ __forceinline__ void rowblock_ln(const Params &a, GridBarrier &bar, unsigned tag, const half_t *z, const half_t *resid, const half_t *gam,
@@ -533,7 +534,7 @@ __device__ __forceinline__ void attn_item(half_t *lds_h, const Params &a, int it
   unsigned char *lds = reinterpret_cast<unsigned char *>(lds_h);
   __syncthreads();   // LDS reuse
   attn_issue<NKT>(lds, a, item);
-  __builtin_amdgcn_s_waitcnt(0);
+  wait_all_memory();
   __syncthreads();
   attn_compute<COH, NKT>(lds, a, item);
 }

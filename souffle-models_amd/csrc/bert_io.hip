@@ -15,12 +15,16 @@ namespace bert_io {
 constexpr int H = 768;
 
 // One wave per token: gather three rows, sum in fp32, two-pass LayerNorm in registers.
-__global__ void __launch_bounds__(256) k_embed(const int *tok, const int *seg, const half_t *word, const half_t *pos,
-                                               const half_t *type, const half_t *gam, const half_t *bet, float eps,
-                                               int rows, int S, half_t *out) {
+// An id outside its table is clamped into it (the row is then wrong, but no address outside the tables is read) and
+// counted in *bad_ids.
+__global__ void __launch_bounds__(256) k_embed(const int *tok, const int *seg, const half_t *word, int vocab, const half_t *pos,
+                                               const half_t *type, int type_vocab, const half_t *gam, const half_t *bet, float eps,
+                                               int rows, int S, half_t *out, unsigned *bad_ids) {
   const int lane = threadIdx.x & 63, m = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (m >= rows) return;
-  const int t = tok[m], p = m % S, sg = seg ? seg[m] : 0;
+  const int t_raw = tok[m], p = m % S, sg_raw = seg ? seg[m] : 0;
+  const int t = min(max(t_raw, 0), vocab - 1), sg = type ? min(max(sg_raw, 0), type_vocab - 1) : 0;
+  if (lane == 0 && bad_ids && (t != t_raw || (type && sg != sg_raw))) atomicAdd(bad_ids, 1u);
   f4 v[3];
   float sum = 0.f;
 #pragma unroll
@@ -83,20 +87,26 @@ __global__ void __launch_bounds__(256) k_pooler(const half_t *x, const half_t *w
 
 using namespace souffle;
 
-extern "C" int souffle_bert_embed(const int32_t *token_ids, const int32_t *segment_ids, const void *word_emb,
-                                  const void *pos_emb, const void *type_emb, const void *ln_g, const void *ln_b,
-                                  float ln_eps, int batch, int seq_len, int hidden, void *out, souffle_stream_t stream) {
+extern "C" int souffle_bert_embed(const int32_t *token_ids, const int32_t *segment_ids, const void *word_emb, int vocab_size,
+                                  const void *pos_emb, int max_positions, const void *type_emb, int type_vocab_size,
+                                  const void *ln_g, const void *ln_b, float ln_eps, int batch, int seq_len, int hidden,
+                                  void *out, uint32_t *bad_ids, souffle_stream_t stream) {
   if (!token_ids || !word_emb || !pos_emb || !out) return fail(SOUFFLE_ERR_NULL, "token_ids, word_emb, pos_emb and out must not be NULL");
   if (hidden != bert_io::H) return fail(SOUFFLE_ERR_SHAPE, "only hidden=768 is built (got %d)", hidden);
   if (batch <= 0 || seq_len <= 0 || (long long)batch * seq_len > (1 << 24)) return fail(SOUFFLE_ERR_SHAPE, "batch and seq_len must be positive");
   if (!(ln_eps >= 0.f)) return fail(SOUFFLE_ERR_SHAPE, "ln_eps must be >= 0");
+  if (vocab_size <= 0) return fail(SOUFFLE_ERR_SHAPE, "vocab_size (rows of word_emb) must be positive (got %d)", vocab_size);
+  if (max_positions < seq_len) return fail(SOUFFLE_ERR_SHAPE, "pos_emb has %d rows, the sequence length is %d", max_positions, seq_len);
+  if (type_emb && type_vocab_size <= 0) return fail(SOUFFLE_ERR_SHAPE, "type_vocab_size (rows of type_emb) must be positive (got %d)", type_vocab_size);
+  if (reinterpret_cast<uintptr_t>(bad_ids) & 3u) return fail(SOUFFLE_ERR_ALIGN, "bad_ids must be 4-byte aligned");
   const void *ptrs[6] = {word_emb, pos_emb, type_emb, ln_g, ln_b, out};
   for (const void *q : ptrs)
     if (!aligned16(q)) return fail(SOUFFLE_ERR_ALIGN, "embedding tables, LN vectors and out must be 16-byte aligned");
   const int rows = batch * seq_len;
   hipLaunchKernelGGL(bert_io::k_embed, dim3((rows + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), token_ids, segment_ids,
-                     static_cast<const half_t *>(word_emb), static_cast<const half_t *>(pos_emb), static_cast<const half_t *>(type_emb),
-                     static_cast<const half_t *>(ln_g), static_cast<const half_t *>(ln_b), ln_eps, rows, seq_len, static_cast<half_t *>(out));
+                     static_cast<const half_t *>(word_emb), vocab_size, static_cast<const half_t *>(pos_emb),
+                     static_cast<const half_t *>(type_emb), type_vocab_size, static_cast<const half_t *>(ln_g),
+                     static_cast<const half_t *>(ln_b), ln_eps, rows, seq_len, static_cast<half_t *>(out), bad_ids);
   SOUFFLE_HIP_TRY(hipGetLastError());
   return SOUFFLE_OK;
 }

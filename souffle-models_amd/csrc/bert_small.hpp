@@ -188,6 +188,7 @@ __device__ __forceinline__ void sync_end(Sync &sy, int num_layers) {
 __device__ __forceinline__ void publish(const Sync &sy, unsigned seq) {
   wait_vmcnt<0>();                               // this wave's write-through stores are acknowledged
   __builtin_amdgcn_s_barrier();                  // ... and every wave's
+  compiler_fence();
   if (threadIdx.x < kFlagCopies)
     __hip_atomic_store(sy.flags + threadIdx.x * kFlagStride + blockIdx.x, seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -552,7 +553,7 @@ __device__ __forceinline__ void attn_item_split(unsigned char *lds, const AttnAr
   issue_rows64_wave<0>(qs_ + wave * 2048, Q, 0, 16);               // every wave its own copy of the queries
   issue_rows64_wave<0>(ks_, K, wave * TPW * 16, TPW * 16);
   issue_rows64_wave<1>(vs_, V, wave * TPW * 16, TPW * 16);
-  __builtin_amdgcn_s_waitcnt(0);                                   // this wave's rows only: no barrier needed
+  wait_all_memory();                                               // this wave's rows only: no barrier needed
 
   const half_t *kh = reinterpret_cast<const half_t *>(ks_), *vh = reinterpret_cast<const half_t *>(vs_),
                *qh = reinterpret_cast<const half_t *>(qs_ + wave * 2048);

@@ -281,6 +281,14 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("" ::: "memory");
 }
 
+// Every memory operation this wave has issued is complete (write-through stores acknowledged, loads returned,
+// LDS and scalar traffic done), and the compiler moves no memory access across the wait in either direction:
+// the release half of a hand-over to other workgroups, in front of the barrier that precedes the flag store.
+__device__ __forceinline__ void wait_all_memory() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
+// The compiler moves no memory access across this point (the hardware is not involved): behind the poll of a
+// hand-over, so that no load of what other workgroups published is scheduled in front of the poll.
+__device__ __forceinline__ void compiler_fence() { asm volatile("" ::: "memory"); }
+
 // `mid()` is called by every wave after the workgroup has arrived and before it starts to wait:
 // the place to queue loads that do not depend on other workgroups (the next stage's weight
 // slice), so that they travel while the barrier completes.  Wave 0 polls; its polling loads
@@ -289,8 +297,9 @@ template <class Mid>
 __device__ __forceinline__ void grid_sync(GridBarrier &b, Mid mid) {
   const bool tr = b.trace && b.trace_idx < b.trace_cap && threadIdx.x == 0;
   if (tr) b.trace[(size_t)(2 * b.trace_idx) * b.nblk + blockIdx.x] = wall_clock64();
-  __builtin_amdgcn_s_waitcnt(0);           // write-through stores are acknowledged
+  wait_all_memory();                       // write-through stores are acknowledged
   __builtin_amdgcn_s_barrier();
+  compiler_fence();
 #ifdef SOUFFLE_STAGE_MARKS
   trace_mark(b, 7);
 #endif
@@ -321,6 +330,7 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b, Mid mid) {
   b.trace_idx++;
   __builtin_amdgcn_s_barrier();            // no memory wait here: loads queued by mid() may still be in flight
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  compiler_fence();                        // no load of what the other workgroups wrote is scheduled above the poll
 }
 __device__ __forceinline__ void grid_sync(GridBarrier &b) { grid_sync(b, []() {}); }
 
@@ -332,7 +342,7 @@ __device__ __forceinline__ void grid_barrier_end(GridBarrier &b) {
     // The next launch on this control block reads these words first thing.  The wave does not end
     // before they are acknowledged, so that their arrival does not rest on what the end of a kernel
     // waits for when the runtime queues two launches without a cache release in between.
-    __builtin_amdgcn_s_waitcnt(0);
+    wait_all_memory();
   }
 }
 

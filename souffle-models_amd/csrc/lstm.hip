@@ -125,7 +125,7 @@ __global__ void __launch_bounds__(256) k_lstm(Args a) {
   }
   // (acknowledged before the wave ends: a clearing store that were still on its way when the next
   // launch publishes into the same slot would wipe that value out)
-  __builtin_amdgcn_s_waitcnt(0);
+  wait_all_memory();
   grid_barrier_end(bar);
 }
 

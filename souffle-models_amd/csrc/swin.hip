@@ -495,7 +495,7 @@ __device__ __forceinline__ void qchunk_mma(const unsigned char *buf, const half_
 // This workgroup's data of a hand-over are written: publish `val` in its flag word, then wait until
 // the window's four words have reached it.  Every thread calls it; the wait is bounded.
 __device__ __forceinline__ void quad_handover(unsigned *flags, unsigned *ctl, int win, int h, unsigned val) {
-  __builtin_amdgcn_s_waitcnt(0);                 // the write-through stores are acknowledged
+  wait_all_memory();                             // the write-through stores are acknowledged
   __syncthreads();
   if (threadIdx.x == 0) __hip_atomic_store(flags + win * 16 + h, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (threadIdx.x < 64) {
@@ -510,6 +510,7 @@ __device__ __forceinline__ void quad_handover(unsigned *flags, unsigned *ctl, in
     }
   }
   __syncthreads();
+  compiler_fence();                              // no load of the other three workgroups' rows is scheduled above the poll
 }
 
 // One block for one window, as workgroup h of its four.  fv: the flag value of this block's first hand-over.

@@ -92,8 +92,9 @@ SIGNATURES = {
                                              C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "souffle_bert_encoder_unfused": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
                                                C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
-    "souffle_bert_embed": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
-                                     C.c_float, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
+    "souffle_bert_embed": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
+                                     C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                     C.c_void_p]),
     "souffle_bert_pooler": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
     "souffle_lstm_workspace_bytes": (C.c_size_t, [C.POINTER(LstmCfg)]),
     "souffle_lstm_fused": (C.c_int, [C.POINTER(LstmCfg), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -92,20 +92,36 @@ def _block_w(w):
     return s
 
 
-def swin_block_pair(x, block0, block1, height=56, width=56, heads=4, window=7, shift=3, mlp_ratio=4,
-                    use_shift_mask=True, ln_eps=1e-5):
-    """Regular-window block followed by shifted-window block (Swin-Base stage 1 by default).
-    x: [H*W, C] fp16.  block0/block1: dicts with the keys of souffle_swin_block_w."""
+# grid-wide stages of the block-pair kernel that depend on one another (one grid barrier between the two blocks)
+BLOCK_PAIR_GRID_STAGES = 2
+
+
+def block_pair_launcher(x, block0, block1, out, height=56, width=56, heads=4, window=7, shift=3, mlp_ratio=4,
+                        use_shift_mask=True, ln_eps=1e-5):
+    """A closure that launches the block pair on preallocated buffers (x -> out) with one bare C-ABI call on the
+    current stream and raises on a non-zero status: for callers that time or replay the launch."""
     _check("x", x, (height * width, x.shape[-1]))
+    _check("out", out, tuple(x.shape))
     cfg = sh.SwinCfg(height, width, x.shape[-1], heads, window, shift, mlp_ratio, int(use_shift_mask), float(ln_eps))
     nbytes = sh.lib().souffle_swin_workspace_bytes(C.byref(cfg))
     if nbytes == 0:
         raise sh.SouffleError(-2, sh.last_error())
     ws = _ws(("pair", height, width), nbytes, x.device)
     arr = (sh.SwinBlockW * 2)(_block_w(block0), _block_w(block1))
-    y = torch.empty_like(x)
-    sh.check(sh.lib().souffle_swin_block_pair_fused(C.byref(cfg), arr, x.data_ptr(), y.data_ptr(), ws.ptr, ws.nbytes,
-                                                    sh.current_stream()))
+    fn, cfg_ref, xp, yp = sh.lib().souffle_swin_block_pair_fused, C.byref(cfg), x.data_ptr(), out.data_ptr()
+
+    def launch():
+        sh.check(fn(cfg_ref, arr, xp, yp, ws.ptr, ws.nbytes, sh.current_stream()))
+    launch._keep = (cfg, arr, ws, x, out)
+    return launch
+
+
+def swin_block_pair(x, block0, block1, height=56, width=56, heads=4, window=7, shift=3, mlp_ratio=4,
+                    use_shift_mask=True, ln_eps=1e-5, out=None):
+    """Regular-window block followed by shifted-window block (Swin-Base stage 1 by default).
+    x: [H*W, C] fp16.  block0/block1: dicts with the keys of souffle_swin_block_w."""
+    y = torch.empty_like(x) if out is None else out
+    block_pair_launcher(x, block0, block1, y, height, width, heads, window, shift, mlp_ratio, use_shift_mask, ln_eps)()
     return y
 
 
@@ -118,17 +134,28 @@ def index_maps(height, width, window, shift):
     return g, s, r.reshape(N, N), reg
 
 
-def patch_merging(x, height, width, norm_weight, norm_bias, reduction_weight, ln_eps=1e-5):
-    """Patch merging between two stages (python/models/swin_transformer/swin_patch_merge.py:3-13):
-    x [H*W, C] fp16 -> [(H/2)*(W/2), 2C]; norm_weight / norm_bias [4C] (None = 1 / 0),
-    reduction_weight [4C, 2C] (the transpose of torch's Linear weight, like every weight here)."""
+def patch_merge_launcher(x, height, width, norm_weight, norm_bias, reduction_weight, out, ln_eps=1e-5):
+    """A closure that launches patch merging on preallocated buffers with one bare C-ABI call on the current stream."""
     Cc = x.shape[-1]
     _check("x", x, (height * width, Cc))
     _check("reduction_weight", reduction_weight, (4 * Cc, 2 * Cc))
+    _check("out", out, ((height // 2) * (width // 2), 2 * Cc))
     for n, t in (("norm_weight", norm_weight), ("norm_bias", norm_bias)):
         if t is not None:
             _check(n, t, (4 * Cc,))
-    y = torch.empty(((height // 2) * (width // 2), 2 * Cc), dtype=torch.float16, device=x.device)
-    sh.check(sh.lib().souffle_swin_patch_merge(x.data_ptr(), sh.ptr(norm_weight), sh.ptr(norm_bias), reduction_weight.data_ptr(),
-                                               y.data_ptr(), height, width, Cc, float(ln_eps), sh.current_stream()))
+    fn = sh.lib().souffle_swin_patch_merge
+    a = (x.data_ptr(), sh.ptr(norm_weight), sh.ptr(norm_bias), reduction_weight.data_ptr(), out.data_ptr(), height, width, Cc, float(ln_eps))
+
+    def launch():
+        sh.check(fn(*a, sh.current_stream()))
+    launch._keep = (x, norm_weight, norm_bias, reduction_weight, out)
+    return launch
+
+
+def patch_merging(x, height, width, norm_weight, norm_bias, reduction_weight, ln_eps=1e-5, out=None):
+    """Patch merging between two stages (python/models/swin_transformer/swin_patch_merge.py:3-13):
+    x [H*W, C] fp16 -> [(H/2)*(W/2), 2C]; norm_weight / norm_bias [4C] (None = 1 / 0),
+    reduction_weight [4C, 2C] (the transpose of torch's Linear weight, like every weight here)."""
+    y = torch.empty(((height // 2) * (width // 2), 2 * x.shape[-1]), dtype=torch.float16, device=x.device) if out is None else out
+    patch_merge_launcher(x, height, width, norm_weight, norm_bias, reduction_weight, y, ln_eps)()
     return y

@@ -108,11 +108,21 @@ def test_embed_and_pooler_reject_bad_arguments_without_gpu():
     import ctypes as C
     import souffle_hip as sh
     lib = sh.lib()
-    assert lib.souffle_bert_embed(None, None, None, None, None, None, None, 1e-12, 1, 128, 768, None, None) == -1
-    assert lib.souffle_bert_embed(C.c_void_p(16), None, C.c_void_p(16), C.c_void_p(16), None, None, None, 1e-12, 1, 128, 512,
-                                  C.c_void_p(16), None) == -2 and "hidden=768" in sh.last_error()
-    assert lib.souffle_bert_embed(C.c_void_p(16), None, C.c_void_p(24), C.c_void_p(16), None, None, None, 1e-12, 1, 128, 768,
-                                  C.c_void_p(16), None) == -3
+    P = C.c_void_p
+    assert lib.souffle_bert_embed(None, None, None, 30522, None, 512, None, 2, None, None, 1e-12, 1, 128, 768, None, None, None) == -1
+    assert lib.souffle_bert_embed(P(16), None, P(16), 30522, P(16), 512, None, 0, None, None, 1e-12, 1, 128, 512,
+                                  P(16), None, None) == -2 and "hidden=768" in sh.last_error()
+    assert lib.souffle_bert_embed(P(16), None, P(24), 30522, P(16), 512, None, 0, None, None, 1e-12, 1, 128, 768,
+                                  P(16), None, None) == -3
+    # table sizes the host can judge: a position table shorter than the sequence, empty tables
+    assert lib.souffle_bert_embed(P(16), None, P(16), 30522, P(16), 64, None, 0, None, None, 1e-12, 1, 128, 768,
+                                  P(16), None, None) == -2 and "pos_emb has 64 rows" in sh.last_error()
+    assert lib.souffle_bert_embed(P(16), None, P(16), 0, P(16), 512, None, 0, None, None, 1e-12, 1, 128, 768,
+                                  P(16), None, None) == -2 and "vocab_size" in sh.last_error()
+    assert lib.souffle_bert_embed(P(16), P(16), P(16), 30522, P(16), 512, P(16), 0, None, None, 1e-12, 1, 128, 768,
+                                  P(16), None, None) == -2 and "type_vocab_size" in sh.last_error()
+    assert lib.souffle_bert_embed(P(16), None, P(16), 30522, P(16), 512, None, 0, None, None, 1e-12, 1, 128, 768,
+                                  P(16), P(18), None) == -3
     assert lib.souffle_bert_pooler(None, None, None, 1, 128, 768, None, None) == -1
     assert lib.souffle_bert_pooler(C.c_void_p(16), C.c_void_p(16), None, 0, 128, 768, C.c_void_p(16), None) == -2
 
@@ -131,6 +141,33 @@ def test_embed_gpu_matches_oracle(B, S, with_types):
                              dev(gam), dev(bet))
     torch.cuda.synchronize()
     assert_close("embeddings", got, ref)
+
+
+@pytest.mark.gpu
+def test_embed_gpu_clamps_and_counts_ids_outside_the_tables():
+    """Ids that a tokenizer for another vocabulary would produce: no row outside the tables is read (the kernel
+    clamps), the rows with good ids are unaffected, and the binding raises like host-side indexing would."""
+    import bert_binding
+    from gpu_util import announce, assert_close, dev
+    announce("bert embed with out-of-range ids")
+    B, S = 2, 64
+    word, pos, typ, gam, bet = _tables()
+    tok, seg = _ids(B, S, word.shape[0])
+    ref = oracle.bert_embed(tok, word, pos, typ, seg, gam, bet)
+    bad_tok, bad_seg = tok.copy(), seg.copy()
+    bad_tok[0, 3] = word.shape[0]
+    bad_tok[1, 7] = -5
+    bad_tok[1, 9] = 2 ** 31 - 1
+    bad_seg[0, 11] = typ.shape[0] + 4
+    di = lambda a: torch.from_numpy(a).to("cuda:0")
+    with pytest.raises(IndexError, match="4 token or segment ids"):
+        bert_binding.embed(di(bad_tok), dev(word), dev(pos), dev(typ), di(bad_seg), dev(gam), dev(bet))
+    got = bert_binding.embed(di(bad_tok), dev(word), dev(pos), dev(typ), di(bad_seg), dev(gam), dev(bet), check_ids=False)
+    torch.cuda.synchronize()
+    good = np.ones(B * S, dtype=bool)
+    good[[0 * S + 3, 1 * S + 7, 1 * S + 9, 0 * S + 11]] = False
+    assert_close("rows with ids inside the tables", got[torch.from_numpy(good).to("cuda:0")], ref.reshape(B * S, -1)[good])
+    assert torch.isfinite(got.float()).all()
 
 
 @pytest.mark.gpu
@@ -168,3 +205,10 @@ def test_embed_encoder_pooler_chain_gpu():
     y_ref = oracle.bert_encoder(e_ref, ws, B, S)
     assert_close("chain encoder output", y, y_ref)
     assert_close("chain pooled", pooled, oracle.bert_pooler(y_ref, pw, None, B, S))
+
+
+def test_erf_gelu_is_not_taken_for_the_tanh_form():
+    import bert_binding
+    with pytest.raises(ValueError, match="gelu_tanh"):
+        bert_binding.make_cfg(1, 128, act="gelu")
+    assert bert_binding.make_cfg(1, 128, act="gelu_tanh").act == bert_binding.make_cfg(1, 128).act

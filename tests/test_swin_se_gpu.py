@@ -112,7 +112,6 @@ def test_fused_feed_mlp(M, K, F):
     torch.cuda.synchronize()
     assert_close("fc1", y1, y1r)
     # the second GEMM consumes the fp16-rounded first output, as the reference kernel does
-    _, y2r = oracle.swin_ffn(np.zeros_like(x), w1, w2)
     y2r = oracle.gemm(y1.float().cpu().numpy(), w2)
     assert_close("fc2", y2, y2r)
 
