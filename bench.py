@@ -239,7 +239,8 @@ def bench_encoder(args, B, S, L, name):
     except sh.SouffleError as e:
         roof["measured_ceilings_error"] = str(e)
     # the same launch as a cooperative one (hipLaunchCooperativeKernel): the co-residency the hand-overs need is then
-    # guaranteed by the runtime instead of checked with the occupancy query
+    # guaranteed by the runtime instead of checked with the occupancy query.  Last GPU work of the process: memory
+    # re-used after cooperative launches was seen overwritten by what their ordinary stores had left in an L2.
     try:
         sh.set_cooperative_launch(1)
         _, coop_ev = time_steps(lambda i: encs[i % len(encs)](x, out=out), max(20, args.steps // 2), 5)
@@ -264,10 +265,10 @@ def main():
         print("no GPU available", file=sys.stderr)
         sys.exit(3)
     if args.workload == "encoder":
+        # (the sub-results first: the headline ends with cooperative launches, after which this process launches nothing)
+        sub = {} if args.no_sub else {"encoder_s384": encoder_sub_result(args, 1, 384), "encoder_b32": encoder_sub_result(args, 32, 128)}
         res = bench_encoder(args, 1, 128, 12, "BERT-base 12-layer encoder, B=1, S=128, fp16 (BASELINE configs[2], first shape)")
-        if not args.no_sub:
-            res["extra"]["encoder_s384"] = encoder_sub_result(args, 1, 384)
-            res["extra"]["encoder_b32"] = encoder_sub_result(args, 32, 128)
+        res["extra"].update(sub)
     elif args.workload == "layer":
         res = bench_encoder(args, 1, 128, 1, "single BERT-base encoder layer, B=1, S=128, fp16 (BASELINE configs[0])")
     elif args.workload == "encoder_s384":

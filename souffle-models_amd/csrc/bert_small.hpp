@@ -636,7 +636,7 @@ __device__ __forceinline__ void attn_item_split(unsigned char *lds, const AttnAr
     for (int tt = 0; tt < TPW; ++tt) {
       const f4 pr = sc[tt] * scale[wave];
       const h4 ph = {(half_t)pr[0], (half_t)pr[1], (half_t)pr[2], (half_t)pr[3]};
-      st8<false>(a.probs, (int)((((size_t)(b * NH + hh) * S + q) * S + (wave * TPW + tt) * 16 + g * 4) * 2), as_u2(ph));
+      st8<true>(a.probs, (int)((((size_t)(b * NH + hh) * S + q) * S + (wave * TPW + tt) * 16 + g * 4) * 2), as_u2(ph));
     }
   }
 }
@@ -884,7 +884,7 @@ __device__ __forceinline__ void run_red_item(const Args &a, int l, const It &d, 
   const float rstd = rsqrtf(sum32(cp < 12 ? pq + 64.0f * (pm - mean) * (pm - mean) : 0.f) * (1.0f / 768.0f) + a.eps);
   const h2 z = __builtin_bit_cast(h2, zraw);
   const float y0 = ((float)z[0] - mean) * rstd * (float)gv[0] + (float)ev[0], y1 = ((float)z[1] - mean) * rstd * (float)gv[1] + (float)ev[1];
-  if (a.ln1_out) *reinterpret_cast<h2 *>(a.ln1_out + (size_t)m * H + n) = h2{(half_t)y0, (half_t)y1};
+  if (a.ln1_out) st4<true>(a.ln1_out, (m * H + n) * 2, __builtin_bit_cast(unsigned, h2{(half_t)y0, (half_t)y1}));
   float v0 = 0.f, v1 = 0.f;
 #pragma unroll
   for (int k = 0; k < 4; ++k) { v0 += f32_of(pr[k][0]); v1 += f32_of(pr[k][1]); }
@@ -913,7 +913,9 @@ __device__ __forceinline__ void run_fin_item(const Args &a, const It &d) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] += (float)b8[i]; }
   const h8 o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3], (half_t)v[4], (half_t)v[5], (half_t)v[6], (half_t)v[7]};
-  st16<false>(a.y, (m * H + n) * 2, as_u4(o));
+  // (write-through like every store of this kernel: no line of it stays behind in an L2 when the launch ends, whatever the
+  // runtime does or does not write back between launches)
+  st16<true>(a.y, (m * H + n) * 2, as_u4(o));
 }
 
 // for every item of phase ph that belongs to workgroup b: fn(item, first)
