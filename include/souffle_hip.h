@@ -168,6 +168,18 @@ int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert
                                  const void *x, const void *mask, void *y,
                                  void *workspace, size_t workspace_bytes, souffle_stream_t stream);
 
+/* souffle_bert_encoder_fused without a workspace argument and without any allocation: the inter-phase
+ * buffers, flag words and control block live in a 48 MiB array in device memory that belongs to the
+ * library (one per GPU the library runs on, held until the process ends).  It has no counterpart in the
+ * reference; it is for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Same results as souffle_bert_encoder_fused.  A configuration whose
+ * workspace (souffle_bert_workspace_bytes) exceeds the array is refused with SOUFFLE_ERR_WORKSPACE
+ * (12 layers fit at up to 128 rows, fewer layers at more).  Every call on a GPU uses that GPU's one
+ * array: calls that overlap on one GPU (two streams, two threads) race, and the sticky failure word of
+ * the bounded waits cannot be read back through this entry point. */
+int souffle_bert_encoder_fused_static(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
+                                      const void *x, const void *mask, void *y, souffle_stream_t stream);
+
 /* The stage in front of the encoder: out[b*S+s] = LayerNorm(word_emb[token_ids[b*S+s]] +
  * pos_emb[s] + type_emb[segment_ids[b*S+s]]) in fp16, statistics in fp32.  Replaces the
  * HuggingFace embedding module the reference feeds its layer with

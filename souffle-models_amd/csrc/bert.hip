@@ -13,6 +13,7 @@
 //   7 reduce + bias + residual + LN2      [fused_sqq_feedforward.cu:368-835]
 // Softmax is max-subtracted fp32 and LayerNorm statistics are fp32 with a fixed summation order (no float
 // atomics), so results are run-to-run identical.
+#include <mutex>
 #include <type_traits>
 #include "bert_small.hpp"
 #include "gemm_tile.hpp"
@@ -1268,6 +1269,66 @@ extern "C" int souffle_bert_encoder_fused(const souffle_bert_cfg *cfg, const sou
   if (!cfg) return fail(SOUFFLE_ERR_NULL, "cfg is NULL");
   return bert::run_fused(cfg, layers, cfg->num_layers, x, mask, y, nullptr, ws, ws_bytes, stream);
 }
+// ---------------------------------------------------------------- the entry point that allocates nothing ----
+// The encoder's inter-phase buffers, flag words and control block in device memory that belongs to the library
+// instead of a caller's workspace: for callers that cannot allocate (under graph capture, in a serving loop).
+namespace souffle {
+namespace bert {
+constexpr size_t kStaticScratchBytes = (size_t)48 << 20;      // 12 layers at 128 rows need 42.8 MB
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device memory of `scratch` on the current device, looked up once per device (each device has its own copy of the
+// array at its own address; the array's name in host code is a stand-in, not an address), and the configuration of
+// the last call that used it there.
+struct StaticScratch { unsigned char *ptr; size_t cleared_for; };
+static int static_scratch(StaticScratch **out) {
+  constexpr int kMaxDevices = 64;
+  static StaticScratch per_device[kMaxDevices] = {};
+  static std::mutex mu;
+  int dev = -1;
+  SOUFFLE_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(SOUFFLE_ERR_DEVICE, "device index %d is not supported", dev);
+  std::lock_guard<std::mutex> lk(mu);
+  if (!per_device[dev].ptr) {
+    void *p = nullptr;
+    SOUFFLE_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(SOUFFLE_ERR_DEVICE, "the library's static scratch has no address on device %d", dev);
+    per_device[dev].ptr = static_cast<unsigned char *>(p);
+  }
+  *out = &per_device[dev];
+  return SOUFFLE_OK;
+}
+__global__ void __launch_bounds__(256) k_clear16(u4 *p, int n16) {
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < n16; i += gridDim.x * 256) p[i] = u4{0u, 0u, 0u, 0u};
+}
+}  // namespace bert
+}  // namespace souffle
+
+extern "C" int souffle_bert_encoder_fused_static(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
+                                                 const void *x, const void *mask, void *y, souffle_stream_t stream) {
+  if (!cfg) return fail(SOUFFLE_ERR_NULL, "cfg is NULL");
+  if (int rc = bert::validate(cfg)) return rc;
+  const int nl = cfg->num_layers;
+  if (nl < 1 || nl > bert::kMaxLayers) return fail(SOUFFLE_ERR_SHAPE, "num_layers must be in 1..%d (got %d)", bert::kMaxLayers, nl);
+  const bert::Plan p = bert::make_plan(cfg, nl);
+  if (p.total > bert::kStaticScratchBytes)
+    return fail(SOUFFLE_ERR_WORKSPACE, "batch %d x seq_len %d x %d layers needs %zu bytes of scratch, the library's static scratch holds %zu: "
+                "use souffle_bert_encoder_fused with a workspace", cfg->batch, cfg->seq_len, nl, p.total, bert::kStaticScratchBytes);
+  bert::StaticScratch *sc = nullptr;
+  if (int rc = bert::static_scratch(&sc)) return rc;
+  // The control block and the flag words (the first bytes, at the same place for every configuration) must start from
+  // zero when the layout behind them changes: they hold the previous call's barrier counts and flag values.  Between
+  // calls of one configuration they carry over, as in a caller's workspace.  A fill kernel, not a memset node.
+  const size_t key = ((size_t)cfg->batch << 40) ^ ((size_t)cfg->seq_len << 20) ^ (size_t)nl ^ ((size_t)1 << 62);
+  if (sc->cleared_for != key) {
+    const int n16 = (int)(p.off_qkv / 16);
+    hipLaunchKernelGGL(bert::k_clear16, dim3((n16 + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), reinterpret_cast<u4 *>(sc->ptr), n16);
+    SOUFFLE_HIP_TRY(hipGetLastError());
+    sc->cleared_for = key;
+  }
+  return bert::run_fused(cfg, layers, nl, x, mask, y, nullptr, sc->ptr, bert::kStaticScratchBytes, stream);
+}
+
 extern "C" int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
                                             const void *x, const void *mask, void *y, void *ws, size_t ws_bytes,
                                             souffle_stream_t stream) {
