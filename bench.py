@@ -39,6 +39,7 @@ def parse():
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU-baseline sample")
     p.add_argument("--no-cpu", action="store_true")
     p.add_argument("--no-sub", action="store_true", help="skip the S=384 and B=32 sub-results of the default workload")
+    p.add_argument("--no-coop", action="store_true", help="skip the cooperative-launch timing of the encoder workloads")
     p.add_argument("--weight-sets", type=int, default=4)
     return p.parse_args()
 
@@ -242,6 +243,8 @@ def bench_encoder(args, B, S, L, name):
     # guaranteed by the runtime instead of checked with the occupancy query.  Last GPU work of the process: memory
     # re-used after cooperative launches was seen overwritten by what their ordinary stores had left in an L2.
     try:
+        if args.no_coop:
+            raise sh.SouffleError(0, "skipped (--no-coop)")
         sh.set_cooperative_launch(1)
         _, coop_ev = time_steps(lambda i: encs[i % len(encs)](x, out=out), max(20, args.steps // 2), 5)
         res["extra"]["cooperative_launch_us"] = coop_ev * 1e3

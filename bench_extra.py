@@ -25,11 +25,11 @@ def _threads():
     return host_threads()
 
 
-def _kernel_us(launch):
+def _kernel_us(launch, args):
     """(min over rounds of the mean, median) of `launch()` in us, HIP events on the launch stream, the reference's
     timing rule (cpp/souffle_utils/cuda_utils.h:102-136).  `launch` is a bare C-ABI call on preallocated buffers."""
     import souffle_hip as sh
-    return sh.bench_us(launch, warmup=20, rounds=5, repeat=100)
+    return sh.bench_us(launch, warmup=min(20, max(2, args.warmup)), rounds=5, repeat=max(10, min(100, args.steps)))
 
 
 def _floor(extra, stages, launch_us):
@@ -112,7 +112,7 @@ def bench_swin(args):
                    "sample": "%d passes of the 56x56x128 block pair through oracle/swin_oracle.c (OpenMP fp32)" % n}
     launch = sb.block_pair_launcher(dx, dw[0], dw[1], torch.empty_like(dx))       # bare C-ABI call, output preallocated
     wall, ev = time_steps(lambda i: launch(), args.steps, args.warmup)
-    mn, med = _kernel_us(launch)
+    mn, med = _kernel_us(launch, args)
     flops = 2 * (2.0 * 3136 * 196608 + 4.0 * 64 * 4 * 49 * 49 * 32)
     ach = flops / (ev * 1e-3) / 1e12
     roof = {"bound": "mfma", "achieved": ach, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": ach / MFMA_F16_PEAK_TFLOPS,
@@ -137,9 +137,10 @@ def bench_se(args):
     for (Cc, Hh, R), ref_us in zip(shapes, a100):
         x = torch.rand((1, Cc, Hh, Hh), device="cuda:0")
         wr, we = torch.randn((R, Cc), device="cuda:0") * 0.3, torch.randn((Cc, R), device="cuda:0") * 0.3
+        print("se shape C=%d H=%d R=%d" % (Cc, Hh, R), file=sys.stderr, flush=True)
         launch = eb.se_launcher(x, wr, we, torch.empty_like(x), torch.empty((1, Cc), device="cuda:0"), combine="add")
         wall, ev = time_steps(lambda i: launch(), args.steps, args.warmup)
-        mn, med = _kernel_us(launch)
+        mn, med = _kernel_us(launch, args)
         rows.append({"C": Cc, "H": Hh, "R": R, "us": ev * 1e3, "kernel_us_min_of_means": mn, "reference_a100_us": ref_us,
                      "vs_reference_a100": ref_us / mn, "GBps": 2.0 * Cc * Hh * Hh * 4 / (mn * 1e-6) / 1e9})
     tot = sum(r["us"] for r in rows)
@@ -235,7 +236,7 @@ def bench_swin_merge(args):
                    "sample": "%d passes of the 56x56x128 patch merge through oracle/swin_oracle.c (OpenMP fp32)" % n}
     launch = sb.patch_merge_launcher(dx, H, W, dg, db, dw, torch.empty((H // 2 * (W // 2), 2 * Cc), dtype=torch.float16, device="cuda:0"))
     wall, ev = time_steps(lambda i: launch(), args.steps, args.warmup)
-    mn, med = _kernel_us(launch)
+    mn, med = _kernel_us(launch, args)
     bytes_alg = x.nbytes + w.nbytes + g.nbytes + b.nbytes + y.size * 2
     ach = bytes_alg / (ev * 1e-3) / 1e9
     roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
