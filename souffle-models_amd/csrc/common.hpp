@@ -214,17 +214,35 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 //    8-lane load until all have reached that number.
 // Counters and barrier numbers only grow (across launches too) and are compared as signed
 // differences, so a fast workgroup arriving at the next barrier never disturbs a slow one.
-// Control block (uint32 words, zeroed once before first use):
-//   [32*x]        arrival counter x              [256 + 32*x]  done flag x
-//   [384 + x]     value counter x holds between launches, [392] barrier number between launches:
-//                 rewritten by grid_barrier_end() (all workgroups read them before their first
-//                 arrival, nobody writes them before the last barrier of the launch has completed)
-//   [kCtlErrWord] sticky error flag for kernels with bounded spin loops (bit 0: LSTM wait,
-//                 bit 1: grid barrier or hand-over of the encoder)
+// Control block (uint32 words, zeroed once before first use); x = workgroup index % 8, the XCD it runs on:
+//   [kCtlArrive + 32 x]  arrival counter x        [kCtlDone + 32 x]  done flag x (number of the last barrier completed)
+//   [kCtlCarry + 32 x]   the value counter x holds between launches, [kCtlEpoch] the barrier number between launches:
+//                        rewritten by grid_barrier_end() (all workgroups read them before their first arrival,
+//                        nobody writes them before the last barrier of the launch has completed)
+//   [kCtlErrWord]        sticky error flag for kernels with bounded spin loops (bit 0: LSTM wait,
+//                        bit 1: grid barrier or hand-over of the encoder)
+// Every word has a place of its own (the assertions below): a done flag that shared its word with a carried counter
+// value would read as "completed" to every waiter, since counter values are far larger than barrier numbers.
 // Data exchanged across a barrier must be written with st*<true> (write-through); the barrier
 // itself carries no cache write-back or invalidate.
+constexpr int kCtlArrive = 0, kCtlDone = 256, kCtlCarry = 16, kCtlEpoch = 24;
 constexpr int kCtlWords = 512;
 constexpr int kCtlErrWord = 400;
+constexpr bool ctl_words_distinct() {
+  for (int x = 0; x < 8; ++x) {
+    const int w[3] = {kCtlArrive + 32 * x, kCtlDone + 32 * x, kCtlCarry + 32 * x};
+    for (int y = 0; y < 8; ++y) {
+      const int v[3] = {kCtlArrive + 32 * y, kCtlDone + 32 * y, kCtlCarry + 32 * y};
+      for (int i = 0; i < 3; ++i)
+        for (int j = 0; j < 3; ++j)
+          if ((x != y || i != j) && w[i] == v[j]) return false;
+    }
+    for (int i = 0; i < 3; ++i)
+      if (w[i] == kCtlEpoch || w[i] == kCtlErrWord || w[i] < 0 || w[i] >= 512) return false;
+  }
+  return kCtlEpoch != kCtlErrWord;
+}
+static_assert(ctl_words_distinct(), "two words of the control block share a place");
 constexpr int kMaxBarrierSpin = 1 << 20;       // about a second of polling; a barrier normally completes in microseconds
 
 struct GridBarrier {
@@ -265,8 +283,8 @@ __device__ __forceinline__ void grid_barrier_begin(GridBarrier &b, unsigned *ctl
   b.trace_cap = 0;
   const unsigned x = blockIdx.x & 7;
   b.gsz = (b.nblk + 7 - x) >> 3;
-  b.target = __hip_atomic_load(ctl + 384 + x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  b.epoch = __hip_atomic_load(ctl + 392, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  b.target = __hip_atomic_load(ctl + kCtlCarry + 32 * x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  b.epoch = __hip_atomic_load(ctl + kCtlEpoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // s_waitcnt with only the vector-memory counter: all but the youngest N vector memory
@@ -307,8 +325,8 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b, Mid mid) {
   b.epoch += 1;
   if (threadIdx.x == 0) {
     const unsigned x = blockIdx.x & 7;
-    const unsigned old = __hip_atomic_fetch_add(b.ctl + 32 * x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (old + 1 == b.target) __hip_atomic_store(b.ctl + 256 + 32 * x, b.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned old = __hip_atomic_fetch_add(b.ctl + kCtlArrive + 32 * x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old + 1 == b.target) __hip_atomic_store(b.ctl + kCtlDone + 32 * x, b.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __builtin_amdgcn_s_barrier();            // the arrival (and the done flag) precede whatever mid() queues
   mid();
@@ -316,7 +334,7 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b, Mid mid) {
     for (int spin = 0; spin < kMaxBarrierSpin; ++spin) {
       bool ok = true;
       if (threadIdx.x < 8 && threadIdx.x < b.nblk)
-        ok = (int)(__hip_atomic_load(b.ctl + 256 + 32 * threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - b.epoch) >= 0;
+        ok = (int)(__hip_atomic_load(b.ctl + kCtlDone + 32 * threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - b.epoch) >= 0;
       if (__all(ok)) break;
       __builtin_amdgcn_s_sleep(1);
       if (spin == kMaxBarrierSpin - 1) {   // gave up: the launch's output is invalid, and it ends without further waits
@@ -337,8 +355,8 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b) { grid_sync(b, []() {}
 // Call once by every workgroup before the kernel returns.
 __device__ __forceinline__ void grid_barrier_end(GridBarrier &b) {
   if (b.count > 0 && blockIdx.x < 8 && threadIdx.x == 0) {
-    __hip_atomic_store(b.ctl + 384 + blockIdx.x, b.target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (blockIdx.x == 0) __hip_atomic_store(b.ctl + 392, b.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(b.ctl + kCtlCarry + 32 * blockIdx.x, b.target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (blockIdx.x == 0) __hip_atomic_store(b.ctl + kCtlEpoch, b.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // The next launch on this control block reads these words first thing.  The wave does not end
     // before they are acknowledged, so that their arrival does not rest on what the end of a kernel
     // waits for when the runtime queues two launches without a cache release in between.
