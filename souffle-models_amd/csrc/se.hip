@@ -26,7 +26,8 @@ struct Args {
 };
 
 __global__ void __launch_bounds__(256) k_se(Args a) {
-  __shared__ float p_s[MAX_C];
+  __shared__ __attribute__((aligned(16))) float p_s[MAX_C];
+  __shared__ float u_s[4096];
   __shared__ float r_s[MAX_R];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int gw = blockIdx.x * 4 + wave, nw = gridDim.x * 4;
@@ -55,22 +56,60 @@ __global__ void __launch_bounds__(256) k_se(Args a) {
   }
   grid_sync(bar);
 
-  // pooled mean of every channel (all workgroups need all of it for the reduce layer)
+  // pooled mean of every channel (all workgroups need all of it for the reduce layer): the partial sums of all
+  // (channel, chunk) units are requested at once, 256 per round, and summed per channel out of LDS
+  {
+    constexpr int ROUNDS = 4096 / 256;
+    unsigned raw[ROUNDS];
+#pragma unroll
+    for (int i = 0; i < ROUNDS; ++i)
+      if (i * 256 < units) raw[i] = ld4<true>(a.part, min(tid + i * 256, units - 1) * 4);
+#pragma unroll
+    for (int i = 0; i < ROUNDS; ++i)
+      if (i * 256 < units && tid + i * 256 < units) u_s[tid + i * 256] = __uint_as_float(raw[i]);
+  }
+  __syncthreads();
   for (int c = tid; c < a.C; c += 256) {
     float s = 0.f;
-    for (int ch = 0; ch < a.chunks; ++ch) s += __uint_as_float(ld4<true>(a.part, (c * a.chunks + ch) * 4));
+    for (int ch = 0; ch < a.chunks; ++ch) s += u_s[c * a.chunks + ch];
     s *= 1.0f / a.HW;
     p_s[c] = s;
     if (blockIdx.x == 0 && a.pooled) a.pooled[c] = s;
   }
   __syncthreads();
-  // r = swish(W_r p + b_r)
-  for (int j = wave; j < a.R; j += 4) {
-    float s = 0.f;
-    for (int c = lane; c < a.C; c += 64) s += a.w_reduce[(size_t)j * a.C + c] * p_s[c];
-    s = wave_sum(s);
-    if (a.b_reduce) s += a.b_reduce[j];
-    if (lane == 0) r_s[j] = s / (1.0f + __expf(-s));
+  // r = swish(W_r p + b_r): wave w takes outputs w, w + 4, ..., four at a time so that their loads travel together;
+  // a lane takes four consecutive channels per load where C allows it
+  for (int j0 = wave; j0 < a.R; j0 += 16) {
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    if ((a.C & 3) == 0 && (reinterpret_cast<uintptr_t>(a.w_reduce) & 15u) == 0) {
+      const int c4n = a.C >> 2;
+#pragma unroll 2
+      for (int c4 = lane; c4 < c4n; c4 += 64) {
+        const f4 pv = *reinterpret_cast<const f4 *>(p_s + 4 * c4);
+        f4 wv[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          wv[q] = ldg<f4>(reinterpret_cast<const f4 *>(a.w_reduce + (size_t)min(j0 + 4 * q, a.R - 1) * a.C) + c4);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) s[q] += wv[q][0] * pv[0] + wv[q][1] * pv[1] + wv[q][2] * pv[2] + wv[q][3] * pv[3];
+      }
+    } else {
+#pragma unroll 4
+      for (int c = lane; c < a.C; c += 64) {
+        const float pv = p_s[c];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) s[q] += a.w_reduce[(size_t)min(j0 + 4 * q, a.R - 1) * a.C + c] * pv;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int j = j0 + 4 * q;
+      float t = wave_sum(s[q]);
+      if (j < a.R) {
+        if (a.b_reduce) t += a.b_reduce[j];
+        if (lane == 0) r_s[j] = t / (1.0f + __expf(-t));
+      }
+    }
   }
   __syncthreads();
   // e = sigmoid(W_e r + b_e) for this wave's channels, then combine with the held slice
