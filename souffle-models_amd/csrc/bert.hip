@@ -896,7 +896,7 @@ static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += round_up(bytes, 256); return o; };
   p.off_ctl = take(kCtlWords * 4);
-  p.off_flags = take(sk::kFlagWords * 4);              // (at a fixed place, whatever the configuration)
+  p.off_flags = take(sk::kFlagRegionWords * 4);        // (at a fixed place, whatever the configuration)
   const size_t first = off;
   p.off_qkv = take(3 * M * H * 2);
   p.off_ctx = take(M * H * 2);
@@ -1085,8 +1085,8 @@ static int run_small_unfused_t(sk::Args &a, int grid, hipStream_t st) {
     attr_done = true;
   }
   for (int l = 0; l < a.num_layers; ++l)
-    for (int ph = sk::PH_QKV; ph <= sk::PH_RED; ++ph) {
-      const int need = ph == sk::PH_ATT ? sk::attn_lds_bytes(a.S) : ph == sk::PH_RED ? 0 : sk::kLdsBytes;
+    for (int ph = sk::PH_QKV; ph <= sk::PH_FC2; ++ph) {
+      const int need = ph == sk::PH_ATT ? sk::attn_lds_bytes(a.S) : sk::kLdsBytes;
       hipLaunchKernelGGL(sk::k_small_phase<NKT>, dim3(grid), dim3(256), need, st, a, l, ph);
     }
   hipLaunchKernelGGL(sk::k_small_phase<NKT>, dim3(grid), dim3(256), 0, st, a, a.num_layers - 1, (int)sk::PH_FIN);

@@ -58,6 +58,15 @@ constexpr int kFlagCopies = 8, kFlagStride = 256;
 constexpr int kFlagBaseWord = kFlagCopies * kFlagStride;       // number the flags of this launch start from
 constexpr int kFlagDoneWord = kFlagBaseWord + 1;               // workgroups of the launch that have ended
 constexpr int kFlagWords = kFlagBaseWord + 64;
+// Behind the flag words: one word per 32 x 64 tile of the FC2 sum (m-tile * 12 + n-slice), again in 8 copies, which
+// the workgroup that completes the tile sets to the sequence number of (layer, RED); and per layer and tile a ticket
+// counter that the four workgroups of the tile's K quarters draw from (the one that draws the fourth ticket sums the
+// tile).  Counters only grow, by exactly four per launch and tile, so they need no clearing.
+constexpr int kTileWords = 384;                                  // 31 m-tiles x 12 n-slices at most, padded
+constexpr int kTileDoneWord = kFlagWords;                        // 8 copies of kTileWords
+constexpr int kTileCntWord = kTileDoneWord + kFlagCopies * kTileWords;          // kMaxLayers x kTileWords
+constexpr int kFlagRegionWords = kTileCntWord + kMaxLayers * kTileWords;
+static_assert(kFlagWords % 4 == 0 && kTileWords % 4 == 0, "16-byte polls");
 constexpr int kMaxFlagSpin = 1 << 21;                          // about a second of polling
 
 struct Shape {
@@ -192,14 +201,14 @@ __device__ __forceinline__ void publish(const Sync &sy, unsigned seq) {
   if (threadIdx.x < kFlagCopies)
     __hip_atomic_store(sy.flags + threadIdx.x * kFlagStride + blockIdx.x, seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// Wait until the workgroups named by `mask` (wave 0: 4 bits per lane) have published `seq` or something later.
-// Bounded: a wait that gives up flags the control block and ends all waiting of the launch.
-__device__ __forceinline__ void await(Sync &sy, unsigned mask, unsigned seq, int slot) {
+// Wait until the words named by `mask` (wave 0: lane i answers for words 4 i .. 4 i + 3 behind `words`, one bit
+// each) have reached `seq` or something later.  Bounded: a wait that gives up flags the control block and ends all
+// waiting of the launch.
+__device__ __forceinline__ void await_words(Sync &sy, const unsigned *words, unsigned mask, unsigned seq, int slot) {
   stamp_wait(sy, slot, 0);
   if (threadIdx.x < 64 && !sy.failed) {
-    const unsigned *copy = sy.flags + (blockIdx.x & (kFlagCopies - 1)) * kFlagStride;
     for (int spin = 0;; ++spin) {
-      const u4 f = ld16<true>(copy, (int)threadIdx.x * 16);
+      const u4 f = ld16<true>(words, (int)threadIdx.x * 16);
       bool ok = true;
 #pragma unroll
       for (int t = 0; t < 4; ++t) ok &= !((mask >> t) & 1u) || (int)(f[t] - seq) >= 0;
@@ -218,6 +227,14 @@ __device__ __forceinline__ void await(Sync &sy, unsigned mask, unsigned seq, int
 #endif
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+}
+// ... the workgroups named by `mask` (4 per lane) have published `seq`
+__device__ __forceinline__ void await(Sync &sy, unsigned mask, unsigned seq, int slot) {
+  await_words(sy, sy.flags + (blockIdx.x & (kFlagCopies - 1)) * kFlagStride, mask, seq, slot);
+}
+// ... the twelve 32 x 64 tiles of m-tile mt of the FC2 sum are complete (set by the workgroup that summed each)
+__device__ __forceinline__ void await_tiles(Sync &sy, int mt, unsigned seq, int slot) {
+  await_words(sy, sy.flags + kTileDoneWord + (blockIdx.x & (kFlagCopies - 1)) * kTileWords + mt * 12, threadIdx.x < 3 ? 15u : 0u, seq, slot);
 }
 
 // Sums over groups of neighbouring lanes with DPP moves (a few cycles each; a shuffle through the LDS crossbar
@@ -673,10 +690,11 @@ struct Job {
   const half_t *gam, *bet;             // of that LayerNorm
   const half_t *bias;                  // of the item's columns (LDS copy at kBiasOff), or null
   const half_t *rgam, *rbet;           // OUT: gamma / beta of the LayerNorm that produces the residual (LDS copies), or null
-  const half_t *res;                   // OUT: the residual rows [M][768] before that LayerNorm
-  const float *rstats;                 // OUT: their statistics, null = the residual is taken as it is (layer 0)
+  const half_t *res;                   // OUT, FC2: the residual rows [M][768] before that LayerNorm
+  const float *rstats;                 // their statistics, null = the residual is taken as it is (OUT of layer 0)
   half_t *out;                         // qkv / z1 / h of the layer
-  float *aux;                          // OUT: st1; FC2: the partial sums
+  float *aux;                          // FC2: the partial sums
+  float *stat_out;                     // OUT: statistics of z1; FC2: of z2 (written by the workgroup that sums the tile)
   int which, head;                     // QKV: q, k or v and the head; FC2: which = K quarter
   bool x_sc1;
 };
@@ -712,7 +730,7 @@ __device__ __forceinline__ Job make_job_t(const Args &a, int l, const It &d) {
       j.rgam = a.layers[l - 1].ln2_g; j.rbet = a.layers[l - 1].ln2_b;
       j.res = prev.z2; j.rstats = prev.st2;
     } else j.res = a.x;
-    j.out = cur.z1; j.aux = cur.st1;
+    j.out = cur.z1; j.stat_out = cur.st1;
   } else if constexpr (PH == PH_FC1) {
     j.g.W = w.w_fc1; j.g.ldw = F; j.g.kw0 = 0; j.g.n0 = d.b * 64;
     j.g.X = cur.z1; j.g.ldx = H; j.g.kx0 = 0;
@@ -727,6 +745,9 @@ __device__ __forceinline__ Job make_job_t(const Args &a, int l, const It &d) {
     j.g.W = w.w_fc2; j.g.ldw = H; j.g.kw0 = ks * 768; j.g.n0 = ns * 64;
     j.g.X = cur.h; j.g.ldx = F; j.g.kx0 = ks * 768;
     j.aux = cur.part;
+    // what the workgroup that completes the tile adds: bias, residual LN1(z1)
+    j.bias = w.b_fc2; j.res = cur.z1; j.rstats = cur.st1; j.rgam = w.ln1_g; j.rbet = w.ln1_b;
+    j.out = cur.z2; j.stat_out = cur.st2;
   }
   return j;
 }
@@ -740,7 +761,7 @@ __device__ __forceinline__ Job make_job(const Args &a, int l, int ph, const It &
 template <class T>
 __device__ __forceinline__ void keep_scalar(T *&p) { asm volatile("" : "+s"(p)); }
 __device__ __forceinline__ void pin(Job &j) {
-  keep_scalar(j.g.X); keep_scalar(j.stats); keep_scalar(j.res); keep_scalar(j.rstats); keep_scalar(j.out); keep_scalar(j.aux);
+  keep_scalar(j.g.X); keep_scalar(j.stats); keep_scalar(j.res); keep_scalar(j.rstats); keep_scalar(j.out); keep_scalar(j.aux); keep_scalar(j.stat_out);
 }
 // The loads of an item that depend on no other workgroup: weight slice, LayerNorm vectors, bias.
 __device__ __forceinline__ void issue_weights(unsigned char *lds, const Job &j, bool ahead) {
@@ -762,7 +783,7 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
   if (!w_ready) issue_weights(lds, j, false);
   // what the item reads of other workgroups' results, statistics first (they are needed first)
   if (j.ln != LN_NONE) issue_stats<4>(lds, j.stats, j.g.m0);
-  if constexpr (ph == PH_OUT) {
+  if constexpr (ph == PH_OUT || ph == PH_FC2) {
     const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
     // residual patch: rows m0 .. m0 + 31, columns n0 .. n0 + 63 -> [32][128 B] at kAuxOff
     dma16<true>(uniform_ptr(j.res + (size_t)(j.g.m0 + 8 * w) * H + j.g.n0), (unsigned)((lane >> 3) * H * 2 + (lane & 7) * 16),
@@ -793,6 +814,37 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       hi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]};
     }
   };
+  // A row of a pre-LayerNorm sum (8 columns per thread): + bias + the residual (normalised from its statistics when it
+  // is itself a pre-LayerNorm sum), rounded to fp16, written with the statistics of the rounded values.
+  auto finish_row = [&](int row, int col0, f4 lo, f4 hi, int slice, half_t *res_out) {
+    add_bias(col0, lo, hi);
+    const h8 rv = *reinterpret_cast<const h8 *>(lds + kAuxOff + row * 128 + col0 * 2);
+    f4 rlo = f4{(float)rv[0], (float)rv[1], (float)rv[2], (float)rv[3]}, rhi = f4{(float)rv[4], (float)rv[5], (float)rv[6], (float)rv[7]};
+    const int m = j.g.m0 + row;
+    if (j.rstats) {
+      const float *sp = reinterpret_cast<const float *>(lds + kAuxOff + 4096) + row * 24;
+      float mean = 0.f;
+#pragma unroll
+      for (int i = 0; i < 12; ++i) mean += sp[2 * i];
+      mean *= (1.0f / 12.0f);
+      float q = 0.f;
+#pragma unroll
+      for (int i = 0; i < 12; ++i) q += sp[2 * i + 1] + 64.0f * (sp[2 * i] - mean) * (sp[2 * i] - mean);
+      const float rstd = rsqrtf(q * (1.0f / 768.0f) + a.eps);
+      rlo = (rlo - mean) * rstd; rhi = (rhi - mean) * rstd;
+      if (j.rgam) { const h8 gg = *reinterpret_cast<const h8 *>(lds + kGamOff + col0 * 2); rlo *= f4{(float)gg[0], (float)gg[1], (float)gg[2], (float)gg[3]}; rhi *= f4{(float)gg[4], (float)gg[5], (float)gg[6], (float)gg[7]}; }
+      if (j.rbet) { const h8 bb = *reinterpret_cast<const h8 *>(lds + kGamOff + 128 + col0 * 2); rlo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]}; rhi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]}; }
+      if (res_out) st16<true>(res_out, (m * H + j.g.n0 + col0) * 2, pack_h8(rlo, rhi));      // (the normalised residual itself, on request)
+    }
+    lo += rlo; hi += rhi;
+    const u4 packed = pack_h8(lo, hi);
+    st16<true>(j.out, (m * H + j.g.n0 + col0) * 2, packed);
+    const h8 r8 = as_h8(packed);
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (float)r8[i];
+    put_stat<8, 8>(j.stat_out, m, slice, v, opaque_thread_id() & 7);
+  };
   if constexpr (ph == PH_QKV) {
     const int which = j.which, head = j.head;
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
@@ -801,34 +853,7 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       st16<true>(j.out, ((((which * a.B + b) * NH + head) * a.S + s) * HD + col0) * 2, pack_h8(lo, hi));
     });
   } else if constexpr (ph == PH_OUT) {
-    reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
-      add_bias(col0, lo, hi);
-      const h8 rv = *reinterpret_cast<const h8 *>(lds + kAuxOff + row * 128 + col0 * 2);
-      f4 rlo = f4{(float)rv[0], (float)rv[1], (float)rv[2], (float)rv[3]}, rhi = f4{(float)rv[4], (float)rv[5], (float)rv[6], (float)rv[7]};
-      if (j.rstats) {   // the residual is LN2 of the previous layer's sum: normalise the patch
-        const float *sp = reinterpret_cast<const float *>(lds + kAuxOff + 4096) + row * 24;
-        float mean = 0.f;
-#pragma unroll
-        for (int i = 0; i < 12; ++i) mean += sp[2 * i];
-        mean *= (1.0f / 12.0f);
-        float q = 0.f;
-#pragma unroll
-        for (int i = 0; i < 12; ++i) q += sp[2 * i + 1] + 64.0f * (sp[2 * i] - mean) * (sp[2 * i] - mean);
-        const float rstd = rsqrtf(q * (1.0f / 768.0f) + a.eps);
-        rlo = (rlo - mean) * rstd; rhi = (rhi - mean) * rstd;
-        if (j.rgam) { const h8 gg = *reinterpret_cast<const h8 *>(lds + kGamOff + col0 * 2); rlo *= f4{(float)gg[0], (float)gg[1], (float)gg[2], (float)gg[3]}; rhi *= f4{(float)gg[4], (float)gg[5], (float)gg[6], (float)gg[7]}; }
-        if (j.rbet) { const h8 bb = *reinterpret_cast<const h8 *>(lds + kGamOff + 128 + col0 * 2); rlo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]}; rhi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]}; }
-      }
-      lo += rlo; hi += rhi;
-      const int m = j.g.m0 + row;
-      const u4 packed = pack_h8(lo, hi);
-      st16<true>(j.out, (m * H + j.g.n0 + col0) * 2, packed);
-      const h8 r8 = as_h8(packed);
-      float v[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = (float)r8[i];
-      put_stat<8, 8>(j.aux, m, d.b, v, opaque_thread_id() & 7);
-    });
+    reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) { finish_row(row, col0, lo, hi, d.b, nullptr); });
   } else if constexpr (ph == PH_FC1) {
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
       add_bias(col0, lo, hi);
@@ -842,11 +867,48 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       st16<true>(j.out, ((j.g.m0 + row) * F + j.g.n0 + col0) * 2, pack_h8(lo, hi));
     });
   } else {
-    const int ks = j.which;
+    // FC2: the partial sum of this K quarter goes to memory; the four workgroups of a tile draw a ticket each once
+    // their partial sums are acknowledged, and the one that draws the last ticket adds the other three to its own
+    // (in the order of the quarters, whoever is last), finishes the rows (bias, residual LN1(z1), statistics) and
+    // marks the tile complete for the workgroups of the next layer.
+    const int ks = j.which, ns = d.b >> 2;
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
-      const int off = ((ks * a.M + j.g.m0 + row) * H + j.g.n0 + col0) * 4;
+      const int tid = opaque_thread_id();
+      const int m = j.g.m0 + row, off = ((ks * a.M + m) * H + j.g.n0 + col0) * 4;
       st16<true>(j.aux, off, __builtin_bit_cast(u4, lo));
       st16<true>(j.aux, off + 16, __builtin_bit_cast(u4, hi));
+      wait_all_memory();
+      __syncthreads();
+      unsigned *ticket_lds = reinterpret_cast<unsigned *>(lds + kBiasOff + 256);
+      if (tid == 0) {
+        unsigned *cnt = a.flags + kTileCntWord + (l * kTileWords + d.a * 12 + ns);
+        *ticket_lds = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __syncthreads();
+      const bool last = (*ticket_lds & 3u) == 3u;
+      compiler_fence();
+      if (!last) return;
+      f4 slo = {0.f, 0.f, 0.f, 0.f}, shi = {0.f, 0.f, 0.f, 0.f};
+      u4 plo[4], phi[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (k != ks) {
+          const int offk = ((k * a.M + m) * H + j.g.n0 + col0) * 4;
+          plo[k] = ld16<true>(j.aux, offk);
+          phi[k] = ld16<true>(j.aux, offk + 16);
+        }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        slo += k == ks ? lo : __builtin_bit_cast(f4, plo[k]);
+        shi += k == ks ? hi : __builtin_bit_cast(f4, phi[k]);
+      }
+      finish_row(row, col0, slo, shi, ns, a.ln1_out);
+      if (sy) {
+        wait_all_memory();
+        __syncthreads();
+        if (tid < kFlagCopies)
+          __hip_atomic_store(a.flags + kTileDoneWord + tid * kTileWords + d.a * 12 + ns, phase_seq(*sy, l, PH_RED), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     });
   }
 }
@@ -855,44 +917,6 @@ __device__ __forceinline__ void run_gemm_item(unsigned char *lds, const Args &a,
   else if (ph == PH_OUT) run_gemm_item_t<PH_OUT>(lds, a, l, d, j, w_ready, sy);
   else if (ph == PH_FC1) run_gemm_item_t<PH_FC1>(lds, a, l, d, j, w_ready, sy);
   else run_gemm_item_t<PH_FC2>(lds, a, l, d, j, w_ready, sy);
-}
-
-// RED: rows 8 ks .. 8 ks + 7 of the tile of FC2 item (m-tile, n-slice * 4 + ks): z2 = sum of the four partial sums
-// (in order) + bias + LN1(z1), rounded to fp16, and the statistics of those 64 values per row.
-// `pre` (the wait for the three sibling items) runs after the loads that need no sibling have been requested and
-// before anything is computed from them: they travel while the workgroup polls.
-template <class Pre>
-__device__ __forceinline__ void run_red_item(const Args &a, int l, const It &d, Pre pre) {
-  const LayerW &w = a.layers[l];
-  const Bufs cur = layer_bufs(a, l);
-  const int tid = opaque_thread_id(), row = tid >> 5, cp = tid & 31;
-  const int ks = d.b & 3, ns = d.b >> 2, m = d.a * 32 + ks * 8 + row, n = ns * 64 + 2 * cp;
-  // LN1 of the residual: twelve lanes of the row's 32 read one slice of its statistics each
-  u2 part_stat = {0u, 0u};
-  if (cp < 12) part_stat = ld8<true>(cur.st1, (m * 12 + cp) * 8);
-  const unsigned zraw = ld4<true>(cur.z1, (m * H + n) * 2);
-  h2 gv = {(half_t)1.f, (half_t)1.f}, ev = {(half_t)0.f, (half_t)0.f}, cv = {(half_t)0.f, (half_t)0.f};
-  if (w.ln1_g) gv = ldg<h2>(w.ln1_g + n);
-  if (w.ln1_b) ev = ldg<h2>(w.ln1_b + n);
-  if (w.b_fc2) cv = ldg<h2>(w.b_fc2 + n);
-  pre();
-  u2 pr[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) pr[k] = ld8<true>(cur.part, ((k * a.M + m) * H + n) * 4);
-  const float pm = cp < 12 ? f32_of(part_stat[0]) : 0.f, pq = f32_of(part_stat[1]);
-  const float mean = sum32(pm) * (1.0f / 12.0f);
-  const float rstd = rsqrtf(sum32(cp < 12 ? pq + 64.0f * (pm - mean) * (pm - mean) : 0.f) * (1.0f / 768.0f) + a.eps);
-  const h2 z = __builtin_bit_cast(h2, zraw);
-  const float y0 = ((float)z[0] - mean) * rstd * (float)gv[0] + (float)ev[0], y1 = ((float)z[1] - mean) * rstd * (float)gv[1] + (float)ev[1];
-  if (a.ln1_out) st4<true>(a.ln1_out, (m * H + n) * 2, __builtin_bit_cast(unsigned, h2{(half_t)y0, (half_t)y1}));
-  float v0 = 0.f, v1 = 0.f;
-#pragma unroll
-  for (int k = 0; k < 4; ++k) { v0 += f32_of(pr[k][0]); v1 += f32_of(pr[k][1]); }
-  v0 += (float)cv[0] + y0; v1 += (float)cv[1] + y1;
-  const h2 out = {(half_t)v0, (half_t)v1};
-  st4<true>(cur.z2, (m * H + n) * 2, __builtin_bit_cast(unsigned, out));
-  float vv[2] = {(float)out[0], (float)out[1]};
-  put_stat<2, 32>(cur.st2, m, ns, vv, cp);
 }
 
 // FIN: y = LN2 of the last layer's sum, a 32 x 64 patch per item.
@@ -973,7 +997,8 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
   {
     unsigned needs = 0;
     for (int ph = 0; ph <= PH_FIN; ++ph) {
-      needs |= (wait_needs(sh, ph, b, tid) ? 1u : 0u) << ph;
+      if (ph == PH_RED) continue;          // (the split-K sum is finished inside FC2, by the last of a tile's four workgroups)
+      if (ph != PH_QKV && ph != PH_FIN) needs |= (wait_needs(sh, ph, b, tid) ? 1u : 0u) << ph;      // (those two wait for tiles)
       mine_bits |= (has_items(sh, ph, b) ? 1u : 0u) << ph;
     }
     lds[tid] = (unsigned char)needs;
@@ -1025,7 +1050,7 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
     int rank = 0, peers = 0;                       // among the idle workgroups of this XCD
     for (int ob = b & 7; ob < sh.G; ob += 8) {
       bool idle = true;
-      for (int ph = 0; ph <= PH_FIN; ++ph) idle = idle && !has_items(sh, ph, ob);
+      for (int ph = 0; ph <= PH_FIN; ++ph) idle = idle && (ph == PH_RED || !has_items(sh, ph, ob));
       if (idle) { if (ob < b) ++rank; ++peers; }
     }
     int turn = 0;
@@ -1060,20 +1085,23 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
     pin(j0);
     const bool ready = pf == l * 8 + ph;
     pf = -1;
-    if (l > 0 || ph > PH_QKV) await(sy, wm(ph), phase_seq(sy, ph == PH_QKV ? l - 1 : l, producer_phase(ph)), l * PH_SLOTS + ph);
-    else if (ready) {                                         // (no wait in front of the very first phase)
-      if (tid >= 64) wait_vmcnt<0>();
-      __syncthreads();
-    }
+    if constexpr (ph == PH_QKV) {
+      if (l > 0) await_tiles(sy, f0.d.a, phase_seq(sy, l - 1, PH_RED), l * PH_SLOTS + ph);
+      else if (ready) {                                       // (no wait in front of the very first phase)
+        if (tid >= 64) wait_vmcnt<0>();
+        __syncthreads();
+      }
+    } else await(sy, wm(ph), phase_seq(sy, l, ph - 1), l * PH_SLOTS + ph);
     run_gemm_item_t<ph>(lds, args, l, f0.d, j0, ready, &sy);
     for_items_from(sh, ph, f0.it + sh.G, [&](const It &d) {
       __syncthreads();                                        // the partial tiles of the previous item have been read
+      if (ph == PH_QKV && l > 0) await_tiles(sy, d.a, phase_seq(sy, l - 1, PH_RED), sy.trace_cap);      // (its own m-tile)
       run_gemm_item_t<ph>(lds, args, l, d, make_job_t<ph>(args, l, d), false, &sy);
     });
     stamp_mark(sy, l * PH_SLOTS + ph, 2);
     publish(sy, phase_seq(sy, l, ph));
     stamp_mark(sy, l * PH_SLOTS + ph, 3);
-    if (!(ph == PH_FC2 && mine(PH_RED))) prefetch_after(l, phc);   // (RED follows FC2 at once: the request waits until after it)
+    prefetch_after(l, phc);
   };
   prefetch_after(0, std::integral_constant<int, -1>{});
 #pragma unroll 1
@@ -1092,24 +1120,12 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
     gemm_phase(l, std::integral_constant<int, PH_OUT>{});
     gemm_phase(l, std::integral_constant<int, PH_FC1>{});
     gemm_phase(l, std::integral_constant<int, PH_FC2>{});
-    if (mine(PH_RED)) {
-      bool waited = false;
-      for_items(sh, PH_RED, b, [&](const It &d, bool) {
-        run_red_item(args, l, d, [&]() {
-          if (!waited) await(sy, wm(PH_RED), phase_seq(sy, l, PH_FC2), l * PH_SLOTS + PH_RED);
-          waited = true;
-        });
-      });
-      stamp_mark(sy, l * PH_SLOTS + PH_RED, 2);
-      publish(sy, phase_seq(sy, l, PH_RED));
-      stamp_mark(sy, l * PH_SLOTS + PH_RED, 3);
-      if (pf < 0) prefetch_after(l, std::integral_constant<int, PH_RED>{});
-    }
   }
-  if (mine(PH_FIN)) {
-    await(sy, wm(PH_FIN), phase_seq(sy, L - 1, PH_RED), (L - 1) * PH_SLOTS + PH_FIN);
-    for_items(sh, PH_FIN, b, [&](const It &d, bool) { run_fin_item(args, d); });
-  }
+  if (mine(PH_FIN))
+    for_items(sh, PH_FIN, b, [&](const It &d, bool first) {
+      await_tiles(sy, d.a, phase_seq(sy, L - 1, PH_RED), first ? (L - 1) * PH_SLOTS + PH_FIN : sy.trace_cap);
+      run_fin_item(args, d);
+    });
   sync_end(sy, L);
 }
 
@@ -1123,8 +1139,6 @@ __global__ void __launch_bounds__(256) k_small_phase(Args args, int l, int ph) {
   if (ph == PH_ATT) {
     const AttnArgs aa = attn_args(args, l);
     for_items(sh, ph, b, [&](const It &d, bool) { attn_item_split<NKT>(lds, aa, d.b, d.a); });
-  } else if (ph == PH_RED) {
-    for_items(sh, ph, b, [&](const It &d, bool) { run_red_item(args, l, d, []() {}); });
   } else if (ph == PH_FIN) {
     for_items(sh, ph, b, [&](const It &d, bool) { run_fin_item(args, d); });
   } else {
