@@ -215,7 +215,7 @@ def bench_encoder(args, B, S, L, name):
                   "unfused_per_op_us": unf_ev * 1e3, "fused_speedup_vs_unfused": unf_ev / cold_ev,
                   "unfused_per_op_hip_graph_us": None if graph_ev is None else graph_ev * 1e3,
                   "min_of_means_us_warm": mn, "median_us_warm": med, "parity": parity,
-                  "launches_fused": 1, "launches_unfused": (6 if M < 1024 else 7) * L},
+                  "launches_fused": 1, "launches_unfused": 5 * L + 1 if M < 1024 else 7 * L},
     }
     # empirical ceilings of this device beside the published ones: device-to-device copy and an MFMA-only loop
     try:
@@ -227,10 +227,11 @@ def bench_encoder(args, B, S, L, name):
         if (B, S) == (1, 384):            # mixed shape: both fractions
             roof["mfma_frac"] = flops / (cold_ev * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS
         if few_rows:
-            # Six phases per layer (QKV, attention, out-projection, FC1, FC2, split-K reduction) and the final
-            # LayerNorm follow one another through flag hand-overs among the workgroups that exchange data; no grid
-            # barrier.  The yardstick beside it: a chain of as many grid-wide stages with no arithmetic at all.
-            nst = 6 * L + 1
+            # Five phases per layer (QKV, attention, out-projection, FC1, FC2 with the split-K sum finished by the last
+            # of a tile's four workgroups) and the final LayerNorm follow one another through flag hand-overs among the
+            # workgroups that exchange data; no grid barrier.  The yardstick beside it: a chain of as many grid-wide
+            # stages with no arithmetic at all.
+            nst = 5 * L + 1
             bar_us, floor_us = sh.stage_floor_us(nst)
             res["extra"]["stages_per_launch"] = nst
             res["extra"]["grid_barriers_per_launch"] = 0

@@ -990,27 +990,10 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
   sync_begin(sy, args.flags, args.ctl + kCtlErrWord, args.trace, args.trace_cap);
   const int L = args.num_layers;
   stamp_wait(sy, PH_SLOTS - 1, 0);          // (slot 7 of layer 0 is no phase: start of the kernel, end of its set-up)
-  // Who feeds whom (wave 0: 4 workgroups per lane, one nibble per phase) and in which phases this workgroup
-  // has items (one bit per phase); packed into words so that the phase loop indexes no register array.
-  // Thread t answers for producer workgroup t; the answers travel through LDS to the lanes of wave 0.
+  // In which phases this workgroup has items (one bit per phase; packed so that the phase code indexes no register array).
   unsigned wm_all = 0, mine_bits = 0;
-  {
-    unsigned needs = 0;
-    for (int ph = 0; ph <= PH_FIN; ++ph) {
-      if (ph == PH_RED) continue;          // (the split-K sum is finished inside FC2, by the last of a tile's four workgroups)
-      if (ph != PH_QKV && ph != PH_FIN) needs |= (wait_needs(sh, ph, b, tid) ? 1u : 0u) << ph;      // (those two wait for tiles)
-      mine_bits |= (has_items(sh, ph, b) ? 1u : 0u) << ph;
-    }
-    lds[tid] = (unsigned char)needs;
-    __syncthreads();
-    if (tid < 64) {
-      const unsigned four = *reinterpret_cast<const unsigned *>(lds + 4 * tid);
-      for (int ph = 0; ph <= PH_FIN; ++ph)
-        for (int t = 0; t < 4; ++t) wm_all |= ((four >> (8 * t + ph)) & 1u) << (4 * ph + t);
-    }
-    __syncthreads();
-  }
-  stamp_wait(sy, PH_SLOTS - 1, 1);
+  for (int ph = 0; ph <= PH_FIN; ++ph)
+    if (ph != PH_RED) mine_bits |= (has_items(sh, ph, b) ? 1u : 0u) << ph;       // (the split-K sum is finished inside FC2)
   auto mine = [&](int ph) { return ((mine_bits >> ph) & 1u) != 0; };
   auto wm = [&](int ph) { return (wm_all >> (4 * ph)) & 15u; };
   // The first item of each GEMM phase (at up to 256 rows there is no second one): found once, not per layer.
@@ -1104,6 +1087,22 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
     prefetch_after(l, phc);
   };
   prefetch_after(0, std::integral_constant<int, -1>{});
+  // Who feeds whom (wave 0: 4 workgroups per lane, one nibble per phase), worked out while the first weight slice
+  // travels.  Thread t answers for producer workgroup t; the answers reach the lanes of wave 0 through LDS (the start
+  // of the X region, which nothing has been requested into yet).  QKV and FIN wait for tiles, not for workgroups.
+  if (mine_bits != 0) {
+    unsigned needs = 0;
+    for (int ph = PH_ATT; ph <= PH_FC2; ++ph) needs |= (wait_needs(sh, ph, b, tid) ? 1u : 0u) << ph;
+    lds[tid] = (unsigned char)needs;
+    __syncthreads();
+    if (tid < 64) {
+      const unsigned four = *reinterpret_cast<const unsigned *>(lds + 4 * tid);
+      for (int ph = PH_ATT; ph <= PH_FC2; ++ph)
+        for (int t = 0; t < 4; ++t) wm_all |= ((four >> (8 * t + ph)) & 1u) << (4 * ph + t);
+    }
+    __syncthreads();
+  }
+  stamp_wait(sy, PH_SLOTS - 1, 1);
 #pragma unroll 1
   for (int l = 0; l < L; ++l) {
     gemm_phase(l, std::integral_constant<int, PH_QKV>{});
