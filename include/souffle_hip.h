@@ -180,6 +180,16 @@ int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert
 int souffle_bert_encoder_fused_static(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
                                       const void *x, const void *mask, void *y, souffle_stream_t stream);
 
+/* The work split and the hand-over plan of the encoder below 1024 rows, evaluated on the host by the functions the
+ * kernel itself uses (no GPU needed; no counterpart in the reference, whose stages are separated by grid barriers):
+ * the items of `workgroup` in `phase` (0 QKV, 1 attention, 2 out-projection, 3 FC1, 4 FC2, 6 final LayerNorm) as
+ * pairs (m-tile, weight slice) - attention: (block of 16 queries, batch * 12 + head) - written to items[2 i], items[2 i + 1]
+ * (at most max_items pairs; *n_items is their true number), and needs[p] = 1 for every workgroup p of the `grid` whose
+ * publication of the phase before the workgroup waits for (phases 1..4; QKV and the final LayerNorm wait for the
+ * completion words of the twelve FC2 tiles of their m-tile instead).  items and needs may be NULL. */
+int souffle_bert_handover_plan(int batch, int seq_len, int grid, int phase, int workgroup, int *items, int max_items,
+                               int *n_items, unsigned char *needs);
+
 /* The stage in front of the encoder: out[b*S+s] = LayerNorm(word_emb[token_ids[b*S+s]] +
  * pos_emb[s] + type_emb[segment_ids[b*S+s]]) in fp16, statistics in fp32.  Replaces the
  * HuggingFace embedding module the reference feeds its layer with

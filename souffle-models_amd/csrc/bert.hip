@@ -1329,6 +1329,31 @@ extern "C" int souffle_bert_encoder_fused_static(const souffle_bert_cfg *cfg, co
   return bert::run_fused(cfg, layers, nl, x, mask, y, nullptr, sc->ptr, bert::kStaticScratchBytes, stream);
 }
 
+// The work split and the hand-over plan of the few-rows encoder, evaluated on the host with the very functions the
+// kernel uses: for tests that check the plan against a model of which rows and columns every item reads and writes.
+extern "C" int souffle_bert_handover_plan(int batch, int seq_len, int grid, int phase, int workgroup, int *items, int max_items,
+                                          int *n_items, unsigned char *needs) {
+  namespace sk = bert::sk;
+  if (!n_items) return fail(SOUFFLE_ERR_NULL, "n_items is NULL");
+  if (batch <= 0 || (seq_len != 64 && seq_len != 128 && seq_len != 256 && seq_len != 384 && seq_len != 512) || (long long)batch * seq_len >= 1024)
+    return fail(SOUFFLE_ERR_SHAPE, "the few-rows plan exists for seq_len in {64,128,256,384,512} and fewer than 1024 rows (got %d x %d)", batch, seq_len);
+  if (grid <= 0 || grid > 1024 || workgroup < 0 || workgroup >= grid) return fail(SOUFFLE_ERR_SHAPE, "grid must be in 1..1024 and workgroup below it");
+  if (phase < sk::PH_QKV || phase > sk::PH_FIN || phase == sk::PH_RED) return fail(SOUFFLE_ERR_SHAPE, "phase must be 0 (QKV), 1 (ATT), 2 (OUT), 3 (FC1), 4 (FC2) or 6 (FIN)");
+  const sk::Shape sh{batch, seq_len, batch * seq_len, batch * seq_len / 32, grid};
+  int n = 0;
+  for (int it = workgroup - sk::ph_off(sh, phase); it < sk::ph_span(sh, phase); it += grid) {
+    sk::It d;
+    if (it < 0 || !sk::ph_item(sh, phase, it, d)) continue;
+    if (items && n < max_items) { items[2 * n] = d.a; items[2 * n + 1] = d.b; }
+    ++n;
+  }
+  *n_items = n;
+  if (needs)
+    for (int pb = 0; pb < grid; ++pb)
+      needs[pb] = (phase >= sk::PH_ATT && phase <= sk::PH_FC2 && sk::wait_needs(sh, phase, workgroup, pb)) ? 1 : 0;
+  return SOUFFLE_OK;
+}
+
 extern "C" int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
                                             const void *x, const void *mask, void *y, void *ws, size_t ws_bytes,
                                             souffle_stream_t stream) {

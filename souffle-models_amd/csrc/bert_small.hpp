@@ -114,37 +114,37 @@ __device__ __forceinline__ unsigned u32_of(float v) { return __builtin_bit_cast(
 // ---- item numbering ----
 // Workgroup b runs on XCD b % 8 (each XCD has its own L2).  The m-tiles that share one weight slice are dealt to
 // workgroups of ONE XCD in the same pass, so the slice crosses the fabric once per XCD.
-__device__ __forceinline__ bool xcd_item(int G, int it, int m_tiles, int w_slices, int *mt, int *ws) {
+__host__ __device__ __forceinline__ bool xcd_item(int G, int it, int m_tiles, int w_slices, int *mt, int *ws) {
   if ((G & 7) != 0) { *mt = it % m_tiles; *ws = it / m_tiles; return it < m_tiles * w_slices; }
   const int xcd = it & 7, j = it >> 3;
   *mt = j % m_tiles;
   *ws = (j / m_tiles) * 8 + xcd;
   return *ws < w_slices;
 }
-__device__ __forceinline__ int xcd_item_span(int G, int m_tiles, int w_slices) {   // exclusive upper bound of valid `it`
+__host__ __device__ __forceinline__ int xcd_item_span(int G, int m_tiles, int w_slices) {   // exclusive upper bound of valid `it`
   return (G & 7) != 0 ? m_tiles * w_slices : ((w_slices + 7) >> 3) * m_tiles * 8;
 }
 struct It { int a, b; };     // GEMM phases: (m-tile, slice); ATT: (16-query block, batch * 12 + head)
-__device__ __forceinline__ int ph_slices(int ph) { return ph == PH_QKV ? 36 : (ph == PH_OUT || ph == PH_FIN) ? 12 : 48; }
-__device__ __forceinline__ int ph_span(const Shape &s, int ph) {
+__host__ __device__ __forceinline__ int ph_slices(int ph) { return ph == PH_QKV ? 36 : (ph == PH_OUT || ph == PH_FIN) ? 12 : 48; }
+__host__ __device__ __forceinline__ int ph_span(const Shape &s, int ph) {
   return ph == PH_ATT ? xcd_item_span(s.G, s.S / 16, s.B * 12) : xcd_item_span(s.G, s.m_tiles, ph_slices(ph));
 }
 // Attention items go to workgroups 64.. when there is room, so that the workgroups of the out-projection
 // (the first ones) have their LDS free for the weight slice meanwhile.
-__device__ __forceinline__ int ph_off(const Shape &s, int ph) { return (ph == PH_ATT && ph_span(s, ph) + 64 <= s.G) ? 64 : 0; }
-__device__ __forceinline__ bool ph_item(const Shape &s, int ph, int it, It &d) {
+__host__ __device__ __forceinline__ int ph_off(const Shape &s, int ph) { return (ph == PH_ATT && ph_span(s, ph) + 64 <= s.G) ? 64 : 0; }
+__host__ __device__ __forceinline__ bool ph_item(const Shape &s, int ph, int it, It &d) {
   if (ph == PH_ATT) return xcd_item(s.G, it, s.S / 16, s.B * 12, &d.a, &d.b);
   return xcd_item(s.G, it, s.m_tiles, ph_slices(ph), &d.a, &d.b);
 }
 // items of workgroup b: it = b - off, b - off + G, ... below the span
-__device__ __forceinline__ bool has_items(const Shape &s, int ph, int b) {
+__host__ __device__ __forceinline__ bool has_items(const Shape &s, int ph, int b) {
   It d;
   for (int it = b - ph_off(s, ph); it < ph_span(s, ph); it += s.G)
     if (it >= 0 && ph_item(s, ph, it, d)) return true;
   return false;
 }
 // Does producer item p (of the phase that feeds phase cph) write something that consumer item c reads?
-__device__ __forceinline__ bool feeds(const Shape &s, int cph, const It &c, const It &p) {
+__host__ __device__ __forceinline__ bool feeds(const Shape &s, int cph, const It &c, const It &p) {
   switch (cph) {
     case PH_ATT: {        // p = QKV (m-tile, q/k/v * 12 + head); c = (query block, batch * 12 + head)
       const int b = c.b / 12, h = c.b % 12, j = p.b / 12, head = p.b % 12;
@@ -156,12 +156,12 @@ __device__ __forceinline__ bool feeds(const Shape &s, int cph, const It &c, cons
     default: return p.a == c.a;                                                    // QKV <- RED, FC1 <- OUT, FIN <- RED
   }
 }
-__device__ __forceinline__ int producer_phase(int cph) { return cph == PH_QKV ? PH_RED : cph == PH_FIN ? PH_RED : cph - 1; }
+__host__ __device__ __forceinline__ int producer_phase(int cph) { return cph == PH_QKV ? PH_RED : cph == PH_FIN ? PH_RED : cph - 1; }
 
 // Must workgroup pb have published the producer phase before workgroup b may start its items of phase cph?
 // Exact where both phases are a single pass over the grid; otherwise every workgroup that has an item of the
 // producer phase.
-__device__ bool wait_needs(const Shape &s, int cph, int b, int pb) {
+__host__ __device__ inline bool wait_needs(const Shape &s, int cph, int b, int pb) {
   const int pph = producer_phase(cph);
   const bool fine = ph_span(s, pph) + ph_off(s, pph) <= s.G && ph_span(s, cph) + ph_off(s, cph) <= s.G;
   if (pb >= s.G) return false;
