@@ -159,17 +159,21 @@ __host__ __device__ __forceinline__ bool feeds(const Shape &s, int cph, const It
 __host__ __device__ __forceinline__ int producer_phase(int cph) { return cph == PH_QKV ? PH_RED : cph == PH_FIN ? PH_RED : cph - 1; }
 
 // Must workgroup pb have published the producer phase before workgroup b may start its items of phase cph?
-// Exact where both phases are a single pass over the grid; otherwise every workgroup that has an item of the
-// producer phase.
+// Yes if any item of pb in the producer phase writes something that any item of b in phase cph reads (a workgroup
+// waits once per phase, for all its items; with more items than workgroups each has up to three).
 __host__ __device__ inline bool wait_needs(const Shape &s, int cph, int b, int pb) {
   const int pph = producer_phase(cph);
-  const bool fine = ph_span(s, pph) + ph_off(s, pph) <= s.G && ph_span(s, cph) + ph_off(s, cph) <= s.G;
   if (pb >= s.G) return false;
-  if (!fine) return has_items(s, cph, b) && has_items(s, pph, pb);
-  It c, p;
-  const int cit = b - ph_off(s, cph), pit = pb - ph_off(s, pph);
-  if (!(cit >= 0 && cit < ph_span(s, cph) && ph_item(s, cph, cit, c))) return false;
-  return pit >= 0 && pit < ph_span(s, pph) && ph_item(s, pph, pit, p) && feeds(s, cph, c, p);
+  const int cspan = ph_span(s, cph), pspan = ph_span(s, pph);
+  for (int cit = b - ph_off(s, cph); cit < cspan; cit += s.G) {
+    It c;
+    if (cit < 0 || !ph_item(s, cph, cit, c)) continue;
+    for (int pit = pb - ph_off(s, pph); pit < pspan; pit += s.G) {
+      It p;
+      if (pit >= 0 && ph_item(s, pph, pit, p) && feeds(s, cph, c, p)) return true;
+    }
+  }
+  return false;
 }
 
 // ---- hand-over ----
