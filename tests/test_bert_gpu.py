@@ -193,6 +193,32 @@ def test_few_rows_handovers_on_repeated_launches(B, S, layers):
     assert_close("encoder x1", z_1, oracle.bert_encoder(x1, ws, B, S))
 
 
+def test_few_rows_shapes_take_turns_in_one_workspace():
+    """Flag words, ticket counters and completion words of the few-rows kernel carry over from launch to launch
+    and are indexed by shape-dependent tile numbers: encoders of different shapes and depths, fused and per-op,
+    that take turns in ONE workspace must each give what they give in a workspace of their own."""
+    announce("bert encoder few rows, several shapes sharing a workspace")
+    import bert_binding
+    ws = [synth.bert_layer_weights(6, l, with_bias=True) for l in range(4)]
+    dws = [dev_weights(w) for w in ws]
+    cases = [(1, 128, 4), (2, 64, 2), (1, 256, 3), (3, 128, 1), (1, 384, 2), (1, 128, 4)]
+    encs, xs, want = [], [], []
+    for B, S, layers in cases:
+        enc = bert_binding.Encoder(dws[:layers], B, S)
+        x = dev(synth.bert_input(7, B, S))
+        want.append(enc(x).clone())
+        encs.append(enc)
+        xs.append(x)
+    shared = max(encs, key=lambda e: e.ws.nbytes).ws
+    for e in encs:
+        e.ws = shared
+    for rnd in range(3):
+        for i, (e, x) in enumerate(zip(encs, xs)):
+            got = e(x, fused=(rnd + i) % 3 != 2).clone()
+            assert torch.equal(got, want[i]), "round %d, case %s" % (rnd, cases[i])
+    assert shared.status() == 0
+
+
 @pytest.mark.parametrize("B,S", [(1, 128), (1, 384), (8, 128)])
 def test_layernorm_of_rows_far_from_zero(B, S):
     """Rows whose mean is far larger than their spread, and feature columns of large magnitude: the LayerNorm
