@@ -1,18 +1,20 @@
 // BERT-base encoder, few rows (batch * seq_len < 1024): the weight-stream-bound shapes.
 //
-// A layer is six phases, each a set of independent items dealt to the workgroups of one persistent launch:
+// A layer is five phases, each a set of independent items dealt to the workgroups of one persistent launch:
 //   QKV  (m-tile, 64 of the 2304 q/k/v columns)   X = layer input (layer 0) or LN2 of the previous layer's sum
 //   ATT  (head, 16 queries)                       scores, softmax and P.V; keys split over the waves
 //   OUT  (m-tile, 64 of 768 columns)              z1 = ctx.Wo + b + x, fp16, plus row statistics of its 64 columns
 //   FC1  (m-tile, 64 of 3072 columns)             h = act(LN1(z1).W1 + b)
-//   FC2  (m-tile, 64 of 768 columns, K quarter)   fp32 partial sums
-//   RED  (the same item, 8 of its 32 rows)        z2 = sum of the 4 partials + b + LN1(z1), fp16, plus row statistics
-// and after the last layer FIN (m-tile, 64 columns): y = LN2(z2).
+//   FC2  (m-tile, 64 of 768 columns, K quarter)   fp32 partial sum; the last of a tile's four workgroups to finish adds
+//                                                 the four, the bias and LN1(z1): z2, fp16, plus row statistics
+// and after the last layer FIN (m-tile, 64 columns): y = LN2(z2).  (PH_RED names the completion of that sum: it has a
+// sequence number, which the completion words of the tiles carry, but no items of its own.)
 //
 // There is no grid barrier.  A workgroup that has finished its items of a phase waits for the acknowledgement of
 // its write-through stores and publishes the number of that phase in its flag word; a consumer polls the flag
 // words of exactly the workgroups that produce what its items read (9 to 48 of them; which ones follows from the
-// item numbering and is worked out once per launch).  Flag words exist in eight copies, one per XCD, so that a
+// item numbering and is worked out once per launch; the consumers of the FC2 sum poll one completion word per
+// 32 x 64 tile instead, written by whichever workgroup summed the tile).  Flag words exist in eight copies, one per XCD, so that a
 // line is polled by the 32 workgroups of one XCD only: measured 1.65 us per hand-over against 2.25 us for the
 // grid barrier with per-XCD counters, 3.8 us with a single copy.
 //
@@ -152,11 +154,11 @@ __host__ __device__ __forceinline__ bool feeds(const Shape &s, int cph, const It
     }
     case PH_OUT: return ((p.b / 12) * s.S + 16 * p.a) / 32 == c.a;                 // p = ATT
     case PH_FC2: return p.a == c.a && p.b / 12 == (c.b & 3);                       // p = FC1 slice, c = n-slice * 4 + K quarter
-    case PH_RED: return p.a == c.a && (p.b >> 2) == (c.b >> 2);                    // the four K quarters of one tile
-    default: return p.a == c.a;                                                    // QKV <- RED, FC1 <- OUT, FIN <- RED
+    default: return p.a == c.a;                                                    // FC1 <- OUT (whole rows of the m-tile)
   }
 }
-__host__ __device__ __forceinline__ int producer_phase(int cph) { return cph == PH_QKV ? PH_RED : cph == PH_FIN ? PH_RED : cph - 1; }
+// (phases ATT .. FC2 wait for the flag words of the phase before; QKV and FIN wait for completion words of tiles)
+__host__ __device__ __forceinline__ int producer_phase(int cph) { return cph - 1; }
 
 // Must workgroup pb have published the producer phase before workgroup b may start its items of phase cph?
 // Yes if any item of pb in the producer phase writes something that any item of b in phase cph reads (a workgroup
