@@ -241,8 +241,7 @@ def bench_encoder(args, B, S, L, name):
     except sh.SouffleError as e:
         roof["measured_ceilings_error"] = str(e)
     # the same launch as a cooperative one (hipLaunchCooperativeKernel): the co-residency the hand-overs need is then
-    # guaranteed by the runtime instead of checked with the occupancy query.  Last GPU work of the process: memory
-    # re-used after cooperative launches was seen overwritten by what their ordinary stores had left in an L2.
+    # guaranteed by the runtime instead of checked with the occupancy query
     try:
         if args.no_coop:
             raise sh.SouffleError(0, "skipped (--no-coop)")
@@ -269,7 +268,6 @@ def main():
         print("no GPU available", file=sys.stderr)
         sys.exit(3)
     if args.workload == "encoder":
-        # (the sub-results first: the headline ends with cooperative launches, after which this process launches nothing)
         sub = {} if args.no_sub else {"encoder_s384": encoder_sub_result(args, 1, 384), "encoder_b32": encoder_sub_result(args, 32, 128)}
         res = bench_encoder(args, 1, 128, 12, "BERT-base 12-layer encoder, B=1, S=128, fp16 (BASELINE configs[2], first shape)")
         res["extra"].update(sub)

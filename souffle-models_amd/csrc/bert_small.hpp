@@ -943,8 +943,7 @@ __device__ __forceinline__ void run_fin_item(const Args &a, const It &d) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] += (float)b8[i]; }
   const h8 o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3], (half_t)v[4], (half_t)v[5], (half_t)v[6], (half_t)v[7]};
-  // (write-through like every store of this kernel: no line of it stays behind in an L2 when the launch ends, whatever the
-  // runtime does or does not write back between launches)
+  // (write-through like every store of this kernel)
   st16<true>(a.y, (m * H + n) * 2, as_u4(o));
 }
 

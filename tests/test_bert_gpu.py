@@ -1,8 +1,6 @@
 """GPU parity of the BERT encoder layer / encoder (through the C ABI via bert_binding)
 against the CPU oracle on identical fp16-rounded seeded inputs.
 Tolerance: max-abs <= 2e-2 and mean-abs <= 2e-3 on every tensor the reference returns."""
-import os
-
 import numpy as np
 import pytest
 import torch
@@ -250,43 +248,38 @@ def test_layernorm_of_rows_far_from_zero(B, S):
     assert_close("encoder, rows far from zero", y_f, oracle.bert_encoder(x, ws, B, S))
 
 
-_COOP_CHILD = r"""
-import sys
-sys.path[:0] = [%(pkg)r, %(orc)r, %(tests)r]
-import numpy as np, torch
-import bert_binding, oracle, synth, souffle_hip as sh
-from gpu_util import assert_close, dev, dev_weights
-B, S, layers = 1, 128, 3
-ws = [synth.bert_layer_weights(2, l) for l in range(layers)]
-x = synth.bert_input(2, B, S)
-enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
-y_plain = enc(dev(x)).clone()
-sh.set_cooperative_launch(True)
-y_coop = enc(dev(x)).clone()
-y_coop2 = enc(dev(x)).clone()
-flags = enc.ws.status()
-sh.set_cooperative_launch(False)
-assert flags == 0, flags
-assert torch.equal(y_coop, y_plain) and torch.equal(y_coop2, y_plain)
-assert_close("encoder cooperative", y_coop, oracle.bert_encoder(x, ws, B, S))
-print("COOPERATIVE-OK")
-"""
-
-
 def test_cooperative_launch_matches_oracle():
     """The persistent encoder launched with hipLaunchCooperativeKernel (the runtime's co-residency guarantee)
-    instead of the plain launch: same results, checked against the oracle.  In a process of its own: on this
-    runtime, memory that a process re-uses after it has launched cooperatively was seen to be overwritten later by
-    what ordinary (not write-through) stores of the cooperative kernel had left in an L2, so the other tests do
-    not share a process with such a launch."""
-    announce("bert encoder, cooperative launch (child process)")
-    import subprocess
-    import sys
-    here = os.path.dirname(os.path.abspath(__file__))
-    root = os.path.dirname(here)
-    code = _COOP_CHILD % {"pkg": os.path.join(root, "souffle-models_amd"), "orc": os.path.join(root, "oracle"), "tests": here}
-    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
-    assert r.returncode == 0 and "COOPERATIVE-OK" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+    instead of the plain launch: same results, checked against the oracle, and an encoder of the many-rows path
+    built afterwards in memory that the first one has given back works as well."""
+    announce("bert encoder, cooperative launch")
+    import bert_binding
+    import souffle_hip as sh
+    B, S, layers = 1, 128, 3
+    ws = [synth.bert_layer_weights(2, l) for l in range(layers)]
+    x = synth.bert_input(2, B, S)
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    y_plain = enc(dev(x)).clone()
+    sh.set_cooperative_launch(True)
+    try:
+        y_coop = enc(dev(x)).clone()
+        y_coop2 = enc(dev(x)).clone()
+        flags = enc.ws.status()
+        big = bert_binding.Encoder([dev_weights(w) for w in ws[:2]], 8, 128)
+        xb = synth.bert_input(3, 8, 128)
+        y_big_coop = big(dev(xb)).clone()
+        flags |= big.ws.status()
+    finally:
+        sh.set_cooperative_launch(False)
+    assert flags == 0
+    assert torch.equal(y_coop, y_plain) and torch.equal(y_coop2, y_plain)
+    assert_close("encoder cooperative", y_coop, oracle.bert_encoder(x, ws, B, S))
+    del enc, y_coop, y_coop2
+    again = bert_binding.Encoder([dev_weights(w) for w in ws[:2]], 8, 128)      # (in memory the first encoder used)
+    y_big = again(dev(xb))
+    assert again.ws.status() == 0
+    assert torch.equal(y_big, y_big_coop)
+    assert_close("many rows after cooperative launches", y_big, oracle.bert_encoder(xb, ws[:2], 8, 128))
 
 
 @pytest.mark.parametrize("B,S,layers,masked", [(1, 100, 2, False), (2, 77, 1, True), (1, 200, 1, False), (3, 5, 1, False)])
