@@ -822,11 +822,11 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
   };
   // A row of a pre-LayerNorm sum (8 columns per thread): + bias + the residual (normalised from its statistics when it
   // is itself a pre-LayerNorm sum), rounded to fp16, written with the statistics of the rounded values.
-  auto finish_row = [&](int row, int col0, f4 lo, f4 hi, int slice, half_t *res_out) {
-    add_bias(col0, lo, hi);
+  // The residual of a row (8 columns per thread), normalised from its statistics when it is itself a pre-LayerNorm sum.
+  struct Resid { f4 lo, hi; };
+  auto residual = [&](int row, int col0, half_t *res_out) {
     const h8 rv = *reinterpret_cast<const h8 *>(lds + kAuxOff + row * 128 + col0 * 2);
     f4 rlo = f4{(float)rv[0], (float)rv[1], (float)rv[2], (float)rv[3]}, rhi = f4{(float)rv[4], (float)rv[5], (float)rv[6], (float)rv[7]};
-    const int m = j.g.m0 + row;
     if (j.rstats) {
       const float *sp = reinterpret_cast<const float *>(lds + kAuxOff + 4096) + row * 24;
       float mean = 0.f;
@@ -840,9 +840,15 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       rlo = (rlo - mean) * rstd; rhi = (rhi - mean) * rstd;
       if (j.rgam) { const h8 gg = *reinterpret_cast<const h8 *>(lds + kGamOff + col0 * 2); rlo *= f4{(float)gg[0], (float)gg[1], (float)gg[2], (float)gg[3]}; rhi *= f4{(float)gg[4], (float)gg[5], (float)gg[6], (float)gg[7]}; }
       if (j.rbet) { const h8 bb = *reinterpret_cast<const h8 *>(lds + kGamOff + 128 + col0 * 2); rlo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]}; rhi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]}; }
-      if (res_out) st16<true>(res_out, (m * H + j.g.n0 + col0) * 2, pack_h8(rlo, rhi));      // (the normalised residual itself, on request)
+      if (res_out) st16<true>(res_out, ((j.g.m0 + row) * H + j.g.n0 + col0) * 2, pack_h8(rlo, rhi));      // (the normalised residual itself, on request)
     }
-    lo += rlo; hi += rhi;
+    return Resid{rlo, rhi};
+  };
+  // A row of a pre-LayerNorm sum: + bias + residual, rounded to fp16, written with the statistics of the rounded values.
+  auto finish_row = [&](int row, int col0, f4 lo, f4 hi, const Resid &r, int slice) {
+    add_bias(col0, lo, hi);
+    lo += r.lo; hi += r.hi;
+    const int m = j.g.m0 + row;
     const u4 packed = pack_h8(lo, hi);
     st16<true>(j.out, (m * H + j.g.n0 + col0) * 2, packed);
     const h8 r8 = as_h8(packed);
@@ -859,7 +865,7 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       st16<true>(j.out, ((((which * a.B + b) * NH + head) * a.S + s) * HD + col0) * 2, pack_h8(lo, hi));
     });
   } else if constexpr (ph == PH_OUT) {
-    reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) { finish_row(row, col0, lo, hi, d.b, nullptr); });
+    reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) { finish_row(row, col0, lo, hi, residual(row, col0, nullptr), d.b); });
   } else if constexpr (ph == PH_FC1) {
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
       add_bias(col0, lo, hi);
@@ -886,10 +892,12 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       wait_all_memory();
       __syncthreads();
       unsigned *ticket_lds = reinterpret_cast<unsigned *>(lds + kBiasOff + 256);
-      if (tid == 0) {
-        unsigned *cnt = a.flags + kTileCntWord + (l * kTileWords + d.a * 12 + ns);
-        *ticket_lds = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+      unsigned ticket = 0;
+      if (tid == 0) ticket = __hip_atomic_fetch_add(a.flags + kTileCntWord + (l * kTileWords + d.a * 12 + ns), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // (while the ticket travels: what the workgroup that turns out to be last adds to the sum.  ln1_out, asked for by
+      // single-layer callers only, is written by whoever runs this, with the same values.)
+      const Resid res = residual(row, col0, a.ln1_out);
+      if (tid == 0) *ticket_lds = ticket;
       __syncthreads();
       const bool last = (*ticket_lds & 3u) == 3u;
       compiler_fence();
@@ -908,7 +916,7 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
         slo += k == ks ? lo : __builtin_bit_cast(f4, plo[k]);
         shi += k == ks ? hi : __builtin_bit_cast(f4, phi[k]);
       }
-      finish_row(row, col0, slo, shi, ns, a.ln1_out);
+      finish_row(row, col0, slo, shi, res, ns);
       if (sy) {
         wait_all_memory();
         __syncthreads();
