@@ -1054,16 +1054,21 @@ static int launch_mega(Args &a, int grid, hipStream_t st) {
   }
 }
 
-template <int NKT>
-static int launch_small_t(sk::Args &a, int grid, hipStream_t st) {
+template <int NKT, bool MULTI>
+static int launch_small_tt(sk::Args &a, int grid, hipStream_t st) {
   const int lds = lds_bytes_small();
   static bool attr_done = false;
   if (!attr_done) {
-    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)sk::k_encoder_small<NKT>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)sk::k_encoder_small<NKT, MULTI>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     attr_done = true;
   }
   void *args[] = {&a};
-  return launch_persistent((const void *)sk::k_encoder_small<NKT>, grid, 256, args, lds, st);
+  return launch_persistent((const void *)sk::k_encoder_small<NKT, MULTI>, grid, 256, args, lds, st);
+}
+template <int NKT>
+static int launch_small_t(sk::Args &a, int grid, hipStream_t st) {
+  const sk::Shape sh{a.B, a.S, a.M, a.M / 32, grid};
+  return sk::single_pass(sh) ? launch_small_tt<NKT, false>(a, grid, st) : launch_small_tt<NKT, true>(a, grid, st);
 }
 static int launch_small(sk::Args &a, int grid, hipStream_t st) {
   switch (a.S) {
@@ -1165,8 +1170,8 @@ static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *laye
   if (!p.large) {
     static thread_local sk::Args sa;
     if (int rc = fill_small(sa, c, layers, nl, x_in, mask_in, y_out, dump, ws, ws_bytes, p)) return rc;
-    stage_trace(&sa.trace, &sa.trace_cap, df.num_cus);
-    return launch_small(sa, df.num_cus, st);
+    stage_trace(&sa.trace, &sa.trace_cap, df.num_cus & ~7);
+    return launch_small(sa, df.num_cus & ~7, st);        // (a multiple of 8: one weight slice per workgroup and phase, see sk::wg_item)
   }
   static thread_local Args a;
   if (int rc = fill_args(a, c, layers, nl, x_in, mask_in, y_out, dump, ws, ws_bytes, p)) return rc;
@@ -1236,7 +1241,7 @@ static int run_unfused(const souffle_bert_cfg *c, const souffle_bert_layer_w *la
   if (!p.large) {
     static thread_local sk::Args sa;
     if (int rc = fill_small(sa, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
-    return run_small_unfused(sa, df.num_cus, st);
+    return run_small_unfused(sa, df.num_cus & ~7, st);
   }
   static thread_local Args a;
   if (int rc = fill_args(a, c, layers, nl, x, mask, y, dump, ws, ws_bytes, p)) return rc;
@@ -1341,12 +1346,9 @@ extern "C" int souffle_bert_handover_plan(int batch, int seq_len, int grid, int 
   if (phase < sk::PH_QKV || phase > sk::PH_FIN || phase == sk::PH_RED) return fail(SOUFFLE_ERR_SHAPE, "phase must be 0 (QKV), 1 (ATT), 2 (OUT), 3 (FC1), 4 (FC2) or 6 (FIN)");
   const sk::Shape sh{batch, seq_len, batch * seq_len, batch * seq_len / 32, grid};
   int n = 0;
-  for (int it = workgroup - sk::ph_off(sh, phase); it < sk::ph_span(sh, phase); it += grid) {
-    sk::It d;
-    if (it < 0 || !sk::ph_item(sh, phase, it, d)) continue;
+  sk::It d;
+  for (; sk::wg_item(sh, phase, workgroup, n, d); ++n)
     if (items && n < max_items) { items[2 * n] = d.a; items[2 * n + 1] = d.b; }
-    ++n;
-  }
   *n_items = n;
   if (needs)
     for (int pb = 0; pb < grid; ++pb)

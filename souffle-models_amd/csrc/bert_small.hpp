@@ -138,12 +138,44 @@ __host__ __device__ __forceinline__ bool ph_item(const Shape &s, int ph, int it,
   if (ph == PH_ATT) return xcd_item(s.G, it, s.S / 16, s.B * 12, &d.a, &d.b);
   return xcd_item(s.G, it, s.m_tiles, ph_slices(ph), &d.a, &d.b);
 }
-// items of workgroup b: it = b - off, b - off + G, ... below the span
+// Does every workgroup have at most one item in every GEMM phase?
+__host__ __device__ inline bool single_pass(const Shape &s) {
+  return (s.G & 7) == 0 && xcd_item_span(s.G, s.m_tiles, 48) <= s.G;      // (FC1 and FC2 have the most slices)
+}
+// Item i (0, 1, ...) of workgroup b in phase ph; false when the workgroup has no i-th item.
+// GEMM phases (and FIN, which has the out-projection's items) with more items than workgroups: XCD x owns the weight
+// slices ws = x, x + 8, ...; its G / 8 workgroups are dealt to those slices round-robin (local number w -> slice number w % n, rank w / n among the
+// k workgroups of that slice), and a workgroup takes the m-tiles rank, rank + k, ... of its one slice: whatever the
+// number of rows, a workgroup fetches one weight slice per phase, and the slice crosses the fabric once per XCD.
+// Attention: items in the order of xcd_item, one per pass over the grid.
+// a / n for 0 <= a < 65536 and 1 <= n <= 64, without the instruction sequence of an integer division (the set-up of a
+// launch evaluates the work split for every pair of workgroups): (a + 0.5) / n lies at least 0.5 / n away from an
+// integer, far more than the rounding of the reciprocal and the product.
+__host__ __device__ __forceinline__ int idiv_small(int a, int n) { return (int)(((float)a + 0.5f) * (1.0f / (float)n)); }
+__host__ __device__ inline bool wg_item(const Shape &s, int ph, int b, int i, It &d) {
+  if (ph == PH_ATT || (s.G & 7) != 0) {
+    const int span = ph_span(s, ph);
+    for (int it = b - ph_off(s, ph); it < span; it += s.G) {
+      if (it < 0 || !ph_item(s, ph, it, d)) continue;
+      if (i-- == 0) return true;
+    }
+    return false;
+  }
+  if (ph_span(s, ph) <= s.G) {                         // every workgroup has at most one item: m-tiles of a slice side by side
+    if (i != 0 || b >= ph_span(s, ph)) return false;
+    return ph_item(s, ph, b, d);
+  }
+  const int slices = ph_slices(ph), x = b & 7, w = b >> 3, per = s.G >> 3;
+  const int n = (slices - x + 7) >> 3;                 // slices of this XCD
+  if (n <= 0) return false;
+  const int rank = idiv_small(w, n), si = w - rank * n, k = idiv_small(per - si + n - 1, n);      // k workgroups share slice number si
+  d.a = rank + i * k;
+  d.b = si * 8 + x;
+  return d.a < s.m_tiles;
+}
 __host__ __device__ __forceinline__ bool has_items(const Shape &s, int ph, int b) {
   It d;
-  for (int it = b - ph_off(s, ph); it < ph_span(s, ph); it += s.G)
-    if (it >= 0 && ph_item(s, ph, it, d)) return true;
-  return false;
+  return wg_item(s, ph, b, 0, d);
 }
 // Does producer item p (of the phase that feeds phase cph) write something that consumer item c reads?
 __host__ __device__ __forceinline__ bool feeds(const Shape &s, int cph, const It &c, const It &p) {
@@ -166,15 +198,15 @@ __host__ __device__ __forceinline__ int producer_phase(int cph) { return cph - 1
 __host__ __device__ inline bool wait_needs(const Shape &s, int cph, int b, int pb) {
   const int pph = producer_phase(cph);
   if (pb >= s.G) return false;
-  const int cspan = ph_span(s, cph), pspan = ph_span(s, pph);
-  for (int cit = b - ph_off(s, cph); cit < cspan; cit += s.G) {
-    It c;
-    if (cit < 0 || !ph_item(s, cph, cit, c)) continue;
-    for (int pit = pb - ph_off(s, pph); pit < pspan; pit += s.G) {
-      It p;
-      if (pit >= 0 && ph_item(s, pph, pit, p) && feeds(s, cph, c, p)) return true;
-    }
+  It c, p;
+  if (ph_span(s, pph) + ph_off(s, pph) <= s.G && ph_span(s, cph) + ph_off(s, cph) <= s.G) {      // one item each at most
+    const int cit = b - ph_off(s, cph), pit = pb - ph_off(s, pph);
+    if (!(cit >= 0 && cit < ph_span(s, cph) && ph_item(s, cph, cit, c))) return false;
+    return pit >= 0 && pit < ph_span(s, pph) && ph_item(s, pph, pit, p) && feeds(s, cph, c, p);
   }
+  for (int ci = 0; wg_item(s, cph, b, ci, c); ++ci)
+    for (int pi = 0; wg_item(s, pph, pb, pi, p); ++pi)
+      if (feeds(s, cph, c, p)) return true;
   return false;
 }
 
@@ -958,33 +990,23 @@ __device__ __forceinline__ void run_fin_item(const Args &a, const It &d) {
 // for every item of phase ph that belongs to workgroup b: fn(item, first)
 template <class Fn>
 __device__ __forceinline__ void for_items(const Shape &sh, int ph, int b, Fn fn) {
-  const int span = ph_span(sh, ph);
-  bool first = true;
-  for (int it = b - ph_off(sh, ph); it < span; it += sh.G) {
-    It d;
-    if (it < 0 || !ph_item(sh, ph, it, d)) continue;
-    fn(d, first);
-    first = false;
-  }
+  It d;
+  for (int i = 0; wg_item(sh, ph, b, i, d); ++i) fn(d, i == 0);
 }
-// the items of workgroup b in phase ph from item number `it` on (it + G, it + 2 G, ...): fn(item)
-template <class Fn>
-__device__ __forceinline__ void for_items_from(const Shape &sh, int ph, int it, Fn fn) {
-  const int span = ph_span(sh, ph);
-  for (; it < span; it += sh.G) {
-    It d;
-    if (it < 0 || !ph_item(sh, ph, it, d)) continue;
-    fn(d);
-  }
-}
-// the number of workgroup b's first item in phase ph (for_items_from continues behind it), -1 = none
-struct FirstItem { int it; It d; };
+// workgroup b's items in a GEMM phase: the first one, how many there are and how far apart their m-tiles lie (found once
+// per launch, so that the phase code divides nothing)
+struct FirstItem { int count, step; It d; };
 __device__ __forceinline__ FirstItem first_item(const Shape &sh, int ph, int b) {
-  const int span = ph_span(sh, ph);
-  FirstItem f{-1, It{0, 0}};
-  for (int it = b - ph_off(sh, ph); it < span && f.it < 0; it += sh.G) {
-    It d;
-    if (it >= 0 && ph_item(sh, ph, it, d)) { f.it = it; f.d = d; }
+  FirstItem f{0, 0, It{0, 0}};
+  It d;
+  if (ph_span(sh, ph) <= sh.G) {                       // one item at most
+    f.count = b < ph_span(sh, ph) && ph_item(sh, ph, b, f.d) ? 1 : 0;
+    return f;
+  }
+  while (wg_item(sh, ph, b, f.count, d)) {
+    if (f.count == 0) f.d = d;
+    if (f.count == 1) f.step = d.a - f.d.a;
+    ++f.count;
   }
   return f;
 }
@@ -994,7 +1016,9 @@ __device__ __forceinline__ AttnArgs attn_args(const Args &a, int l) {
 }
 
 // ------------------------------------------------------------------ fused kernel ----
-template <int NKT>
+// MULTI: some workgroup has more than one item in some GEMM phase (more rows than one pass over the grid covers); the
+// single-pass instantiation carries no code for further items.
+template <int NKT, bool MULTI>
 __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int b = blockIdx.x, tid = threadIdx.x;
@@ -1089,11 +1113,12 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
       }
     } else await(sy, wm(ph), phase_seq(sy, l, ph - 1), l * PH_SLOTS + ph);
     run_gemm_item_t<ph>(lds, args, l, f0.d, j0, ready, &sy);
-    for_items_from(sh, ph, f0.it + sh.G, [&](const It &d) {
+    if constexpr (MULTI) for (int i = 1; i < f0.count; ++i) {      // further m-tiles of the same weight slice, which stays where it is
+      const It d{f0.d.a + i * f0.step, f0.d.b};
       __syncthreads();                                        // the partial tiles of the previous item have been read
       if (ph == PH_QKV && l > 0) await_tiles(sy, d.a, phase_seq(sy, l - 1, PH_RED), sy.trace_cap);      // (its own m-tile)
-      run_gemm_item_t<ph>(lds, args, l, d, make_job_t<ph>(args, l, d), false, &sy);
-    });
+      run_gemm_item_t<ph>(lds, args, l, d, make_job_t<ph>(args, l, d), true, &sy);
+    }
     stamp_mark(sy, l * PH_SLOTS + ph, 2);
     publish(sy, phase_seq(sy, l, ph));
     stamp_mark(sy, l * PH_SLOTS + ph, 3);
@@ -1156,7 +1181,7 @@ __global__ void __launch_bounds__(256) k_small_phase(Args args, int l, int ph) {
   } else {
     for_items(sh, ph, b, [&](const It &d, bool first) {
       if (!first) __syncthreads();
-      run_gemm_item(lds, args, l, ph, d, make_job(args, l, ph, d), false);
+      run_gemm_item(lds, args, l, ph, d, make_job(args, l, ph, d), !first);      // (the first item's weight slice stays: the grid is a multiple of 8)
     });
   }
 }
