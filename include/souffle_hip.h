@@ -56,7 +56,7 @@ int souffle_device_info(souffle_devinfo *out);
  * workspace (souffle_workspace_init; 16 KiB are enough).  mode 0: the grid barrier alone; mode 1: 16 bytes
  * written through, the barrier, and a read of what a workgroup of another XCD wrote, per stage.  Timed by
  * the caller it gives the latency floor of a chain of dependent stages on this device, which bounds the
- * skinny shapes (B*S < 1024) rather than the HBM or MFMA roofline. */
+ * skinny shapes (B*S up to about a thousand rows) rather than the HBM or MFMA roofline. */
 int souffle_stage_floor_probe(void *workspace, size_t workspace_bytes, int stages, int mode, souffle_stream_t stream);
 /* Queues one MFMA-only kernel (4 waves per CU, `iters` x 16 independent fp16 16x16x32 MFMAs per wave, no
  * memory traffic) and reports the flops it performs: timed by the caller, it gives the empirical

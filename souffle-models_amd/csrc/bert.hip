@@ -1,6 +1,6 @@
 // BERT-base encoder layer(s) on gfx950: one persistent launch for all stages of all layers, and the same
 // stages as separate launches (the unfused per-op baseline).  Two paths:
-//   few rows (batch * seq_len < 1024): bert_small.hpp (flag hand-overs between the producers and consumers of a tile);
+//   few rows (batch * seq_len <= 1024, and up to 1408 where it is no multiple of 256: many_rows()): bert_small.hpp (flag hand-overs between the producers and consumers of a tile);
 //   many rows: this file (256-row or 128 x 128 GEMM tiles, hand-overs per 256-row block or grid barriers).
 //
 // Stage list per layer (reference counterparts in brackets):
@@ -709,7 +709,7 @@ __device__ __forceinline__ void stage_ln(const Params &a, const half_t *bias, co
 }
 
 // ------------------------------------------------------------ megakernel ----
-// Many rows (M >= 1024).  MODE 1: 128 x 128 tiles; 2: 256-row tiles (M a multiple of 256)
+// Many rows (many_rows(M)).  MODE 1: 128 x 128 tiles; 2: 256-row tiles (M a multiple of 256)
 template <int MODE, int NKT>
 __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
   static_assert(MODE == 1 || MODE == 2, "the few-rows path is k_encoder_small");
@@ -881,18 +881,25 @@ static int validate(const souffle_bert_cfg *c) {
   if (c->seq_len > 512) return fail(SOUFFLE_ERR_SHAPE, "seq_len must be at most 512 (got %d)", c->seq_len);
   const int s = padded_len(c->seq_len);          // other lengths run padded to the next built one
   const long long m = (long long)c->batch * s;
-  if (m >= 1024 && m % 128 != 0) return fail(SOUFFLE_ERR_SHAPE, "batch*seq_len >= 1024 must be a multiple of 128 (got %lld)", m);
+  if (m >= 1536 && m % 128 != 0) return fail(SOUFFLE_ERR_SHAPE, "batch*seq_len >= 1536 must be a multiple of 128 (got %lld)", m);
   if (m > 65536) return fail(SOUFFLE_ERR_SHAPE, "batch*seq_len must be <= 65536 (got %lld)", m);
   if (c->act != SOUFFLE_ACT_GELU_TANH && c->act != SOUFFLE_ACT_RELU) return fail(SOUFFLE_ERR_SHAPE, "unknown activation %d", c->act);
   if (!(c->ln_eps >= 0.f)) return fail(SOUFFLE_ERR_SHAPE, "ln_eps must be >= 0");
   return SOUFFLE_OK;
 }
 
+// Which kernel runs a shape.  The few-rows kernel (one weight slice per workgroup and phase, flag hand-overs) is the
+// faster one up to 1024 rows (12 layers at 8 x 128: 1042 us against 1209; at 2 x 512: 1101 against 1427) and, where
+// the rows are no multiple of 256 and the many-rows kernel has to fall back to its 128 x 128 tiles, up to 1408 rows
+// (1152 rows: 1158 against 1436; 1408: 1363 against 1638; at 1280 rows the two are level and at 1536 the 256-row
+// tiles win, 1204 against 1451).
+static bool many_rows(size_t M) { return M >= 1536 || (M > 1024 && M % 256 == 0); }
+
 static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   Plan p{};
   const size_t M = (size_t)c->batch * padded_len(c->seq_len);
-  p.large = M >= 1024;
-  p.big = M >= 1024 && M % 256 == 0;     // (12 layers at M = 1024: 1222 us, with the 128 x 128 tiles 1409 us; at M = 1536: 1225 against 1661)
+  p.large = many_rows(M);
+  p.big = p.large && M % 256 == 0;     // (12 layers at M = 1024: 1222 us, with the 128 x 128 tiles 1409 us; at M = 1536: 1225 against 1661)
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += round_up(bytes, 256); return o; };
   p.off_ctl = take(kCtlWords * 4);
@@ -1340,8 +1347,8 @@ extern "C" int souffle_bert_handover_plan(int batch, int seq_len, int grid, int 
                                           int *n_items, unsigned char *needs) {
   namespace sk = bert::sk;
   if (!n_items) return fail(SOUFFLE_ERR_NULL, "n_items is NULL");
-  if (batch <= 0 || (seq_len != 64 && seq_len != 128 && seq_len != 256 && seq_len != 384 && seq_len != 512) || (long long)batch * seq_len >= 1024)
-    return fail(SOUFFLE_ERR_SHAPE, "the few-rows plan exists for seq_len in {64,128,256,384,512} and fewer than 1024 rows (got %d x %d)", batch, seq_len);
+  if (batch <= 0 || (seq_len != 64 && seq_len != 128 && seq_len != 256 && seq_len != 384 && seq_len != 512) || bert::many_rows((size_t)batch * seq_len))
+    return fail(SOUFFLE_ERR_SHAPE, "the few-rows plan exists for seq_len in {64,128,256,384,512} and the row counts that the few-rows kernel runs (got %d x %d)", batch, seq_len);
   if (grid <= 0 || grid > 1024 || workgroup < 0 || workgroup >= grid) return fail(SOUFFLE_ERR_SHAPE, "grid must be in 1..1024 and workgroup below it");
   if (phase < sk::PH_QKV || phase > sk::PH_FIN || phase == sk::PH_RED) return fail(SOUFFLE_ERR_SHAPE, "phase must be 0 (QKV), 1 (ATT), 2 (OUT), 3 (FC1), 4 (FC2) or 6 (FIN)");
   const sk::Shape sh{batch, seq_len, batch * seq_len, batch * seq_len / 32, grid};

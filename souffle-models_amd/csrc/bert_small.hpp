@@ -1,4 +1,5 @@
-// BERT-base encoder, few rows (batch * seq_len < 1024): the weight-stream-bound shapes.
+// BERT-base encoder, few rows (batch * seq_len up to 1024, and up to 1408 where the rows are no multiple of 256): the
+// weight-stream-bound shapes.
 //
 // A layer is five phases, each a set of independent items dealt to the workgroups of one persistent launch:
 //   QKV  (m-tile, 64 of the 2304 q/k/v columns)   X = layer input (layer 0) or LN2 of the previous layer's sum
@@ -64,7 +65,7 @@ constexpr int kFlagWords = kFlagBaseWord + 64;
 // the workgroup that completes the tile sets to the sequence number of (layer, RED); and per layer and tile a ticket
 // counter that the four workgroups of the tile's K quarters draw from (the one that draws the fourth ticket sums the
 // tile).  Counters only grow, by exactly four per launch and tile, so they need no clearing.
-constexpr int kTileWords = 384;                                  // 31 m-tiles x 12 n-slices at most, padded
+constexpr int kTileWords = 576;                                  // 48 m-tiles x 12 n-slices: up to 1536 rows
 constexpr int kTileDoneWord = kFlagWords;                        // 8 copies of kTileWords
 constexpr int kTileCntWord = kTileDoneWord + kFlagCopies * kTileWords;          // kMaxLayers x kTileWords
 constexpr int kFlagRegionWords = kTileCntWord + kMaxLayers * kTileWords;

@@ -217,13 +217,14 @@ def test_few_rows_shapes_take_turns_in_one_workspace():
     assert shared.status() == 0
 
 
-@pytest.mark.parametrize("B,S", [(1, 128), (1, 384), (8, 128)])
+@pytest.mark.parametrize("B,S", [(1, 128), (1, 384), (8, 128), (16, 128)])
 def test_layernorm_of_rows_far_from_zero(B, S):
     """Rows whose mean is far larger than their spread, and feature columns of large magnitude: the LayerNorm
     statistics (per-slice mean and squared deviations, combined pairwise) and the normalisation in the operand
     registers must not lose the spread to cancellation.  Checked against the oracle on the few-rows path, at both
     places where a LayerNorm is applied on load (LN1 inside FC1, LN2 inside the next layer's QKV and at the end),
-    and on the many-rows path (1024 rows), whose LayerNorm stages are separate passes over the rows."""
+    at 1024 rows (several m-tiles per workgroup), and on the many-rows path (2048 rows), whose LayerNorm stages are
+    separate passes over the rows."""
     announce("bert encoder B=%d S=%d, rows with a large mean" % (B, S))
     import bert_binding
     layers = 2

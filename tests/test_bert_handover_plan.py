@@ -19,7 +19,7 @@ def plan(B, S, G, phase, b):
     n = C.c_int(0)
     needs = (C.c_ubyte * G)()
     sh.check(sh.lib().souffle_bert_handover_plan(B, S, G, phase, b, items, 32, C.byref(n), needs))
-    assert n.value <= 32
+    assert n.value <= 32, n.value
     return [(items[2 * i], items[2 * i + 1]) for i in range(n.value)], np.frombuffer(needs, dtype=np.uint8).copy()
 
 
@@ -62,7 +62,7 @@ def overlap(r, w):
         max(r[2].start, w[2].start) < min(r[2].stop, w[2].stop)
 
 
-SHAPES = [(1, 64), (1, 128), (2, 128), (1, 256), (3, 256), (1, 384), (2, 384), (1, 512), (7, 128), (15, 64)]
+SHAPES = [(1, 64), (1, 128), (2, 128), (1, 256), (3, 256), (1, 384), (2, 384), (1, 512), (7, 128), (15, 64), (8, 128), (2, 512), (11, 128)]
 
 
 @pytest.mark.parametrize("B,S", SHAPES)
@@ -99,7 +99,8 @@ def test_every_dependence_is_waited_for_and_every_item_has_one_owner(B, S, G):
 def test_plan_rejects_what_the_few_rows_path_does_not_run():
     n = C.c_int(0)
     lib = sh.lib()
-    assert lib.souffle_bert_handover_plan(8, 128, 256, 0, 0, None, 0, C.byref(n), None) == -2      # 1024 rows: the many-rows path
+    assert lib.souffle_bert_handover_plan(12, 128, 256, 0, 0, None, 0, C.byref(n), None) == -2     # 1536 rows: the many-rows path
+    assert lib.souffle_bert_handover_plan(10, 128, 256, 0, 0, None, 0, C.byref(n), None) == -2     # 1280 rows, a multiple of 256: likewise
     assert lib.souffle_bert_handover_plan(1, 100, 256, 0, 0, None, 0, C.byref(n), None) == -2
     assert lib.souffle_bert_handover_plan(1, 128, 256, 5, 0, None, 0, C.byref(n), None) == -2
     assert lib.souffle_bert_handover_plan(1, 128, 256, 0, 256, None, 0, C.byref(n), None) == -2
