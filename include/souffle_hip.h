@@ -180,7 +180,8 @@ int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert
 int souffle_bert_encoder_fused_static(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
                                       const void *x, const void *mask, void *y, souffle_stream_t stream);
 
-/* The work split and the hand-over plan of the encoder below 1024 rows, evaluated on the host by the functions the
+/* The work split and the hand-over plan of the encoder at few rows (up to 1024, and below 1536 where the count is
+ * no multiple of 256), evaluated on the host by the functions the
  * kernel itself uses (no GPU needed; no counterpart in the reference, whose stages are separated by grid barriers):
  * the items of `workgroup` in `phase` (0 QKV, 1 attention, 2 out-projection, 3 FC1, 4 FC2, 6 final LayerNorm) as
  * pairs (m-tile, weight slice) - attention: (block of 16 queries, batch * 12 + head) - written to items[2 i], items[2 i + 1]
