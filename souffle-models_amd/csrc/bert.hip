@@ -326,8 +326,9 @@ __device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, 
 // LayerNorm adds them in order, then the residual.
 __device__ __forceinline__ half_t *fc2_sums(const Params &a) { return reinterpret_cast<half_t *>(a.part); }
 template <bool COH>
-__device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a, const half_t *X, int K, const half_t *W,
-                                            const half_t *bias, int first, int stride) {
+__device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a, const half_t *X, int K, const half_t *W, int first, int stride) {
+  // (the bias is added by the LayerNorm that sums the four parts: a tile that added it took 2.4 us longer than the
+  // other three of its column group, and the hand-over behind the stage waits for the slowest)
   const int m_tiles = a.M / 256;
   for (int it = first; it < m_tiles * 16; it += stride) {
     int tm, tn2;
@@ -335,21 +336,18 @@ __device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a,
     const int ks = tn2 % kFc2Split, n0 = (tn2 / kFc2Split) * BigFc2::kBN, k0 = ks * (K / kFc2Split);
     half_t *zp = fc2_sums(a) + (size_t)ks * a.M * H;
     auto wptr = [&](int k, int col) { return W + (size_t)k * H + n0 + col; };
-    const half_t *bz = bias ? bias : g_zero_row;
-    auto cvt_first = [&](int, int nr, f4 v) { return pack_h4(add_row4(v, bz, n0 + nr)); };
-    auto cvt_rest = [&](int, int, f4 v) { return pack_h4(v); };
+    auto cvt = [&](int, int, f4 v) { return pack_h4(v); };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(zp, (m * H + n0 + nr) * 2, v); };
     f4 acc[BigFc2::MI][BigFc2::NT];
     BigFc2::mainloop(lds, X, K, tm * 256, k0, (K / kFc2Split) / 32, wptr, acc);
-    if (ks == 0) BigFc2::epilogue(lds, tm * 256, acc, cvt_first, store16);
-    else BigFc2::epilogue(lds, tm * 256, acc, cvt_rest, store16);
+    BigFc2::epilogue(lds, tm * 256, acc, cvt, store16);
   }
 }
 // out[m] = LN(z[0][m] + ... + z[NZ-1][m] + resid[m]) * g + b (z[p] = z + p M H; summed in this order);
 // one wave per row, two-pass statistics in fp32 registers.
 // NR rows (m0, m0 + mstep, ...) per call: their loads are all issued before the first is used.
 template <bool COH, int NR, int NZ>
-__device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z, const half_t *resid, const half_t *gam, const half_t *bet, half_t *out, int m0, int mstep) {
+__device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z, const half_t *resid, const half_t *bias, const half_t *gam, const half_t *bet, half_t *out, int m0, int mstep) {
   const int lane = opaque_thread_id() & 63;
   u2 raw[NR][NZ + 1][3];
 #pragma unroll
@@ -375,6 +373,10 @@ __device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z, co
       for (int p = 1; p <= NZ; ++p) {
         const h4 q2 = as_h4(raw[r][p][c]);
         v[c] += f4{(float)q2[0], (float)q2[1], (float)q2[2], (float)q2[3]};
+      }
+      if (bias) {                                   // (of the GEMM whose partial sums these are: added once per row here, not per tile there)
+        const h4 bb = ldg<h4>(bias + c * 256 + lane * 4);
+        v[c] += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
       }
       sum += v[c][0] + v[c][1] + v[c][2] + v[c][3];
     }
@@ -404,8 +406,8 @@ __device__ __forceinline__ void big_ln_rows(const Params &a, const half_t *z, co
   }
 }
 template <bool COH, int NZ>
-__device__ __forceinline__ void big_ln(const Params &a, const half_t *z, const half_t *resid, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
-  for (int m = first_row; m < a.M; m += row_stride) big_ln_rows<COH, 1, NZ>(a, z, resid, gam, bet, out, m, 0);
+__device__ __forceinline__ void big_ln(const Params &a, const half_t *z, const half_t *resid, const half_t *bias, const half_t *gam, const half_t *bet, half_t *out, int first_row, int row_stride) {
+  for (int m = first_row; m < a.M; m += row_stride) big_ln_rows<COH, 1, NZ>(a, z, resid, bias, gam, bet, out, m, 0);
 }
 
 // The LayerNorm that follows a pre-LayerNorm sum, without a grid barrier in between (rowblock_ln).  A 256-row
@@ -460,14 +462,14 @@ __device__ __forceinline__ void rowblock_sync(const Params &a, GridBarrier &bar,
   compiler_fence();                              // no load of the other tiles' results is scheduled above the poll
 }
 template <bool COH, int NZ>
-__device__ __forceinline__ void rowblock_ln(const Params &a, GridBarrier &bar, unsigned tag, const half_t *z, const half_t *resid, const half_t *gam,
-                                            const half_t *bet, half_t *out, int first, int stride) {
+__device__ __forceinline__ void rowblock_ln(const Params &a, GridBarrier &bar, unsigned tag, const half_t *z, const half_t *resid, const half_t *bias,
+                                            const half_t *gam, const half_t *bet, half_t *out, int first, int stride) {
   const int m_tiles = a.M / 256, wave = threadIdx.x >> 6;
   rowblock_sync(a, bar, tag, first, stride, 1, []() {});
   for (int it = first; it < m_tiles * 16; it += stride) {
     int tm, tn;
     big_tile(it, m_tiles, 16, &tm, &tn);
-    big_ln_rows<COH, 4, NZ>(a, z, resid, gam, bet, out, tm * 256 + tn * 16 + wave * 4, 1);
+    big_ln_rows<COH, 4, NZ>(a, z, resid, bias, gam, bet, out, tm * 256 + tn * 16 + wave * 4, 1);
   }
 }
 
@@ -753,12 +755,12 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
       else stage_attn_t<true, NKT>(lds, a, first, stride);
       sync(2);
       big_presum<true>(lds_raw, a, a.ctx, H, w.w_o, w.b_o, first, stride);
-      rowblock_ln<true, 1>(a, bar, 7u * l + 3u, a.z1, xin, w.ln1_g, w.ln1_b, a.y1, first, stride);
+      rowblock_ln<true, 1>(a, bar, 7u * l + 3u, a.z1, xin, nullptr, w.ln1_g, w.ln1_b, a.y1, first, stride);
       sync(4);
       big_fc1<true>(lds_raw, a, w, first, stride, &bar);
       sync(5);
-      big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, w.b_fc2, first, stride);
-      rowblock_ln<true, kFc2Split>(a, bar, 7u * l + 6u, fc2_sums(a), a.y1, w.ln2_g, w.ln2_b, yout, first, stride);
+      big_presum2<true>(lds_raw, a, a.h, F, w.w_fc2, first, stride);
+      rowblock_ln<true, kFc2Split>(a, bar, 7u * l + 6u, fc2_sums(a), a.y1, w.b_fc2, w.ln2_g, w.ln2_b, yout, first, stride);
       if (l + 1 < a.num_layers) {   // the next layer writes this layer's buffers again: see Params
         auto invalidate = [&]() { if (threadIdx.x < 64) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); };
         if (local) rowblock_sync(a, bar, 7u * l + 7u, first, stride, group, invalidate);
@@ -811,13 +813,13 @@ __global__ void __launch_bounds__(256) k_presum_big(Args a, const half_t *X, int
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   big_presum<false>(lds_raw, a, X, K, W, bias, blockIdx.x, gridDim.x);
 }
-__global__ void __launch_bounds__(256) k_presum2_big(Args a, const half_t *X, int K, const half_t *W, const half_t *bias) {
+__global__ void __launch_bounds__(256) k_presum2_big(Args a, const half_t *X, int K, const half_t *W) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  big_presum2<false>(lds_raw, a, X, K, W, bias, blockIdx.x, gridDim.x);
+  big_presum2<false>(lds_raw, a, X, K, W, blockIdx.x, gridDim.x);
 }
 template <int NZ>
-__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *z, const half_t *resid, const half_t *gam, const half_t *bet, half_t *out) {
-  big_ln<false, NZ>(a, z, resid, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
+__global__ void __launch_bounds__(256) k_ln_big(Args a, const half_t *z, const half_t *resid, const half_t *bias, const half_t *gam, const half_t *bet, half_t *out) {
+  big_ln<false, NZ>(a, z, resid, bias, gam, bet, out, blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
 }
 template <int MODE>
 __global__ void __launch_bounds__(256) k_fc1(Args a, int l) {
@@ -1212,15 +1214,15 @@ static int run_unfused_t(Args &a, int nl, int num_cus, hipStream_t st) {
     hipLaunchKernelGGL(k_attn, dim3(grid_for(a.B * NH * (a.S / 64))), dim3(256), 2 * a.S * 128 + 64 * 128, st, a);
     if constexpr (MODE == 2) {
       hipLaunchKernelGGL(k_presum_big, dim3(grid_for((a.M / 256) * 16)), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, w.b_o);
-      hipLaunchKernelGGL(k_ln_big<1>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.z1, xin, w.ln1_g, w.ln1_b, a.y1);
+      hipLaunchKernelGGL(k_ln_big<1>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.z1, xin, (const half_t *)nullptr, w.ln1_g, w.ln1_b, a.y1);
     } else {
       hipLaunchKernelGGL(k_partial, dim3(grid_for((a.M / BM) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.ctx, H, w.w_o, 1);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, w.b_o, xin, w.ln1_g, w.ln1_b, a.y1);
     }
     hipLaunchKernelGGL(k_fc1<MODE>, dim3(grid_for((a.M / BM) * (F / BN))), dim3(256), GEMM_LDS, st, a, l);
     if constexpr (MODE == 2) {
-      hipLaunchKernelGGL(k_presum2_big, dim3(grid_for((a.M / 256) * 16)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, w.b_fc2);
-      hipLaunchKernelGGL(k_ln_big<kFc2Split>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.part, (const half_t *)a.y1, w.ln2_g, w.ln2_b, yout);
+      hipLaunchKernelGGL(k_presum2_big, dim3(grid_for((a.M / 256) * 16)), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2);
+      hipLaunchKernelGGL(k_ln_big<kFc2Split>, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, (const half_t *)a.part, (const half_t *)a.y1, w.b_fc2, w.ln2_g, w.ln2_b, yout);
     } else {
       hipLaunchKernelGGL(k_partial, dim3(grid_for((a.M / BM) * (H / BN))), dim3(256), GEMM_LDS, st, a, a.h, F, w.w_fc2, 1);
       hipLaunchKernelGGL(k_ln, dim3(grid_for((a.M + 3) / 4)), dim3(256), 0, st, a, w.b_fc2, a.y1, w.ln2_g, w.ln2_b, yout);
