@@ -260,16 +260,19 @@ __device__ __forceinline__ void big_qkv(unsigned char *lds, const Params &a, con
     };
     const half_t *bq = w.b_qkv ? w.b_qkv : g_zero_row;
     const int bq_stride = w.b_qkv ? H : 0;
-    auto cvt = [&](int, int nr, f4 v) {
+    auto bias_at = [&](int nr) {
       const int c = n0 + nr, j = c / H, n = c - j * H;
-      return pack_h4(add_row4(v, bq + j * bq_stride, n));
+      return ldg<h4>(bq + j * bq_stride + n);
     };
+    auto cvt = [&](int, int, f4 v, h4 bb) { return pack_h4(v + f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]}); };
     auto store16 = [&](int m, int nr, u4 v) {                // 8 columns never straddle a head (64 columns)
       const int c = n0 + nr, j = c / H, n = c - j * H;
       const int b = m / a.S, s = m % a.S, hh = n / HD, d = n % HD;
       st16<COH>(a.qkv, ((((j * a.B + b) * NH + hh) * a.S + s) * HD + d) * 2, v);
     };
-    BigQkv::run(lds, xin, H, tm * 256, 0, H / 32, wptr, cvt, store16, tb);
+    f4 acc[BigQkv::MI][BigQkv::NT];
+    BigQkv::mainloop(lds, xin, H, tm * 256, 0, H / 32, wptr, acc, tb);
+    BigQkv::epilogue_rowvec(lds, tm * 256, acc, bias_at, cvt, store16, tb);
   }
 }
 template <bool COH>
@@ -281,14 +284,15 @@ __device__ __forceinline__ void big_fc1(unsigned char *lds, const Params &a, con
     const int n0 = tn * BigFc1::kBN;
     auto wptr = [&](int k, int col) { return w.w_fc1 + (size_t)k * F + n0 + col; };
     const half_t *b1 = w.b_fc1 ? w.b_fc1 : g_zero_row;
-    auto cvt_relu = [&](int, int nr, f4 v) {
-      v = add_row4(v, b1, n0 + nr);
+    auto bias_at = [&](int nr) { return ldg<h4>(b1 + n0 + nr); };
+    auto cvt_relu = [&](int, int, f4 v, h4 bb) {
+      v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] = fmaxf(v[i], 0.f);
       return pack_h4(v);
     };
-    auto cvt_gelu = [&](int, int nr, f4 v) {
-      v = add_row4(v, b1, n0 + nr);
+    auto cvt_gelu = [&](int, int, f4 v, h4 bb) {
+      v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] = gelu_tanh(v[i]);
       return pack_h4(v);
@@ -296,8 +300,8 @@ __device__ __forceinline__ void big_fc1(unsigned char *lds, const Params &a, con
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.h, (m * F + n0 + nr) * 2, v); };
     f4 acc[BigFc1::MI][BigFc1::NT];
     BigFc1::mainloop(lds, a.y1, H, tm * 256, 0, H / 32, wptr, acc, tb);
-    if (a.act == SOUFFLE_ACT_RELU) BigFc1::epilogue(lds, tm * 256, acc, cvt_relu, store16, tb);
-    else BigFc1::epilogue(lds, tm * 256, acc, cvt_gelu, store16, tb);
+    if (a.act == SOUFFLE_ACT_RELU) BigFc1::epilogue_rowvec(lds, tm * 256, acc, bias_at, cvt_relu, store16, tb);
+    else BigFc1::epilogue_rowvec(lds, tm * 256, acc, bias_at, cvt_gelu, store16, tb);
   }
 }
 // z = X[M][K].W[K][768] + bias, fp16, into a.z1 (the out-projection; no split of K: 256 tiles already
@@ -315,9 +319,12 @@ __device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, 
     const int n0 = (tn >> 1) * BigOut::kBN, m0 = tm * 256 + (tn & 1) * BigOut::kBM;
     auto wptr = [&](int k, int col) { return W + (size_t)k * H + n0 + col; };
     const half_t *bz = bias ? bias : g_zero_row;
-    auto cvt = [&](int, int nr, f4 v) { return pack_h4(add_row4(v, bz, n0 + nr)); };
+    auto bias_at = [&](int nr) { return ldg<h4>(bz + n0 + nr); };
+    auto cvt = [&](int, int, f4 v, h4 bb) { return pack_h4(v + f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]}); };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.z1, (m * H + n0 + nr) * 2, v); };
-    BigOut::run(lds, X, K, m0, 0, K / 32, wptr, cvt, store16);
+    f4 acc[BigOut::MI][BigOut::NT];
+    BigOut::mainloop(lds, X, K, m0, 0, K / 32, wptr, acc);
+    BigOut::epilogue_rowvec(lds, m0, acc, bias_at, cvt, store16);
   }
 }
 // A pre-LayerNorm sum in kFc2Split parts of K: part 0 = X[:, part 0].W[part 0] + bias, part

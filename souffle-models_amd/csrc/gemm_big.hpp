@@ -240,7 +240,20 @@ struct GemmBig {
 
   template <class Cvt, class Store16>
   __device__ static __forceinline__ void epilogue(unsigned char *lds, int m0, f4 (&acc)[MI][NT], Cvt cvt, Store16 store16, const GridBarrier *tb = nullptr) {
+    epilogue_rowvec(lds, m0, acc, [](int) { return h4{(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f}; },
+                    [&](int m, int n, f4 v, h4) { return cvt(m, n, v); }, store16, tb);
+  }
+  // The same with a per-column vector (a bias) that the conversion adds: vec_at(n) -> the four values for columns
+  // n .. n + 3 (relative to the tile's first column), fetched for all of a lane's column groups at once before the first
+  // conversion, so that the epilogue waits for memory once and not once per accumulator tile;
+  // cvt(m, n, v, vec) -> u2.
+  template <class VecAt, class Cvt, class Store16>
+  __device__ static __forceinline__ void epilogue_rowvec(unsigned char *lds, int m0, f4 (&acc)[MI][NT], VecAt vec_at, Cvt cvt, Store16 store16,
+                                                         const GridBarrier *tb = nullptr) {
     const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+    h4 vec[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) vec[j] = vec_at(j * 16 + g * 4);
     // Epilogue.  A lane holds 4 consecutive columns of 16 rows per accumulator tile; stored
     // directly that would be 8-byte pieces of 32-byte row segments.  The converted tile instead
     // goes through the wave's own slice of the (now idle) ring, and leaves as 16 bytes per lane
@@ -257,7 +270,7 @@ struct GemmBig {
       for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = ch * TPC; j < (ch + 1) * TPC; ++j)
-          lds_store8(mine + (i * 16 + l16) * EPITCH + (j * 16 + g * 4) * 2, cvt(m0 + wave * RW + i * 16 + l16, j * 16 + g * 4, acc[i][j]));
+          lds_store8(mine + (i * 16 + l16) * EPITCH + (j * 16 + g * 4) * 2, cvt(m0 + wave * RW + i * 16 + l16, j * 16 + g * 4, acc[i][j], vec[j]));
       if constexpr (ch == ECH - 1) STAGE_MARK(tb, 3);
       static_assert((RW * CPC) % 64 == 0, "whole wave-wide stores");
 #pragma unroll
