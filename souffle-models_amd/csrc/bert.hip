@@ -265,9 +265,13 @@ __device__ __forceinline__ void big_qkv(unsigned char *lds, const Params &a, con
       return ldg<h4>(bq + j * bq_stride + n);
     };
     auto cvt = [&](int, int, f4 v, h4 bb) { return pack_h4(v + f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]}); };
+    // (batch and position of a row without a division per store: the tile's first row is divided once, a row of the
+    // tile lies at most 256 + S - 1 positions behind the start of that row's sequence)
+    const int b0 = (tm * 256) / a.S, s0 = tm * 256 - b0 * a.S;
     auto store16 = [&](int m, int nr, u4 v) {                // 8 columns never straddle a head (64 columns)
       const int c = n0 + nr, j = c / H, n = c - j * H;
-      const int b = m / a.S, s = m % a.S, hh = n / HD, d = n % HD;
+      const int rr = m - tm * 256 + s0, kb = sk::idiv_small(rr, a.S);
+      const int b = b0 + kb, s = rr - kb * a.S, hh = n / HD, d = n % HD;
       st16<COH>(a.qkv, ((((j * a.B + b) * NH + hh) * a.S + s) * HD + d) * 2, v);
     };
     f4 acc[BigQkv::MI][BigQkv::NT];

@@ -735,6 +735,7 @@ struct Job {
   float *aux;                          // FC2: the partial sums
   float *stat_out;                     // OUT: statistics of z1; FC2: of z2 (written by the workgroup that sums the tile)
   int which, head;                     // QKV: q, k or v and the head; FC2: which = K quarter
+  int batch, pos0;                     // QKV: sequence and position of the tile's first row
   bool x_sc1;
 };
 template <int PH>
@@ -749,6 +750,7 @@ __device__ __forceinline__ Job make_job_t(const Args &a, int l, const It &d) {
   if constexpr (PH == PH_QKV) {
     const int which = d.b / 12, head = d.b % 12;
     j.which = which; j.head = head;
+    j.batch = j.g.m0 / a.S; j.pos0 = j.g.m0 - j.batch * a.S;
     j.g.W = w.w_qkv + (size_t)which * H * H; j.g.ldw = H; j.g.kw0 = 0; j.g.n0 = head * HD;
     j.g.ldx = H; j.g.kx0 = 0;
     if (l == 0) { j.g.X = a.x; j.x_sc1 = false; }
@@ -894,7 +896,7 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
     const int which = j.which, head = j.head;
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
       add_bias(col0, lo, hi);
-      const int m = j.g.m0 + row, b = m / a.S, s = m % a.S;
+      const int b = j.batch, s = j.pos0 + row;             // (a 32-row tile never straddles two sequences)
       st16<true>(j.out, ((((which * a.B + b) * NH + head) * a.S + s) * HD + col0) * 2, pack_h8(lo, hi));
     });
   } else if constexpr (ph == PH_OUT) {
