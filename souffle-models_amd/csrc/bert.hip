@@ -233,9 +233,17 @@ using BigFc2 = GemmBig<H * kFc2Split / 16, kBigRing>;
 constexpr int kBigLds = BigFc1::LDS_BYTES;
 static_assert(BigQkv::LDS_BYTES <= kBigLds && BigOut::LDS_BYTES <= kBigLds && BigFc2::LDS_BYTES <= kBigLds, "FC1 has the largest ring");
 
-// Workgroup b runs on XCD b % 8.  An XCD gets a quarter of the row tiles and half of the
-// column tiles, so that its L2 fetches each operand tile it needs once.
+// Workgroup b runs on XCD b % 8.  With a multiple of 8 row tiles an XCD gets an eighth of them and all column
+// tiles; otherwise a quarter of the row tiles and half of the column tiles, so that its L2 fetches each operand
+// tile it needs once.
 __device__ __forceinline__ void big_tile(int it, int m_tiles, int n_tiles, int *tm, int *tn) {
+  if ((gridDim.x & 7) == 0 && (m_tiles & 7) == 0) {
+    // every tile of a row block on one XCD: what the block's 16 workgroups hand over to each other stays in that
+    // XCD's L2 (each XCD then streams all of W instead of half; 12 layers at 4096 rows: 1288 -> 1276 us)
+    const int x = it & 7, i = it >> 3, mo = m_tiles >> 3;
+    *tm = x * mo + i % mo;
+    *tn = i / mo;
+  } else
   if ((gridDim.x & 7) == 0 && (m_tiles & 3) == 0 && (n_tiles & 1) == 0) {
     const int x = it & 7, i = it >> 3, mq = m_tiles >> 2;
     *tm = (x & 3) * mq + i % mq;
@@ -553,6 +561,16 @@ __device__ __forceinline__ void attn_item(half_t *lds_h, const Params &a, int it
   attn_compute<COH, NKT>(lds, a, item);
 }
 
+using TileLarge = GemmTile<128, 128, 64, 2, 2>;
+constexpr int kAttnLdsBytes = 2 * 512 * 128 + 64 * 128;
+constexpr int kAttnAhead256 = 2 * (2 * 256 * 128 + 64 * 128);   // two items of S = 256 at a time
+constexpr int lds_bytes_large() {
+  const int t = TileLarge::LDS_BYTES > kBigLds ? TileLarge::LDS_BYTES : kBigLds;
+  const int u = t > kAttnLdsBytes ? t : kAttnLdsBytes;
+  return u > kAttnAhead256 ? u : kAttnAhead256;
+}
+constexpr int kMegaLds = lds_bytes_large();
+
 // One work unit after the other with the loads of the next in flight while this one is computed
 // (two LDS buffers).  `item_of(it)`: work unit -> item.
 template <bool COH, int NKT, class ItemOf>
@@ -573,6 +591,26 @@ __device__ __forceinline__ void attn_items_pipelined(unsigned char *lds, const P
     __syncthreads();   // this buffer is refilled in the next turn
     cur ^= 1;
   }
+}
+
+// Three items (base, base + 1, base + 2) with the loads of all three requested at once: an item's operands come from
+// the other workgroups of the row block and take some 2 us to arrive, its arithmetic 0.8 us, so that with one item
+// requested ahead each item still waited for most of a round trip.  Without mask and probabilities an item's
+// arithmetic issues exactly four vector memory instructions per lane (the context stores), which the waits count:
+// vector memory instructions of a wave complete in issue order.
+template <bool COH, int NKT>
+__device__ __forceinline__ void attn_three(unsigned char *lds, const Params &a, int base) {
+  constexpr int KL = kAttnLoads<NKT>, ITEM = kAttnItemLds<NKT>, STORES = HD / 16;
+  static_assert(3 * ITEM <= kMegaLds && 3 * KL + 2 * STORES < 64, "three buffers; vmcnt is a 6-bit counter");
+  __syncthreads();   // LDS reuse
+#pragma unroll
+  for (int j = 0; j < 3; ++j) attn_issue<NKT>(lds + j * ITEM, a, base + j);
+  static_for<0, 3>([&](auto jc) {
+    constexpr int j = decltype(jc)::value;
+    wait_vmcnt<(2 - j) * KL + j * STORES>();
+    __syncthreads();
+    attn_compute_t<COH, NKT, true>(lds + j * ITEM, a, base + j);
+  });
 }
 
 template <bool COH, int NKT, bool PLAIN>
@@ -669,7 +707,7 @@ __device__ __forceinline__ int attn_item_of(int it, int qblocks, int items) {
 template <bool COH, int NKT>
 __device__ __forceinline__ void stage_attn_t(half_t *lds, const Params &a, int first, int stride) {
   const int items = a.B * NH * (a.S / 64);
-  if constexpr (2 * kAttnItemLds<NKT> <= kBigLds)     // (the megakernel's LDS allocation is at least this)
+  if constexpr (2 * kAttnItemLds<NKT> <= kMegaLds)    // (the megakernel's LDS allocation)
     attn_items_pipelined<COH, NKT>(reinterpret_cast<unsigned char *>(lds), a, first, stride, items,
                                    [&](int it) { return attn_item_of(it, a.S / 64, items); });
   else
@@ -684,7 +722,10 @@ __device__ __forceinline__ void stage_attn_rowblock(unsigned char *lds, const Pa
     int tm, tn;
     big_tile(it, m_tiles, 16, &tm, &tn);
     const int base = tm * 48 + tn * 3;           // (the tiles of a group are numbered through: 16 tm + tn)
-    if constexpr (2 * kAttnItemLds<NKT> <= kBigLds)
+    if constexpr (3 * kAttnItemLds<NKT> <= kMegaLds) {
+      if (!a.mask && !a.probs) { attn_three<COH, NKT>(lds, a, base); continue; }
+    }
+    if constexpr (2 * kAttnItemLds<NKT> <= kMegaLds)
       attn_items_pipelined<COH, NKT>(lds, a, 0, 1, 3, [&](int j) { return base + j; });
     else
       for (int j = 0; j < 3; ++j) attn_item<COH, NKT>(reinterpret_cast<half_t *>(lds), a, base + j);
@@ -705,12 +746,6 @@ __device__ __forceinline__ void stage_attn(half_t *lds, const Params &a, int fir
   }
 }
 
-using TileLarge = GemmTile<128, 128, 64, 2, 2>;
-constexpr int kAttnLdsBytes = 2 * 512 * 128 + 64 * 128;
-constexpr int lds_bytes_large() {
-  const int t = TileLarge::LDS_BYTES > kBigLds ? TileLarge::LDS_BYTES : kBigLds;
-  return t > kAttnLdsBytes ? t : kAttnLdsBytes;
-}
 constexpr int lds_bytes_small() { return sk::kLdsBytes > sk::attn_lds_bytes(512) ? sk::kLdsBytes : sk::attn_lds_bytes(512); }
 static_assert(lds_bytes_small() <= 160 * 1024, "LDS of a CU");
 
