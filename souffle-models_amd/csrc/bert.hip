@@ -283,7 +283,7 @@ __device__ __forceinline__ void big_qkv(unsigned char *lds, const Params &a, con
       st16<COH>(a.qkv, ((((j * a.B + b) * NH + hh) * a.S + s) * HD + d) * 2, v);
     };
     f4 acc[BigQkv::MI][BigQkv::NT];
-    BigQkv::mainloop(lds, xin, H, tm * 256, 0, H / 32, wptr, acc, tb);
+    BigQkv::mainloop<H / 32>(lds, xin, H, tm * 256, 0, wptr, acc, tb);
     BigQkv::epilogue_rowvec(lds, tm * 256, acc, bias_at, cvt, store16, tb);
   }
 }
@@ -311,7 +311,7 @@ __device__ __forceinline__ void big_fc1(unsigned char *lds, const Params &a, con
     };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.h, (m * F + n0 + nr) * 2, v); };
     f4 acc[BigFc1::MI][BigFc1::NT];
-    BigFc1::mainloop(lds, a.y1, H, tm * 256, 0, H / 32, wptr, acc, tb);
+    BigFc1::mainloop<H / 32>(lds, a.y1, H, tm * 256, 0, wptr, acc, tb);
     if (a.act == SOUFFLE_ACT_RELU) BigFc1::epilogue_rowvec(lds, tm * 256, acc, bias_at, cvt_relu, store16, tb);
     else BigFc1::epilogue_rowvec(lds, tm * 256, acc, bias_at, cvt_gelu, store16, tb);
   }
@@ -335,7 +335,7 @@ __device__ __forceinline__ void big_presum(unsigned char *lds, const Params &a, 
     auto cvt = [&](int, int, f4 v, h4 bb) { return pack_h4(v + f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]}); };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.z1, (m * H + n0 + nr) * 2, v); };
     f4 acc[BigOut::MI][BigOut::NT];
-    BigOut::mainloop(lds, X, K, m0, 0, K / 32, wptr, acc);
+    BigOut::mainloop<H / 32>(lds, X, H, m0, 0, wptr, acc);      // (K = H: the out-projection)
     BigOut::epilogue_rowvec(lds, m0, acc, bias_at, cvt, store16);
   }
 }
@@ -358,7 +358,7 @@ __device__ __forceinline__ void big_presum2(unsigned char *lds, const Params &a,
     auto cvt = [&](int, int, f4 v) { return pack_h4(v); };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(zp, (m * H + n0 + nr) * 2, v); };
     f4 acc[BigFc2::MI][BigFc2::NT];
-    BigFc2::mainloop(lds, X, K, tm * 256, k0, (K / kFc2Split) / 32, wptr, acc);
+    BigFc2::mainloop<F / kFc2Split / 32>(lds, X, F, tm * 256, k0, wptr, acc);      // (K = F: FC2)
     BigFc2::epilogue(lds, tm * 256, acc, cvt, store16);
   }
 }

@@ -107,6 +107,9 @@ struct GemmBig {
     wait_vmcnt<A * LPW>();
   }
 
+  template <int KM, class Step, class A, class B, class C>
+  __device__ static __forceinline__ void template_km(Step &step, int kt, A a, B b, C c) { step(kt, std::integral_constant<int, KM>{}, a, b, c); }
+
   // LDS read look-ahead, in column tiles: the transposing reads of tile f + D are issued before the
   // MFMAs of tile f (f counts tiles across steps).  D + 1 divides NT, so the rotating operand
   // registers are used identically in every step.
@@ -127,11 +130,11 @@ struct GemmBig {
   // pipeline of the CU 30 cycles or more and stalls the wave meanwhile, which the four MFMAs
   // issued just before it cover.  (Issued as one burst after the barrier, the loads of the four
   // waves queue up behind each other and every SIMD idles: measured 2x the time per step.)
-  template <class WPtr, class Cvt, class Store16>
-  __device__ static __forceinline__ void run(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, int nkt, WPtr wptr, Cvt cvt, Store16 store16,
+  template <int NKT, class WPtr, class Cvt, class Store16>
+  __device__ static __forceinline__ void run(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, WPtr wptr, Cvt cvt, Store16 store16,
                                              const GridBarrier *tb = nullptr) {
     f4 acc[MI][NT];
-    mainloop(lds, X, ldx, m0, k0, nkt, wptr, acc, tb);
+    mainloop<NKT>(lds, X, ldx, m0, k0, wptr, acc, tb);
     epilogue(lds, m0, acc, cvt, store16, tb);
   }
 
@@ -139,9 +142,14 @@ struct GemmBig {
   // which half of K): they branch once between two epilogue() calls.  A uniform condition tested inside
   // cvt is not hoisted by the compiler but tested per result, and the tiny basic blocks in between
   // serialise every dependent chain (FC1 with GELU: 12.8 us per tile instead of 5).
-  template <class WPtr>
-  __device__ static __forceinline__ void mainloop(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, int nkt, WPtr wptr, f4 (&acc)[MI][NT],
+  // NKT: K steps of the tile, a compile-time multiple of NSTAGE: the steps between the first and the last NSTAGE-1
+  // then run in groups of NSTAGE in which every step knows its ring stage at compile time, so that the LDS addresses
+  // of a step's operand reads are a register that does not change plus an immediate.  (With the stage a run-time
+  // value a step began with some forty address instructions during which no MFMA was in flight.)
+  template <int NKT, class WPtr>
+  __device__ static __forceinline__ void mainloop(unsigned char *lds, const half_t *X, int ldx, int m0, int k0, WPtr wptr, f4 (&acc)[MI][NT],
                                                   const GridBarrier *tb = nullptr) {
+    static_assert(NKT % NSTAGE == 0 && NKT >= 2 * NSTAGE, "whole groups of steps between the first step and the last NSTAGE-1");
     const int tid = opaque_thread_id(), lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
     STAGE_MARK(tb, 0);
     __syncthreads();                                        // the previous user of the ring is done
@@ -165,9 +173,15 @@ struct GemmBig {
     }
     const int rho = wrow_of(g * 8 + (l16 >> 2));             // LDS row of the first of this lane's two k rows (k, k + 4: LDS rows rho, rho + 8)
     const int wrow = X_STAGE + rho * (BN * 2) + (l16 & 1) * 8, wsw = wswz(rho), wc = (l16 & 3) >> 1;
+    // slot of tile j: (2 j + wc) ^ wsw with wsw = 2 h, h < 4, i.e. 2 (j ^ h) + wc = 8 (j >> 2) + 2 ((j & 3) ^ h) + wc:
+    // four per-lane offsets (one per j & 3) and a compile-time 128 bytes per j >> 2
+    int woff[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) woff[q] = wrow + ((((q * 2 + wc) ^ wsw)) << 4);
 
-    auto read_w = [&](const unsigned char *st, int j) {
-      const half_t *p = reinterpret_cast<const half_t *>(st + wrow + (((j * 2 + wc) ^ wsw) << 4));
+    auto read_w = [&](const unsigned char *st, auto jc) {
+      constexpr int j = decltype(jc)::value;
+      const half_t *p = reinterpret_cast<const half_t *>(st + woff[j & 3] + (j >> 2) * 128);
       const h4 lo = lds_read_tr16(p), hh = lds_read_tr16(p + 8 * BN);
       return h8{lo[0], lo[1], lo[2], lo[3], hh[0], hh[1], hh[2], hh[3]};
     };
@@ -179,18 +193,18 @@ struct GemmBig {
     STAGE_MARK(tb, 1);
 #pragma unroll
     for (int i = 0; i < MI; ++i) x[i] = as_h8(lds_load16(lds + xoff[i]));
-#pragma unroll
-    for (int j = 0; j < D; ++j) w[j] = read_w(lds, j);
+    static_for<0, D>([&](auto jc) { w[decltype(jc)::value] = read_w(lds, jc); });
 
     // One K step.  LOAD_A: the tiles before the barrier issue the rest of stage kt+NSTAGE-2;
     // LOAD_B: the tiles from the barrier on issue the first part of stage kt+NSTAGE-1;
     // AHEAD: stages requested after stage kt+1 at the time of the wait.  All compile-time so that
     // the body has no branches.
-    auto step = [&](int kt, auto load_a, auto load_b, auto ahead_c) {
+    // kmc: kt % NSTAGE as a constant
+    auto step = [&](int kt, auto kmc, auto load_a, auto load_b, auto ahead_c) {
       constexpr bool LOAD_A = decltype(load_a)::value, LOAD_B = decltype(load_b)::value;
-      constexpr int AHEAD = decltype(ahead_c)::value;
-      const unsigned char *st = lds + (kt % NSTAGE) * STAGE, *stn = lds + ((kt + 1) % NSTAGE) * STAGE;
-      const unsigned ring_a = ring + ((kt + NSTAGE - 2) % NSTAGE) * STAGE, ring_b = ring + ((kt + NSTAGE - 1) % NSTAGE) * STAGE;
+      constexpr int AHEAD = decltype(ahead_c)::value, KM = decltype(kmc)::value;
+      const unsigned char *st = lds + KM * STAGE, *stn = lds + ((KM + 1) % NSTAGE) * STAGE;
+      const unsigned ring_a = ring + ((KM + NSTAGE - 2) % NSTAGE) * STAGE, ring_b = ring + ((KM + NSTAGE - 1) % NSTAGE) * STAGE;
       const int kk_a = k0 + (kt + NSTAGE - 2) * 32, kk_b = kk_a + 32;
       static_for<0, NT>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
@@ -204,7 +218,8 @@ struct GemmBig {
           for (int i = 0; i < MI; ++i) xn[i] = as_h8(lds_load16(stn + xoff[i]));
         }
         // (in the last step these read a stale buffer; the values are never used)
-        w[(j + D) % (D + 1)] = j + D < NT ? read_w(st, j + D) : read_w(stn, j + D - NT);
+        if constexpr (j + D < NT) w[(j + D) % (D + 1)] = read_w(st, std::integral_constant<int, j + D>{});
+        else w[(j + D) % (D + 1)] = read_w(stn, std::integral_constant<int, j + D - NT>{});
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
           mfma_16x16x32_inplace(acc[i][j], w[j % (D + 1)], x[i]);
@@ -222,17 +237,22 @@ struct GemmBig {
     };
     using T = std::true_type;
     using F = std::false_type;
-    // nkt >= NSTAGE (the callers' shapes: K >= 192).  Stages 0 .. NSTAGE-2 were requested above.
-    const int main_end = nkt - (NSTAGE - 1);               // steps 1 .. main_end-1 request on both sides of the barrier
-    step(0, F{}, T{}, std::integral_constant<int, NSTAGE - 3>{});
-    for (int kt = 1; kt < main_end; ++kt) step(kt, T{}, T{}, std::integral_constant<int, NSTAGE - 3>{});
-    // the last NSTAGE-1 steps: the first still completes stage nkt-1; after stage kt+1 there are
+    // Stages 0 .. NSTAGE-2 were requested above.
+    constexpr int main_end = NKT - (NSTAGE - 1);           // steps 1 .. main_end-1 request on both sides of the barrier
+    static_assert((main_end - 1) % NSTAGE == 0, "whole groups");
+    template_km<0>(step, 0, F{}, T{}, std::integral_constant<int, NSTAGE - 3>{});
+    for (int kt = 1; kt < main_end; kt += NSTAGE)
+      static_for<0, NSTAGE>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        template_km<(1 + i) % NSTAGE>(step, kt + i, T{}, T{}, std::integral_constant<int, NSTAGE - 3>{});
+      });
+    // the last NSTAGE-1 steps: the first still completes stage NKT-1; after stage kt+1 there are
     // NSTAGE-3, ..., 1, 0, 0 stages in flight
-    step(main_end + 0, T{}, F{}, std::integral_constant<int, (NSTAGE - 3 > 0 ? NSTAGE - 3 : 0)>{});
-    step(main_end + 1, F{}, F{}, std::integral_constant<int, (NSTAGE - 4 > 0 ? NSTAGE - 4 : 0)>{});
-    step(main_end + 2, F{}, F{}, std::integral_constant<int, (NSTAGE - 5 > 0 ? NSTAGE - 5 : 0)>{});
-    if constexpr (NSTAGE >= 5) step(main_end + 3, F{}, F{}, std::integral_constant<int, (NSTAGE - 6 > 0 ? NSTAGE - 6 : 0)>{});
-    if constexpr (NSTAGE >= 6) step(main_end + 4, F{}, F{}, std::integral_constant<int, 0>{});
+    template_km<(main_end + 0) % NSTAGE>(step, main_end + 0, T{}, F{}, std::integral_constant<int, (NSTAGE - 3 > 0 ? NSTAGE - 3 : 0)>{});
+    template_km<(main_end + 1) % NSTAGE>(step, main_end + 1, F{}, F{}, std::integral_constant<int, (NSTAGE - 4 > 0 ? NSTAGE - 4 : 0)>{});
+    template_km<(main_end + 2) % NSTAGE>(step, main_end + 2, F{}, F{}, std::integral_constant<int, (NSTAGE - 5 > 0 ? NSTAGE - 5 : 0)>{});
+    if constexpr (NSTAGE >= 5) template_km<(main_end + 3) % NSTAGE>(step, main_end + 3, F{}, F{}, std::integral_constant<int, (NSTAGE - 6 > 0 ? NSTAGE - 6 : 0)>{});
+    if constexpr (NSTAGE >= 6) template_km<(main_end + 4) % NSTAGE>(step, main_end + 4, F{}, F{}, std::integral_constant<int, 0>{});
 #pragma unroll
     for (int i = 0; i < MI; ++i) mfma_pin(acc[i], false);
     STAGE_MARK(tb, 2);
