@@ -951,6 +951,7 @@ static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += round_up(bytes, 256); return o; };
   p.off_ctl = take(kCtlWords * 4);
+  off = round_up(off, 4096);                           // (the 4 KB blocks of the flag copies on 4 KB boundaries of an aligned workspace)
   p.off_flags = take(sk::kFlagRegionWords * 4);        // (at a fixed place, whatever the configuration)
   const size_t first = off;
   p.off_qkv = take(3 * M * H * 2);
