@@ -1412,6 +1412,24 @@ extern "C" int souffle_bert_handover_plan(int batch, int seq_len, int grid, int 
   return SOUFFLE_OK;
 }
 
+extern "C" int souffle_bert_polled_copies(const void *ws, size_t ws_bytes, int *votes_cast, int *copy_block, souffle_stream_t stream) {
+  namespace sk = bert::sk;
+  if (!ws || !votes_cast || !copy_block) return fail(SOUFFLE_ERR_NULL, "ws, votes_cast and copy_block must not be NULL");
+  souffle_bert_cfg c{};
+  c.batch = 1; c.seq_len = 128;
+  const bert::Plan p = bert::make_plan(&c, 1);          // (the flag words lie at the same place in every plan)
+  if (ws_bytes < p.off_flags + (size_t)sk::kFlagWords * 4) return fail(SOUFFLE_ERR_WORKSPACE, "workspace too small to hold the flag words");
+  unsigned words[8];
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  SOUFFLE_HIP_TRY(hipMemcpyAsync(words, static_cast<const char *>(ws) + p.off_flags + (size_t)sk::kSideWord * 4, sizeof(words), hipMemcpyDeviceToHost, st));
+  SOUFFLE_HIP_TRY(hipStreamSynchronize(st));
+  for (int x = 0; x < 8; ++x) {
+    votes_cast[x] = (int)(words[x] & 0xffffu);
+    copy_block[x] = sk::pair_base_of(x) + (((int)words[x] >> 16) < 0 ? 2 : 0);
+  }
+  return SOUFFLE_OK;
+}
+
 extern "C" int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
                                             const void *x, const void *mask, void *y, void *ws, size_t ws_bytes,
                                             souffle_stream_t stream) {

@@ -191,6 +191,39 @@ def test_few_rows_handovers_on_repeated_launches(B, S, layers):
     assert_close("encoder x1", z_1, oracle.bert_encoder(x1, ws, B, S))
 
 
+def test_few_rows_polled_copy_is_voted_in_the_first_launches():
+    """Each XCD polls one of two copies of the hand-over words; which one is decided by votes that workgroup x of
+    XCD x casts at the end of the first eight launches on a workspace.  A fresh workspace has no votes and polls the
+    first copy of every pair; after ten launches every XCD has its eight votes and polls a block of its own pair;
+    the output is the same bits whichever copy is polled."""
+    announce("bert encoder few rows: votes on the polled copy")
+    import ctypes as C
+    import bert_binding
+    import souffle_hip as sh
+    B, S, layers = 1, 128, 2
+    dws = [dev_weights(synth.bert_layer_weights(3, l, with_bias=True)) for l in range(layers)]
+    enc = bert_binding.Encoder(dws, B, S)
+    enc.ws = sh.Workspace(enc.ws.nbytes)                     # (a fresh, zeroed one: the binding shares workspaces between encoders)
+    x = dev(synth.bert_input(9, B, S))
+
+    def polled():
+        votes, blocks = (C.c_int * 8)(), (C.c_int * 8)()
+        sh.check(sh.lib().souffle_bert_polled_copies(enc.ws.ptr, enc.ws.nbytes, votes, blocks, sh.current_stream()))
+        return list(votes), list(blocks)
+
+    votes, blocks = polled()
+    assert votes == [0] * 8 and blocks == [(x_ >> 1) * 4 + (x_ & 1) for x_ in range(8)]
+    first = enc(x).clone()
+    for i in range(9):
+        assert torch.equal(enc(x), first), "launch %d" % (i + 2)
+    votes, blocks = polled()
+    assert votes == [8] * 8, votes
+    for x_ in range(8):
+        base = (x_ >> 1) * 4 + (x_ & 1)
+        assert blocks[x_] in (base, base + 2), (x_, blocks)
+    assert enc.ws.status() == 0
+
+
 def test_few_rows_shapes_take_turns_in_one_workspace():
     """Flag words, ticket counters and completion words of the few-rows kernel carry over from launch to launch
     and are indexed by shape-dependent tile numbers: encoders of different shapes and depths, fused and per-op,
