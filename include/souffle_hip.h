@@ -193,7 +193,7 @@ int souffle_bert_handover_plan(int batch, int seq_len, int grid, int phase, int 
 
 /* Which copy of its hand-over words each XCD polls in the few-rows encoder, read back from a workspace (a diagnostic;
  * synchronises the stream; no counterpart in the reference).  The words exist in 16 copies of 4 KB, two per XCD and
- * 8 KB apart, so that one of the two lies in memory channels on the XCD's side of the package; workgroup x of XCD x
+ * 8 KB apart (their addresses differ in bit 13 only), so that one of the two lies in memory channels on the XCD's side of the package; workgroup x of XCD x
  * times loads of both at the end of each of the first 8 launches on a workspace and the majority decides.
  * votes_cast[x] = votes so far (0..8), copy_block[x] = the 4 KB block XCD x polls in the next launch. */
 int souffle_bert_polled_copies(const void *ws, size_t ws_bytes, int *votes_cast, int *copy_block, souffle_stream_t stream);
