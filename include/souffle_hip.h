@@ -130,7 +130,21 @@ typedef struct {
   const void *w_fc2;  /* [3072][768]   */
   const void *b_fc2;  /* [768]         */
   const void *ln2_g, *ln2_b;
+  const void *w_fc2_packed;  /* optional: the copy of w_fc2 that souffle_bert_pack_fc2 makes, or NULL */
 } souffle_bert_layer_w;
+
+/* A one-time copy of a layer's w_fc2 ([3072][768], which stays required) in the order the few-rows encoder reads it:
+ * 48 slices of 16 output columns, each the 96 k-steps of its MFMA operands, contiguous (souffle_bert_fc2_packed_bytes()
+ * = 3072 * 768 * 2 bytes, 16-byte aligned, not overlapping w_fc2).  Make it once when a model is loaded and pass it
+ * as w_fc2_packed of the layer.  When EVERY layer of a call has it, and the call runs on the few-rows kernel (up to
+ * 1024 rows, and below 1536 where the count is no multiple of 256), a workgroup computes 32 rows x 16 columns of FC2
+ * over the whole K = 3072 and finishes them itself (bias, residual, row statistics).  Without it FC2 is cut into four
+ * K quarters whose fp32 partial sums are exchanged through memory (the in-block split-K of
+ * cpp/bert/kernels/gemm.cu:1260-1330 spread over four workgroups), which costs about 3 us more per layer.
+ * Same arithmetic up to the order of the fp32 additions over K.  The reference keeps [K][N] only; it has no
+ * counterpart of the packed copy. */
+size_t souffle_bert_fc2_packed_bytes(void);
+int souffle_bert_pack_fc2(const void *w_fc2, void *packed, souffle_stream_t stream);
 
 /* Optional fp16 device outputs for the per-stage tensors the reference binding returns
  * (cpp/bert/bert_binding.cu:534); any member (or the struct pointer) may be NULL. */
@@ -184,11 +198,13 @@ int souffle_bert_encoder_fused_static(const souffle_bert_cfg *cfg, const souffle
  * no multiple of 256), evaluated on the host by the functions the
  * kernel itself uses (no GPU needed; no counterpart in the reference, whose stages are separated by grid barriers):
  * the items of `workgroup` in `phase` (0 QKV, 1 attention, 2 out-projection, 3 FC1, 4 FC2, 6 final LayerNorm) as
- * pairs (m-tile, weight slice) - attention: (block of 16 queries, batch * 12 + head) - written to items[2 i], items[2 i + 1]
+ * pairs (m-tile, weight slice) - attention: (block of 16 queries, batch * 12 + head); FC2: slice = 16 output columns
+ * when fc2_packed != 0 (every layer brings w_fc2_packed), else 64-column slice * 4 + K quarter - written to items[2 i], items[2 i + 1]
  * (at most max_items pairs; *n_items is their true number), and needs[p] = 1 for every workgroup p of the `grid` whose
- * publication of the phase before the workgroup waits for (phases 1..4; QKV and the final LayerNorm wait for the
- * completion words of the twelve FC2 tiles of their m-tile instead).  items and needs may be NULL. */
-int souffle_bert_handover_plan(int batch, int seq_len, int grid, int phase, int workgroup, int *items, int max_items,
+ * publication of the phase before the workgroup waits for (phases 1..4; QKV of a later layer and the final LayerNorm
+ * wait for FC2: with fc2_packed for the publications of its workgroups, reported here for phases 0 and 6 too, otherwise
+ * for the completion words of the twelve FC2 tiles of their m-tile).  items and needs may be NULL. */
+int souffle_bert_handover_plan(int batch, int seq_len, int grid, int fc2_packed, int phase, int workgroup, int *items, int max_items,
                                int *n_items, unsigned char *needs);
 
 /* Which copy of its hand-over words each XCD polls in the few-rows encoder, read back from a workspace (a diagnostic;

@@ -52,8 +52,18 @@ def make_cfg(batch, seq_len, act="gelu_tanh", scale=0.125, ln_eps=1e-12, num_lay
     return sh.BertCfg(batch, seq_len, HIDDEN, HEADS, FFN, acts[act], float(scale), float(ln_eps), num_layers, 0)
 
 
+def pack_fc2(fc2_weight):
+    """The one-time copy of a layer's fc2 weight [3072][768] in the order the few-rows encoder reads it
+    (souffle_bert_pack_fc2): made once per model, passed as fc2_packed of the layer."""
+    _check_f16_cuda("feed_forward_fc2_weight", fc2_weight, (FFN, HIDDEN))
+    packed = torch.empty(sh.lib().souffle_bert_fc2_packed_bytes() // 2, dtype=torch.float16, device=fc2_weight.device)
+    sh.check(sh.lib().souffle_bert_pack_fc2(fc2_weight.data_ptr(), packed.data_ptr(), sh.current_stream()))
+    return packed
+
+
 def make_layer_w(qkv_weight, attn_fc_weight, fc1_weight, fc2_weight, qkv_bias=None, attn_fc_bias=None,
-                 ln1_gamma=None, ln1_beta=None, fc1_bias=None, fc2_bias=None, ln2_gamma=None, ln2_beta=None):
+                 ln1_gamma=None, ln1_beta=None, fc1_bias=None, fc2_bias=None, ln2_gamma=None, ln2_beta=None,
+                 fc2_packed=None):
     _check_f16_cuda("qkv_weight", qkv_weight, (3, HIDDEN, HIDDEN))
     _check_f16_cuda("attn_fc_weight", attn_fc_weight, (HIDDEN, HIDDEN))
     _check_f16_cuda("feed_forward_fc1_weight", fc1_weight, (HIDDEN, FFN))
@@ -68,9 +78,13 @@ def make_layer_w(qkv_weight, attn_fc_weight, fc1_weight, fc2_weight, qkv_bias=No
                 raise ValueError("%s must have %d elements" % (name, n))
     w = sh.BertLayerW(sh.ptr(qkv_weight), sh.ptr(qkv_bias), sh.ptr(attn_fc_weight), sh.ptr(attn_fc_bias),
                       sh.ptr(ln1_gamma), sh.ptr(ln1_beta), sh.ptr(fc1_weight), sh.ptr(fc1_bias),
-                      sh.ptr(fc2_weight), sh.ptr(fc2_bias), sh.ptr(ln2_gamma), sh.ptr(ln2_beta))
+                      sh.ptr(fc2_weight), sh.ptr(fc2_bias), sh.ptr(ln2_gamma), sh.ptr(ln2_beta), sh.ptr(fc2_packed))
+    if fc2_packed is not None:
+        _check_f16_cuda("fc2_packed", fc2_packed)
+        if fc2_packed.numel() != FFN * HIDDEN:
+            raise ValueError("fc2_packed must have %d elements" % (FFN * HIDDEN))
     w._keep = (qkv_weight, attn_fc_weight, fc1_weight, fc2_weight, qkv_bias, attn_fc_bias, ln1_gamma, ln1_beta,
-               fc1_bias, fc2_bias, ln2_gamma, ln2_beta)
+               fc1_bias, fc2_bias, ln2_gamma, ln2_beta, fc2_packed)
     return w
 
 
@@ -86,12 +100,13 @@ def _batch_seq(src, batch, seq_len):
 
 def souffle_bert_layer(src, qkv_weight, attn_fc_weight, feed_forward_fc1_weight, feed_forward_fc2_weight,
                        opt_level, *, act="gelu_tanh", scale=0.125, ln_eps=1e-12, reference_compat=False,
-                       mask=None, batch=None, seq_len=None, dump=True, **biases):
+                       mask=None, batch=None, seq_len=None, dump=True, pack=False, **biases):
     """One encoder layer.  opt_level 0-2: per-op HIP launches; 3-4: the fused megakernel
     (the reference's levels: cpp/bert/bert_binding.cu:119-531).  Returns
     [output_qkv, query_key_output, attn_value_output, attn_fc_output,
      feed_forward_fc1_output, feed_forward_fc2_output] as cpp/bert/bert_binding.cu:534.
-    With dump=False only the final output is produced and returned (fast path)."""
+    With dump=False only the final output is produced and returned (fast path).  pack=True makes the packed copy
+    of the fc2 weight for this call (a model object makes it once: Encoder), so that FC2 runs in its whole-K form."""
     if opt_level not in (0, 1, 2, 3, 4):
         raise ValueError("opt_level %r is not supported" % (opt_level,))   # reference prints and returns
     _check_f16_cuda("src", src)
@@ -101,6 +116,8 @@ def souffle_bert_layer(src, qkv_weight, attn_fc_weight, feed_forward_fc1_weight,
         act, scale, ln_eps = "relu", 1.0 / (HIDDEN ** 0.5), 1e-5
     B, S = _batch_seq(src, batch, seq_len)
     cfg = make_cfg(B, S, act, scale, ln_eps)
+    if pack and biases.get("fc2_packed") is None:
+        biases = dict(biases, fc2_packed=pack_fc2(feed_forward_fc2_weight))
     w = make_layer_w(qkv_weight, attn_fc_weight, feed_forward_fc1_weight, feed_forward_fc2_weight, **biases)
     if mask is not None:
         _check_f16_cuda("mask", mask, (B, S, S))
@@ -145,8 +162,12 @@ class Encoder:
     (fused=True) or as per-op launches.  Stands in for the reference's souffle_bert_base()
     (cpp/bert/bert_base_impl.cu:277-308), which allocates its own zero weights."""
 
-    def __init__(self, layers, batch, seq_len, act="gelu_tanh", scale=0.125, ln_eps=1e-12, device="cuda:0"):
+    def __init__(self, layers, batch, seq_len, act="gelu_tanh", scale=0.125, ln_eps=1e-12, device="cuda:0", pack=True):
         self.cfg = make_cfg(batch, seq_len, act, scale, ln_eps, num_layers=len(layers))
+        # a model object is built once: the place for the one-time packed copy of every fc2 weight (pack=False keeps
+        # the [K][N] matrices only, as the per-call entry point souffle_bert_layer does)
+        if pack:
+            layers = [l if l.get("fc2_packed") is not None else dict(l, fc2_packed=pack_fc2(l["fc2_weight"])) for l in layers]
         self._w = [make_layer_w(**l) for l in layers]
         self.warr = (sh.BertLayerW * len(layers))(*self._w)
         self.ws = _workspace(self.cfg, torch.device(device))

@@ -966,8 +966,8 @@ static Plan make_plan(const souffle_bert_cfg *c, int num_layers) {
   } else {
     p.off_part = take((size_t)4 * M * H * 4);
     p.off_z2 = take(M * H * 2);
-    p.off_st1 = take(M * 12 * 8);
-    p.off_st2 = take(M * 12 * 8);
+    p.off_st1 = take(M * sk::kNS1 * 8);
+    p.off_st2 = take(M * sk::kNS2 * 8);
   }
   p.layer_stride = off - first;                       // one set of inter-stage buffers per layer
   const int nl = num_layers < 1 ? 1 : num_layers;
@@ -1013,6 +1013,8 @@ static int fill_layers(LayerW *dst, const souffle_bert_layer_w *layers, int nl) 
     d.w_qkv = (const half_t *)s.w_qkv; d.b_qkv = (const half_t *)s.b_qkv; d.w_o = (const half_t *)s.w_o; d.b_o = (const half_t *)s.b_o;
     d.ln1_g = (const half_t *)s.ln1_g; d.ln1_b = (const half_t *)s.ln1_b; d.w_fc1 = (const half_t *)s.w_fc1; d.b_fc1 = (const half_t *)s.b_fc1;
     d.w_fc2 = (const half_t *)s.w_fc2; d.b_fc2 = (const half_t *)s.b_fc2; d.ln2_g = (const half_t *)s.ln2_g; d.ln2_b = (const half_t *)s.ln2_b;
+    d.w_fc2p = (const half_t *)s.w_fc2_packed;
+    if (!aligned16(s.w_fc2_packed)) return fail(SOUFFLE_ERR_ALIGN, "layer %d: w_fc2_packed is not 16-byte aligned", l);
   }
   return SOUFFLE_OK;
 }
@@ -1073,18 +1075,25 @@ static int fill_small(sk::Args &a, const souffle_bert_cfg *c, const souffle_bert
   a.layer_stride = p.layer_stride;
   a.probs = nullptr;
   a.ln1_out = nullptr;
+  a.fc1_out = nullptr;
   a.trace = nullptr;
   a.trace_cap = 0;
   if (dump) {   // (a single layer: the per-stage tensors are produced in the reference's own layouts, in place)
     if (dump->qkv) a.qkv = static_cast<half_t *>(dump->qkv);
     if (dump->ctx) a.ctx = static_cast<half_t *>(dump->ctx);
-    if (dump->fc1) a.h = static_cast<half_t *>(dump->fc1);
+    a.fc1_out = static_cast<half_t *>(dump->fc1);      // (moved into a.h below unless h is kept in operand order)
     a.ln1_out = static_cast<half_t *>(dump->ln1);
     a.probs = static_cast<half_t *>(dump->probs);
-    if (!aligned16(a.qkv) || !aligned16(a.ctx) || !aligned16(a.ln1_out) || !aligned16(a.h) || !aligned16(a.probs))
+    if (!aligned16(a.qkv) || !aligned16(a.ctx) || !aligned16(a.ln1_out) || !aligned16(a.fc1_out) || !aligned16(a.probs))
       return fail(SOUFFLE_ERR_ALIGN, "dump pointers must be 16-byte aligned");
   }
-  return fill_layers(a.layers, layers, nl);
+  if (int rc = fill_layers(a.layers, layers, nl)) return rc;
+  // FC2 runs in its whole-K form when every layer brings the packed copy of its weights (souffle_bert_pack_fc2)
+  a.packed = 1;
+  for (int l = 0; l < nl; ++l)
+    if (!a.layers[l].w_fc2p) a.packed = 0;
+  if (!a.packed && a.fc1_out) { a.h = a.fc1_out; a.fc1_out = nullptr; }      // row-major h: written in place
+  return SOUFFLE_OK;
 }
 
 template <int MODE, int NKT>
@@ -1102,11 +1111,16 @@ static int launch_mega_t(Args &a, int grid, hipStream_t st) {
 template <int MODE>
 static int launch_mega(Args &a, int grid, hipStream_t st) {
   switch (a.S) {
+#ifdef SOUFFLE_DEV_ONLY_S128      // development builds: one sequence length, a fifth of the compile time
+    case 128: return launch_mega_t<MODE, 8>(a, grid, st);
+    default: return fail(SOUFFLE_ERR_SHAPE, "development build: seq_len 128 only");
+#else
     case 64: return launch_mega_t<MODE, 4>(a, grid, st);
     case 128: return launch_mega_t<MODE, 8>(a, grid, st);
     case 256: return launch_mega_t<MODE, 16>(a, grid, st);
     case 384: return launch_mega_t<MODE, 24>(a, grid, st);
     default: return launch_mega_t<MODE, 32>(a, grid, st);
+#endif
   }
 }
 
@@ -1123,16 +1137,21 @@ static int launch_small_tt(sk::Args &a, int grid, hipStream_t st) {
 }
 template <int NKT>
 static int launch_small_t(sk::Args &a, int grid, hipStream_t st) {
-  const sk::Shape sh{a.B, a.S, a.M, a.M / 32, grid};
+  const sk::Shape sh{a.B, a.S, a.M, a.M / 32, grid, a.packed};
   return sk::single_pass(sh) ? launch_small_tt<NKT, false>(a, grid, st) : launch_small_tt<NKT, true>(a, grid, st);
 }
 static int launch_small(sk::Args &a, int grid, hipStream_t st) {
   switch (a.S) {
+#ifdef SOUFFLE_DEV_ONLY_S128      // development builds: one sequence length, a fifth of the compile time
+    case 128: return launch_small_t<8>(a, grid, st);
+    default: return fail(SOUFFLE_ERR_SHAPE, "development build: seq_len 128 only");
+#else
     case 64: return launch_small_t<4>(a, grid, st);
     case 128: return launch_small_t<8>(a, grid, st);
     case 256: return launch_small_t<16>(a, grid, st);
     case 384: return launch_small_t<24>(a, grid, st);
     default: return launch_small_t<32>(a, grid, st);
+#endif
   }
 }
 // The same phases as separate launches: 6 per layer and one at the end.  Every launch has the grid of the fused
@@ -1156,11 +1175,16 @@ static int run_small_unfused_t(sk::Args &a, int grid, hipStream_t st) {
 }
 static int run_small_unfused(sk::Args &a, int grid, hipStream_t st) {
   switch (a.S) {
+#ifdef SOUFFLE_DEV_ONLY_S128      // development builds: one sequence length, a fifth of the compile time
+    case 128: return run_small_unfused_t<8>(a, grid, st);
+    default: return fail(SOUFFLE_ERR_SHAPE, "development build: seq_len 128 only");
+#else
     case 64: return run_small_unfused_t<4>(a, grid, st);
     case 128: return run_small_unfused_t<8>(a, grid, st);
     case 256: return run_small_unfused_t<16>(a, grid, st);
     case 384: return run_small_unfused_t<24>(a, grid, st);
     default: return run_small_unfused_t<32>(a, grid, st);
+#endif
   }
 }
 
@@ -1390,9 +1414,39 @@ extern "C" int souffle_bert_encoder_fused_static(const souffle_bert_cfg *cfg, co
   return bert::run_fused(cfg, layers, nl, x, mask, y, nullptr, sc->ptr, bert::kStaticScratchBytes, stream);
 }
 
+// w_fc2 [3072][768] -> 48 slices of 16 output columns, each 96 k-steps of 1 KB: lane L of a wave finds the eight
+// halves W[32 t + 8 (L / 16) + 0..7][16 s + L % 16] (its A operand of the 16x16x32 MFMA of k-step t) at
+// ((s * 96 + t) * 64 + L) * 16 bytes.  One thread per 16 bytes of output.
+namespace souffle {
+namespace bert {
+__global__ void __launch_bounds__(256) k_pack_fc2(const half_t *w, half_t *out) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;               // (s * 96 + t) * 64 + L
+  if (idx >= 48 * 96 * 64) return;
+  const int L = idx & 63, t = (idx >> 6) % 96, s = idx / (96 * 64);
+  const half_t *src = w + (size_t)(32 * t + 8 * (L >> 4)) * H + 16 * s + (L & 15);
+  h8 v;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = src[(size_t)j * H];
+  *reinterpret_cast<h8 *>(out + (size_t)idx * 8) = v;
+}
+}  // namespace bert
+}  // namespace souffle
+extern "C" size_t souffle_bert_fc2_packed_bytes(void) { return (size_t)bert::F * bert::H * 2; }
+extern "C" int souffle_bert_pack_fc2(const void *w_fc2, void *packed, souffle_stream_t stream) {
+  if (!w_fc2 || !packed) return fail(SOUFFLE_ERR_NULL, "w_fc2 and packed must not be NULL");
+  if (!aligned16(w_fc2) || !aligned16(packed)) return fail(SOUFFLE_ERR_ALIGN, "w_fc2 and packed must be 16-byte aligned");
+  const char *a = static_cast<const char *>(w_fc2), *b = static_cast<const char *>(packed);
+  const size_t n = souffle_bert_fc2_packed_bytes();
+  if (a < b + n && b < a + n) return fail(SOUFFLE_ERR_SHAPE, "w_fc2 and packed overlap");
+  hipLaunchKernelGGL(bert::k_pack_fc2, dim3(48 * 96 * 64 / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const half_t *>(w_fc2), static_cast<half_t *>(packed));
+  SOUFFLE_HIP_TRY(hipGetLastError());
+  return SOUFFLE_OK;
+}
+
 // The work split and the hand-over plan of the few-rows encoder, evaluated on the host with the very functions the
 // kernel uses: for tests that check the plan against a model of which rows and columns every item reads and writes.
-extern "C" int souffle_bert_handover_plan(int batch, int seq_len, int grid, int phase, int workgroup, int *items, int max_items,
+extern "C" int souffle_bert_handover_plan(int batch, int seq_len, int grid, int fc2_packed, int phase, int workgroup, int *items, int max_items,
                                           int *n_items, unsigned char *needs) {
   namespace sk = bert::sk;
   if (!n_items) return fail(SOUFFLE_ERR_NULL, "n_items is NULL");
@@ -1400,7 +1454,7 @@ extern "C" int souffle_bert_handover_plan(int batch, int seq_len, int grid, int 
     return fail(SOUFFLE_ERR_SHAPE, "the few-rows plan exists for seq_len in {64,128,256,384,512} and the row counts that the few-rows kernel runs (got %d x %d)", batch, seq_len);
   if (grid <= 0 || grid > 1024 || workgroup < 0 || workgroup >= grid) return fail(SOUFFLE_ERR_SHAPE, "grid must be in 1..1024 and workgroup below it");
   if (phase < sk::PH_QKV || phase > sk::PH_FIN || phase == sk::PH_RED) return fail(SOUFFLE_ERR_SHAPE, "phase must be 0 (QKV), 1 (ATT), 2 (OUT), 3 (FC1), 4 (FC2) or 6 (FIN)");
-  const sk::Shape sh{batch, seq_len, batch * seq_len, batch * seq_len / 32, grid};
+  const sk::Shape sh{batch, seq_len, batch * seq_len, batch * seq_len / 32, grid, fc2_packed ? 1 : 0};
   int n = 0;
   sk::It d;
   for (; sk::wg_item(sh, phase, workgroup, n, d); ++n)
@@ -1408,7 +1462,8 @@ extern "C" int souffle_bert_handover_plan(int batch, int seq_len, int grid, int 
   *n_items = n;
   if (needs)
     for (int pb = 0; pb < grid; ++pb)
-      needs[pb] = (phase >= sk::PH_ATT && phase <= sk::PH_FC2 && sk::wait_needs(sh, phase, workgroup, pb)) ? 1 : 0;
+      needs[pb] = (((phase >= sk::PH_ATT && phase <= sk::PH_FC2) || (fc2_packed && (phase == sk::PH_QKV || phase == sk::PH_FIN))) &&
+                   sk::wait_needs(sh, phase, workgroup, pb)) ? 1 : 0;
   return SOUFFLE_OK;
 }
 

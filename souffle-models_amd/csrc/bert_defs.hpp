@@ -11,6 +11,7 @@ constexpr int kMaxLayers = 24;
 
 struct LayerW {
   const half_t *w_qkv, *b_qkv, *w_o, *b_o, *ln1_g, *ln1_b, *w_fc1, *b_fc1, *w_fc2, *b_fc2, *ln2_g, *ln2_b;
+  const half_t *w_fc2p;      // w_fc2 in the layout of souffle_bert_pack_fc2, or null
 };
 
 __device__ __forceinline__ void add_bias8(f4 &lo, f4 &hi, const half_t *bias, int n) {

@@ -48,10 +48,12 @@ constexpr int kXPart = 12288;                 // per wave: its K quarter of the 
 constexpr int kWOff = 4 * kXPart;             // weight slice [768][64] fp16
 constexpr int kWBytes = 768 * 128;
 constexpr int kGamOff = kWOff + kWBytes;      // gamma and beta of the LayerNorm applied on load: 768 B per wave (its K quarter of each)
-constexpr int kBiasOff = kGamOff + 4 * 768;   // bias of the item's 64 columns
-constexpr int kAuxOff = kBiasOff + 512;       // LN GEMMs: the row statistics, one copy per wave (4 x 3 KB);
-constexpr int kStatBytes = 32 * 12 * 8;       // OUT: residual patch (4 KB) + one copy of the statistics
-constexpr int kLdsBytes = kAuxOff + 4 * kStatBytes;
+constexpr int kBiasOff = kGamOff + 4 * 768;   // bias of the item's columns (128 B), then
+constexpr int kRowTabOff = kBiasOff + 128;    // (mean, rstd) of the tile's 32 rows, combined from staged statistics (256 B), then
+constexpr int kTicketOff = kBiasOff + 384;    // the ticket of an FC2 K quarter (split-K form)
+constexpr int kAuxOff = kBiasOff + 512;       // row statistics: of z1, one copy of the tile's 32 x 12 per wave (4 x 3 KB); of z2,
+constexpr int kStatBytes = 32 * 12 * 8;       // wave w stages those of rows 8 w .. 8 w + 7 (8 x 48 entries = 3 KB); split-K FC2:
+constexpr int kLdsBytes = kAuxOff + 4 * kStatBytes;      // residual patch (4 KB) + one copy of z1's
 static_assert(kLdsBytes <= 160 * 1024, "LDS of a CU");
 constexpr int kRedLd = 68;                    // floats per row of a wave's partial tile
 static_assert(32 * kRedLd * 4 <= kXPart, "a wave's partial tile reuses its X part");
@@ -85,6 +87,7 @@ constexpr int kMaxFlagSpin = 1 << 21;                          // about a second
 
 struct Shape {
   int B, S, M, m_tiles, G;
+  int packed;            // FC2 in its whole-K form (weights packed by souffle_bert_pack_fc2): items (m-tile, 16 columns)
 };
 
 struct Sync {
@@ -199,12 +202,13 @@ __host__ __device__ __forceinline__ bool feeds(const Shape &s, int cph, const It
       return head == h && (32 * p.a) / s.S == b && (j != 0 || (b * s.S + 16 * c.a) / 32 == p.a);
     }
     case PH_OUT: return ((p.b / 12) * s.S + 16 * p.a) / 32 == c.a;                 // p = ATT
-    case PH_FC2: return p.a == c.a && p.b / 12 == (c.b & 3);                       // p = FC1 slice, c = n-slice * 4 + K quarter
-    default: return p.a == c.a;                                                    // FC1 <- OUT (whole rows of the m-tile)
+    case PH_FC2: return p.a == c.a && (s.packed || p.b / 12 == (c.b & 3));         // p = FC1 slice; split-K form: c = n-slice * 4 + K quarter
+    default: return p.a == c.a;                                                    // FC1 <- OUT, QKV / FIN <- FC2 (whole rows of the m-tile)
   }
 }
-// (phases ATT .. FC2 wait for the flag words of the phase before; QKV and FIN wait for completion words of tiles)
-__host__ __device__ __forceinline__ int producer_phase(int cph) { return cph - 1; }
+// Phases ATT .. FC2 wait for the flag words of the phase before.  QKV (of the layers after the first) and FIN wait for
+// FC2: for the flag words of its workgroups in the whole-K form, for the completion words of its tiles in the split-K form.
+__host__ __device__ __forceinline__ int producer_phase(int cph) { return cph == PH_QKV || cph == PH_FIN ? PH_FC2 : cph - 1; }
 
 // Must workgroup pb have published the producer phase before workgroup b may start its items of phase cph?
 // Yes if any item of pb in the producer phase writes something that any item of b in phase cph reads (a workgroup
@@ -345,45 +349,57 @@ __device__ __forceinline__ float sum32(float v) {           // 32 consecutive la
 }
 template <int LANES>
 __device__ __forceinline__ float sum_lanes(float v) {
-  static_assert(LANES == 8 || LANES == 32, "group sizes in use");
-  if constexpr (LANES == 8) return sum8(v); else return sum32(v);
+  static_assert(LANES == 2 || LANES == 4 || LANES == 8 || LANES == 32, "group sizes in use");
+  if constexpr (LANES == 2) return v + dpp_move<0xB1>(v);
+  else if constexpr (LANES == 4) return sum4(v);
+  else if constexpr (LANES == 8) return sum8(v);
+  else return sum32(v);
 }
 
 // ---- row statistics ----
-// st[m][12][2]: per row and per 64-column slice (mean, sum of squared deviations from that mean) of the fp16 values.
-// Combination of the twelve slices of a row (equal counts): mean = average of the means,
-// M2 = sum M2_i + 64 sum (mean_i - mean)^2.
+// st[m][NS][2]: per row and per slice of 768 / NS columns (mean, sum of squared deviations from that mean) of the fp16
+// values.  The out-projection writes its sum z1 in 64-column slices (NS = 12), FC2 its sum z2 in 16-column slices (NS = 48).
+// (Stored slice by slice instead, z2[48][M][16] and st2[48][M][2], an item's 32 rows of a slice are whole cache lines
+// instead of 32-byte and 8-byte pieces of lines that workgroups on other XCDs write at the same time: measured, 12
+// layers at B=1 took 1.5 us longer that way, 268.7 against 267.0 us.)
+// Combination of the slices of a row (equal counts n = 768 / NS): mean = average of the means,
+// M2 = sum M2_i + n sum (mean_i - mean)^2.
+constexpr int kNS1 = 12, kNS2 = 48;
 struct RowStat { float mean, rstd; };
 
-// 8 consecutive lanes share row m: lane t of the group reads slices t and t + 8.
+// 8 consecutive lanes share row m of the FC2 sum: lane t of the group combines slices 6 t .. 6 t + 5.
 __device__ __forceinline__ RowStat row_stat8(const float *st, int m, int t8, float eps) {
-  const u2 p0 = ld8<true>(st, (m * 12 + t8) * 8);
-  u2 p1 = {0u, 0u};
-  if (t8 < 4) p1 = ld8<true>(st, (m * 12 + 8 + t8) * 8);
-  const float m0 = f32_of(p0[0]), q0 = f32_of(p0[1]);
-  const float m1 = f32_of(p1[0]), q1 = f32_of(p1[1]);
-  const float s = sum8(m0 + (t8 < 4 ? m1 : 0.f));
-  const float mean = s * (1.0f / 12.0f);
-  float q = q0 + 64.0f * (m0 - mean) * (m0 - mean);
-  if (t8 < 4) q += q1 + 64.0f * (m1 - mean) * (m1 - mean);
+  float mi[6], qi[6];
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    const u4 v = ld16<true>(st, ((m * kNS2 + 6 * t8) * 2 + 4 * i) * 4);
+    mi[2 * i] = f32_of(v[0]); qi[2 * i] = f32_of(v[1]); mi[2 * i + 1] = f32_of(v[2]); qi[2 * i + 1] = f32_of(v[3]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 6; ++i) s += mi[i];
+  const float mean = sum8(s) * (1.0f / kNS2);
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < 6; ++i) q += qi[i] + (768.0f / kNS2) * (mi[i] - mean) * (mi[i] - mean);
   q = sum8(q);
   return RowStat{mean, rsqrtf(q * (1.0f / 768.0f) + eps)};
 }
-// Publish the statistics of 64 values of a row held by `n` consecutive lanes (v: this lane's values, already
-// rounded to fp16 and widened again); lane 0 of the group stores.
-template <int PER, int LANES>
+// Publish the statistics of the 768 / NS values of a row's slice held by LANES consecutive lanes (v: this lane's
+// values, already rounded to fp16 and widened again); lane 0 of the group stores.
+template <int PER, int LANES, int NS>
 __device__ __forceinline__ void put_stat(float *st, int m, int slice, const float (&v)[PER], int lane_in_group) {
-  static_assert(PER * LANES == 64, "a slice is 64 columns");
+  static_assert(PER * LANES * NS == 768, "a slice is 768 / NS columns");
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < PER; ++i) s += v[i];
   s = sum_lanes<LANES>(s);
-  const float mean = s * (1.0f / 64.0f);
+  const float mean = s * (1.0f / (PER * LANES));
   float q = 0.f;
 #pragma unroll
   for (int i = 0; i < PER; ++i) { const float d = v[i] - mean; q += d * d; }
   q = sum_lanes<LANES>(q);
-  if (lane_in_group == 0) st8<true>(st, (m * 12 + slice) * 8, u2{u32_of(mean), u32_of(q)});
+  if (lane_in_group == 0) st8<true>(st, (m * NS + slice) * 8, u2{u32_of(mean), u32_of(q)});
 }
 
 // ---- GEMM item: 32 rows x 64 columns over a K slice of 768 ----
@@ -396,6 +412,7 @@ __device__ __forceinline__ void put_stat(float *st, int m, int slice, const floa
 struct GemmItem {
   const half_t *X; int ldx, kx0;      // activation rows start at column kx0
   const half_t *W; int ldw, kw0, n0;  // weight rows kw0 .. kw0 + 767, columns n0 .. n0 + 63
+  bool packed;                        // W is one slice of souffle_bert_pack_fc2's layout instead: 96 k-steps x 1 KB, contiguous
   int m0;
   int rot;                            // a wave takes the three pairs of its quarter in the order rot, rot + 1, ... (mod 3)
 };
@@ -405,6 +422,13 @@ __device__ __forceinline__ int pair_of(int i, int rot) { const int t = i + rot; 
 
 // The eight wave-wide loads of rows [64 c, 64 c + 64) of K quarter `quarter` (pair c of that quarter).
 __device__ __forceinline__ void issue_w_pair(unsigned char *lds, const GemmItem &g, int quarter, int c, int lane) {
+  if (g.packed) {      // k-steps 24 quarter + 8 c .. + 7 of the slice: 8 KB that are contiguous in memory and in LDS alike
+    const half_t *pb = uniform_ptr(g.W + (size_t)(24 * quarter + 8 * c) * 512);
+    const unsigned pbase = uni(lds_address(lds) + kWOff + (24 * quarter + 8 * c) * 1024);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) dma16<false>(pb, (unsigned)(lane * 16 + u * 1024), pbase + u * 1024);
+    return;
+  }
   const half_t *sb = uniform_ptr(g.W + (size_t)(g.kw0 + 192 * quarter + 64 * c) * g.ldw + g.n0);
   const int rl = lane >> 3;
   const unsigned voff = (unsigned)(rl * g.ldw * 2 + (((lane & 7) ^ (rl & 2)) * 16));
@@ -433,7 +457,7 @@ __device__ __forceinline__ void issue_w_ahead(unsigned char *lds, const GemmItem
 // kGamOff + 768 q (a missing vector is written as ones / zeros).  Fetched by the wave that multiplies the quarter, or
 // (ahead = true) quarter 0 by wave 1.  The bias of the item's 64 columns is fetched by wave 3.
 __device__ __forceinline__ void issue_params(unsigned char *lds, const half_t *gam, const half_t *bet, bool ln_affine,
-                                             const half_t *bias, int n0, bool ahead) {
+                                             const half_t *bias, int n0, int ncols, bool ahead) {
   const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
   if (ln_affine && lane < 24 && !(ahead && w == 0)) {
     for (int q = (ahead && w == 1) ? 0 : w; q <= w; ++q) {
@@ -444,7 +468,7 @@ __device__ __forceinline__ void issue_params(unsigned char *lds, const half_t *g
       else { const half_t c = (half_t)0.0f; *reinterpret_cast<h8 *>(dst + 384 + lane * 16) = h8{c, c, c, c, c, c, c, c}; }
     }
   }
-  if (bias && w == 3 && lane < 8) dma16<false>(uniform_ptr(bias + n0), (unsigned)lane * 16, uni(lds_address(lds) + kBiasOff));
+  if (bias && w == 3 && lane < ncols / 8) dma16<false>(uniform_ptr(bias + n0), (unsigned)lane * 16, uni(lds_address(lds) + kBiasOff));
 }
 // this wave's twelve X blocks, pair after pair
 template <bool SC1>
@@ -475,6 +499,47 @@ __device__ __forceinline__ void issue_stats(unsigned char *lds, const float *st,
   } else {
     if (w < 3) dma16<true>(sb, (unsigned)(w * 1024 + lane * 16), uni(lds_address(lds) + kAuxOff + 4096 + w * 1024));
   }
+}
+
+// Statistics in two levels, for a tile's 32 rows: wave w stages those of rows m0 + 8 w .. + 7 (contiguous in memory) in
+// its own 3 KB, combines them once they are there and writes (mean, rstd) per row into a table that every wave reads
+// behind the next workgroup barrier.
+template <int NS>
+__device__ __forceinline__ void issue_stats_rows(unsigned char *lds, const float *st, int m0) {
+  static_assert(8 * NS * 8 <= kStatBytes, "a wave's staging area");
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
+  const float *sb = uniform_ptr(st + (size_t)(m0 + 8 * w) * NS * 2);
+  const unsigned base = uni(lds_address(lds) + kAuxOff + kStatBytes * w);
+  constexpr int bytes = 8 * NS * 8;
+#pragma unroll
+  for (int q = 0; q * 1024 < bytes; ++q)
+    if (q * 1024 + lane * 16 < bytes) dma16<true>(sb, (unsigned)(q * 1024 + lane * 16), base + q * 1024);
+}
+// (the caller has waited for the staged statistics of this wave)
+template <int NS>
+__device__ __forceinline__ void combine_stats_rows(unsigned char *lds, float eps) {
+  constexpr int LPR = NS == 48 ? 8 : 4, PER = NS / LPR;      // lanes per row, slices per lane (6 or 3)
+  static_assert(NS == 48 || NS == 12, "slice counts in use");
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
+  const int r = (lane / LPR) & 7, part = lane % LPR;
+  const float *sp = reinterpret_cast<const float *>(lds + kAuxOff + kStatBytes * w) + (r * NS + PER * part) * 2;
+  float mi[PER], qi[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) { const f2 v = *reinterpret_cast<const f2 *>(sp + 2 * i); mi[i] = v[0]; qi[i] = v[1]; }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) s += mi[i];
+  const float mean = sum_lanes<LPR>(s) * (1.0f / NS);
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) q += qi[i] + (768.0f / NS) * (mi[i] - mean) * (mi[i] - mean);
+  q = sum_lanes<LPR>(q);
+  if (part == 0 && lane < 8 * LPR)
+    *reinterpret_cast<f2 *>(lds + kRowTabOff + (8 * w + r) * 8) = f2{mean, rsqrtf(q * (1.0f / 768.0f) + eps)};
+}
+__device__ __forceinline__ RowStat table_stat(const unsigned char *lds, int row) {
+  const f2 v = *reinterpret_cast<const f2 *>(lds + kRowTabOff + row * 8);
+  return RowStat{v[0], v[1]};
 }
 
 enum { LN_NONE = 0, LN_PLAIN = 1, LN_AFFINE = 2 };
@@ -512,11 +577,26 @@ __device__ __forceinline__ void read_ops(const unsigned char *lds, int w, int la
 // LN: the X operand is normalised in registers, (x - mean) * rstd [* gamma + beta], in packed fp16 arithmetic: the
 // fp16 part of the mean is subtracted first (a difference of neighbouring values, rounded relative to itself), what
 // rounding the mean to fp16 left over enters through the addend of the multiply-add, so that it does not shift the row.
-template <int LN>
-__device__ __forceinline__ void mfma_quarter(const unsigned char *lds, f4 (&acc)[2][4], float eps, int rot) {
+// TAB: the statistics are those of z2, staged per wave (issue_stats_rows<kNS2>) and combined through the row table;
+// otherwise those of z1, one copy of the tile's per wave (issue_stats<4>).
+template <int LN, bool TAB>
+__device__ __forceinline__ void mfma_quarter(unsigned char *lds, f4 (&acc)[2][4], float eps, int rot) {
   const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6, l16 = lane & 15, gq = lane >> 4;
   h8 nmh[2], off[2], rs[2];     // -mean (its fp16 part), -(mean - that part) * rstd, rstd
-  if constexpr (LN != LN_NONE) {
+  if constexpr (LN != LN_NONE && TAB) {
+    wait_vmcnt<12>();                    // the staged statistics are older than the twelve X blocks
+    combine_stats_rows<kNS2>(lds, eps);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const RowStat st = table_stat(lds, 16 * i + l16);
+      const float mu = st.mean, r = st.rstd;
+      const half_t a = (half_t)mu, c = (half_t)fminf(r, 65504.0f), b2 = (half_t)(((float)a - mu) * (float)c), na = -a;
+      nmh[i] = h8{na, na, na, na, na, na, na, na};
+      off[i] = h8{b2, b2, b2, b2, b2, b2, b2, b2};
+      rs[i] = h8{c, c, c, c, c, c, c, c};
+    }
+  } else if constexpr (LN != LN_NONE) {
     // Lane L combines row L / 2: slices 6 (L % 2) .. + 5 from this wave's copy of the statistics, then its partner's.
     wait_vmcnt<12>();                    // the three statistics loads are older than the twelve X blocks
     const int row = lane >> 1, half = lane & 1;
@@ -743,12 +823,15 @@ __device__ __forceinline__ void attn_item_split(unsigned char *lds, const AttnAr
 // launch every address is written by one item of one phase and read only afterwards.
 struct Args {
   int B, S, M, act, num_layers;
+  int packed;                          // every layer has w_fc2p: FC2 runs in its whole-K form
   float scale, eps;
   const half_t *x, *mask;
   half_t *y;
   half_t *qkv, *ctx, *z1, *h, *z2;     // [3][B][12][S][64], [M][768], [M][768] (pre-LN1 sum), [M][3072], [M][768] (pre-LN2 sum)
-  float *st1, *st2, *part;             // row statistics of z1 / z2 [M][12][2], FC2 partial sums [4][M][768]
+                                       // (whole-K FC2: h in operand order, h_operand_offset)
+  float *st1, *st2, *part;             // row statistics of z1 [M][12][2] and z2 [M][48][2], FC2 partial sums [4][M][768] (split-K form)
   half_t *probs, *ln1_out;             // optional per-stage outputs (single layer only)
+  half_t *fc1_out;                     // ... the row-major copy of h when h itself is kept in operand order (whole-K FC2)
   size_t layer_stride;
   unsigned *ctl, *flags;
   unsigned long long *trace;
@@ -820,12 +903,19 @@ __device__ __forceinline__ Job make_job_t(const Args &a, int l, const It &d) {
     j.ln = (w.ln1_g || w.ln1_b) ? LN_AFFINE : LN_PLAIN;
     j.bias = w.b_fc1;
     j.out = cur.h;
-  } else {   // PH_FC2: slice = n-slice * 4 + K quarter
+  } else {   // PH_FC2: slice = 16 columns over the whole K, or (split-K form) n-slice * 4 + K quarter
     static_assert(PH == PH_FC2, "a GEMM phase");
-    const int ks = d.b & 3, ns = d.b >> 2;
-    j.which = ks;
-    j.g.W = w.w_fc2; j.g.ldw = H; j.g.kw0 = ks * 768; j.g.n0 = ns * 64;
-    j.g.X = cur.h; j.g.ldx = F; j.g.kx0 = ks * 768;
+    if (a.packed) {
+      j.which = 0;
+      j.g.packed = true;
+      j.g.W = w.w_fc2p + (size_t)d.b * (96 * 512); j.g.ldw = 0; j.g.kw0 = 0; j.g.n0 = d.b * 16;
+      j.g.X = cur.h; j.g.ldx = F; j.g.kx0 = 0;
+    } else {
+      const int ks = d.b & 3, ns = d.b >> 2;
+      j.which = ks;
+      j.g.W = w.w_fc2; j.g.ldw = H; j.g.kw0 = ks * 768; j.g.n0 = ns * 64;
+      j.g.X = cur.h; j.g.ldx = F; j.g.kx0 = ks * 768;
+    }
     j.aux = cur.part;
     // what the workgroup that completes the tile adds: bias, residual LN1(z1)
     j.bias = w.b_fc2; j.res = cur.z1; j.rstats = cur.st1; j.rgam = w.ln1_g; j.rbet = w.ln1_b;
@@ -848,9 +938,10 @@ __device__ __forceinline__ void pin(Job &j) {
 // The loads of an item that depend on no other workgroup: weight slice, LayerNorm vectors, bias.
 __device__ __forceinline__ void issue_weights(unsigned char *lds, const Job &j, bool ahead) {
   if (ahead) issue_w_ahead(lds, j.g); else issue_w(lds, j.g);
-  issue_params(lds, j.gam, j.bet, j.ln == LN_AFFINE, j.bias, j.g.n0, ahead);
+  const int ncols = j.g.packed ? 16 : 64;
+  issue_params(lds, j.gam, j.bet, j.ln == LN_AFFINE, j.bias, j.g.n0, ncols, ahead);
   const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
-  if (w == 2 && lane < 8) {      // the residual's LayerNorm vectors for the item's 64 columns (OUT)
+  if (w == 2 && lane < ncols / 8) {      // the residual's LayerNorm vectors for the item's columns (OUT, FC2)
     if (j.rgam) dma16<false>(uniform_ptr(j.rgam + j.g.n0), (unsigned)lane * 16, uni(lds_address(lds) + kGamOff));
     if (j.rbet) dma16<false>(uniform_ptr(j.rbet + j.g.n0), (unsigned)lane * 16, uni(lds_address(lds) + kGamOff + 128));
   }
@@ -858,19 +949,120 @@ __device__ __forceinline__ void issue_weights(unsigned char *lds, const Job &j, 
 
 __device__ __forceinline__ f4 widen(h4 v) { return f4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]}; }
 
+// h in operand order (whole-K FC2 only): [M / 16][96 k-steps][64 lanes][8 halves], lane L of (16-row tile, k-step t)
+// holding h[16 tile + L % 16][32 t + 8 (L / 16) + 0..7], i.e. the B operand of the 16x16x32 MFMA as one 16-byte load per
+// lane and 1 KB contiguous per wave.  (Row-major, a lane's 16 bytes are contiguous too, but a wave-wide load then asks
+// for 16 rows x 64 bytes, half lines, and a CU took its 196 KB of a tile in over 4.6 us that way.)
+// Offset in halves of the 8 values h[m][n .. n + 7], n a multiple of 8.
+__device__ __forceinline__ int h_operand_offset(int m, int n) {
+  return ((((m >> 4) * 96 + (n >> 5)) * 64) + (m & 15) + 16 * ((n & 31) >> 3)) * 8;
+}
+
+// FC2 in its whole-K form: 32 rows x 16 columns over K = 3072, the weights one contiguous 96 KB slice of the packed
+// copy (k-step t at t KB, lane L's A operand at + 16 L: read back with plain 16-byte LDS reads).  Wave w multiplies
+// the K quarter [768 w, 768 w + 768): its 48 KB of the activation rows go straight into registers (FC1 writes h in
+// operand order for this form, and 196 KB per tile are more than the LDS holds), all requested at once, and the
+// MFMAs run behind the data as it arrives.  The four partial tiles are summed through LDS, and the
+// workgroup that multiplied a tile finishes its rows: + bias + LN1(z1), rounded, with the statistics of the 16
+// columns.  No partial sum leaves the CU.
+__device__ __forceinline__ void run_fc2_whole_k(unsigned char *lds, const Args &a, int l, const It &d, const Job &j, bool w_ready, const Sync *sy) {
+  const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6, l16 = lane & 15, gq = lane >> 4;
+  if (!w_ready) issue_weights(lds, j, false);
+  // the residual: this thread's four columns of z1 (threads 0..127: row tid / 4), and the rows' statistics
+  const int row = (tid >> 2) & 31, c4 = (tid & 3) * 4;
+  const u2 zres = ld8<true>(j.res, ((j.g.m0 + row) * H + j.g.n0 + c4) * 2);
+  issue_stats_rows<kNS1>(lds, j.rstats, j.g.m0);
+  // this wave's K quarter of the 32 rows: segment (8 k-steps = 512 bytes of a row) after segment, in the order rot, rot + 1, ...
+  u4 x[24][2];
+  {
+    const auto rsrc = make_rsrc(j.g.X + (size_t)j.g.m0 * F);      // (h in operand order: the tile's two 16-row tiles, 96 KB each)
+    const int voff0 = 24 * 1024 * w + 16 * lane, voff1 = voff0 + 96 * 1024;
+    static_for<0, 3>([&](auto sgc) {
+      constexpr int sg = decltype(sgc)::value;
+      const int soff = (int)uni((unsigned)pair_of(sg, j.g.rot) * 8192u);
+      static_for<0, 8>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        x[8 * sg + u][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff0, soff + u * 1024, kAuxSc1);
+        x[8 * sg + u][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff1, soff + u * 1024, kAuxSc1);
+      });
+    });
+  }
+  wait_vmcnt<48>();                                   // everything older than the 48 activation loads: residual, statistics, a weight slice requested here
+  if (sy && sy->trace) stamp_mark(*sy, l * PH_SLOTS + PH_FC2, 0);
+  combine_stats_rows<kNS1>(lds, a.eps);               // (read behind the barrier in front of the epilogue)
+  f4 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) { acc[i][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[i][1] = f4{0.f, 0.f, 0.f, 0.f}; }
+  {
+    const unsigned char *wl = lds + kWOff + 24 * 1024 * w + 16 * lane;
+    unsigned seg[3];
+#pragma unroll
+    for (int sg = 0; sg < 3; ++sg) seg[sg] = uni((unsigned)pair_of(sg, j.g.rot) * 8192u);
+    h8 wop[4];
+#pragma unroll
+    for (int t = 0; t < 3; ++t) wop[t] = as_h8(lds_load16(wl + seg[0] + t * 1024));
+    static_for<0, 24>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+      // (the scheduler otherwise sinks every operand read to just in front of its MFMA, one LDS latency per k-step)
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (t + 3 < 24) wop[(t + 3) & 3] = as_h8(lds_load16(wl + seg[(t + 3) / 8] + ((t + 3) & 7) * 1024));
+      acc[0][t & 1] = mfma_16x16x32(wop[t & 3], as_h8(x[t][0]), acc[0][t & 1]);
+      acc[1][t & 1] = mfma_16x16x32(wop[t & 3], as_h8(x[t][1]), acc[1][t & 1]);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (sy) stamp_mark(*sy, l * PH_SLOTS + PH_FC2, 1);
+  // acc[i][.][v]: row 16 i + l16, column 4 gq + v.  Partial tiles [32][20] floats, one per wave, in the (idle) X parts.
+  constexpr int ld = 20;
+  float *mine = reinterpret_cast<float *>(lds + kXPart * w);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) *reinterpret_cast<f4 *>(mine + (16 * i + l16) * ld + 4 * gq) = acc[i][0] + acc[i][1];
+  __syncthreads();
+  if (tid < 128) {
+    const float *src = reinterpret_cast<const float *>(lds) + row * ld + c4;
+    f4 sum = *reinterpret_cast<const f4 *>(src);
+#pragma unroll
+    for (int k = 1; k < 4; ++k) sum += *reinterpret_cast<const f4 *>(src + k * (kXPart / 4));
+    if (j.bias) sum += widen(*reinterpret_cast<const h4 *>(lds + kBiasOff + c4 * 2));
+    const RowStat rs = table_stat(lds, row);
+    f4 r = (widen(as_h4(zres)) - rs.mean) * rs.rstd;
+    if (j.rgam) r *= widen(*reinterpret_cast<const h4 *>(lds + kGamOff + c4 * 2));
+    if (j.rbet) r += widen(*reinterpret_cast<const h4 *>(lds + kGamOff + 128 + c4 * 2));
+    const int m = j.g.m0 + row;
+    if (a.ln1_out) st8<true>(a.ln1_out, (m * H + j.g.n0 + c4) * 2, pack_h4(r));      // (LN1(z1) itself, for single-layer callers)
+    sum += r;
+    const u2 packed = pack_h4(sum);
+    st8<true>(j.out, (m * H + j.g.n0 + c4) * 2, packed);
+    const h4 r4 = as_h4(packed);
+    const float v[4] = {(float)r4[0], (float)r4[1], (float)r4[2], (float)r4[3]};
+    put_stat<4, 4, kNS2>(j.stat_out, m, d.b, v, tid & 3);
+  }
+}
+
 // One GEMM item from operand fetch to the stores of its epilogue.
 template <int PH>
 __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &a, int l, const It &d, const Job &j, bool w_ready, const Sync *sy = nullptr) {
   constexpr int ph = PH;
+  if constexpr (ph == PH_FC2) {
+    if (a.packed) { run_fc2_whole_k(lds, a, l, d, j, w_ready, sy); return; }
+  }
   if (!w_ready) issue_weights(lds, j, false);
   // what the item reads of other workgroups' results, statistics first (they are needed first)
-  if (j.ln != LN_NONE) issue_stats<4>(lds, j.stats, j.g.m0);
-  if constexpr (ph == PH_OUT || ph == PH_FC2) {
+  if (j.ln != LN_NONE) {
+    if constexpr (ph == PH_QKV) issue_stats_rows<kNS2>(lds, j.stats, j.g.m0); else issue_stats<4>(lds, j.stats, j.g.m0);
+  }
+  [[maybe_unused]] u4 zres = {0u, 0u, 0u, 0u};      // OUT: this thread's eight columns of the residual row tid / 8
+  if constexpr (ph == PH_OUT) {
+    const int tid = opaque_thread_id();
+    zres = ld16<true>(j.res, ((j.g.m0 + (tid >> 3)) * H + j.g.n0 + (tid & 7) * 8) * 2);
+    if (j.rstats) issue_stats_rows<kNS2>(lds, j.rstats, j.g.m0);
+  }
+  if constexpr (ph == PH_FC2) {
     const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6;
     // residual patch: rows m0 .. m0 + 31, columns n0 .. n0 + 63 -> [32][128 B] at kAuxOff
     dma16<true>(uniform_ptr(j.res + (size_t)(j.g.m0 + 8 * w) * H + j.g.n0), (unsigned)((lane >> 3) * H * 2 + (lane & 7) * 16),
                 uni(lds_address(lds) + kAuxOff + w * 1024));
-    if (j.rstats) issue_stats<1>(lds, j.rstats, j.g.m0);
+    issue_stats<1>(lds, j.rstats, j.g.m0);
   }
 #ifdef SOUFFLE_STAGE_MARKS      // development build: serialises the weight slice and the X tile to time them apart
   if (sy) stamp_mark(*sy, l * PH_SLOTS + ph, 4);
@@ -884,9 +1076,13 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
 #ifdef SOUFFLE_STAGE_MARKS
   if (sy) { wait_vmcnt<0>(); stamp_mark(*sy, l * PH_SLOTS + ph, 7); }
 #endif
-  if (j.ln == LN_NONE) mfma_quarter<LN_NONE>(lds, acc, a.eps, j.g.rot);
-  else if (j.ln == LN_PLAIN) mfma_quarter<LN_PLAIN>(lds, acc, a.eps, j.g.rot);
-  else mfma_quarter<LN_AFFINE>(lds, acc, a.eps, j.g.rot);
+  if constexpr (ph == PH_OUT) {
+    if (j.rstats) { wait_vmcnt<12>(); combine_stats_rows<kNS2>(lds, a.eps); }      // (read behind the barrier of reduce_tile)
+  }
+  constexpr bool tab = ph == PH_QKV;
+  if (j.ln == LN_NONE) mfma_quarter<LN_NONE, tab>(lds, acc, a.eps, j.g.rot);
+  else if (j.ln == LN_PLAIN) mfma_quarter<LN_PLAIN, tab>(lds, acc, a.eps, j.g.rot);
+  else mfma_quarter<LN_AFFINE, tab>(lds, acc, a.eps, j.g.rot);
   if (sy) stamp_mark(*sy, l * PH_SLOTS + ph, 1);
   const half_t *bias_lds = j.bias ? reinterpret_cast<const half_t *>(lds + kBiasOff) : nullptr;
   auto add_bias = [&](int col0, f4 &lo, f4 &hi) {
@@ -896,31 +1092,32 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       hi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]};
     }
   };
-  // A row of a pre-LayerNorm sum (8 columns per thread): + bias + the residual (normalised from its statistics when it
-  // is itself a pre-LayerNorm sum), rounded to fp16, written with the statistics of the rounded values.
-  // The residual of a row (8 columns per thread), normalised from its statistics when it is itself a pre-LayerNorm sum.
   struct Resid { f4 lo, hi; };
-  auto residual = [&](int row, int col0, half_t *res_out) {
+  // gamma and beta of the LayerNorm that produces the residual, for 8 columns
+  auto residual_affine = [&](int col0, f4 &rlo, f4 &rhi) {
+    if (j.rgam) { const h8 gg = *reinterpret_cast<const h8 *>(lds + kGamOff + col0 * 2); rlo *= f4{(float)gg[0], (float)gg[1], (float)gg[2], (float)gg[3]}; rhi *= f4{(float)gg[4], (float)gg[5], (float)gg[6], (float)gg[7]}; }
+    if (j.rbet) { const h8 bb = *reinterpret_cast<const h8 *>(lds + kGamOff + 128 + col0 * 2); rlo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]}; rhi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]}; }
+  };
+  // Split-K FC2: the residual LN1(z1) of a row (8 columns per thread), normalised from the statistics of z1 in LDS.
+  [[maybe_unused]] auto residual_z1 = [&](int row, int col0, half_t *res_out) {
     const h8 rv = *reinterpret_cast<const h8 *>(lds + kAuxOff + row * 128 + col0 * 2);
     f4 rlo = f4{(float)rv[0], (float)rv[1], (float)rv[2], (float)rv[3]}, rhi = f4{(float)rv[4], (float)rv[5], (float)rv[6], (float)rv[7]};
-    if (j.rstats) {
-      const float *sp = reinterpret_cast<const float *>(lds + kAuxOff + 4096) + row * 24;
-      float mean = 0.f;
+    const float *sp = reinterpret_cast<const float *>(lds + kAuxOff + 4096) + row * 24;
+    float mean = 0.f;
 #pragma unroll
-      for (int i = 0; i < 12; ++i) mean += sp[2 * i];
-      mean *= (1.0f / 12.0f);
-      float q = 0.f;
+    for (int i = 0; i < 12; ++i) mean += sp[2 * i];
+    mean *= (1.0f / 12.0f);
+    float q = 0.f;
 #pragma unroll
-      for (int i = 0; i < 12; ++i) q += sp[2 * i + 1] + 64.0f * (sp[2 * i] - mean) * (sp[2 * i] - mean);
-      const float rstd = rsqrtf(q * (1.0f / 768.0f) + a.eps);
-      rlo = (rlo - mean) * rstd; rhi = (rhi - mean) * rstd;
-      if (j.rgam) { const h8 gg = *reinterpret_cast<const h8 *>(lds + kGamOff + col0 * 2); rlo *= f4{(float)gg[0], (float)gg[1], (float)gg[2], (float)gg[3]}; rhi *= f4{(float)gg[4], (float)gg[5], (float)gg[6], (float)gg[7]}; }
-      if (j.rbet) { const h8 bb = *reinterpret_cast<const h8 *>(lds + kGamOff + 128 + col0 * 2); rlo += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]}; rhi += f4{(float)bb[4], (float)bb[5], (float)bb[6], (float)bb[7]}; }
-      if (res_out) st16<true>(res_out, ((j.g.m0 + row) * H + j.g.n0 + col0) * 2, pack_h8(rlo, rhi));      // (the normalised residual itself, on request)
-    }
+    for (int i = 0; i < 12; ++i) q += sp[2 * i + 1] + 64.0f * (sp[2 * i] - mean) * (sp[2 * i] - mean);
+    const float rstd = rsqrtf(q * (1.0f / 768.0f) + a.eps);
+    rlo = (rlo - mean) * rstd; rhi = (rhi - mean) * rstd;
+    residual_affine(col0, rlo, rhi);
+    if (res_out) st16<true>(res_out, ((j.g.m0 + row) * H + j.g.n0 + col0) * 2, pack_h8(rlo, rhi));      // (the normalised residual itself, on request)
     return Resid{rlo, rhi};
   };
-  // A row of a pre-LayerNorm sum: + bias + residual, rounded to fp16, written with the statistics of the rounded values.
+  // A row of a pre-LayerNorm sum (8 columns per thread): + bias + residual, rounded to fp16, written with the
+  // statistics of the rounded values: of its 64-column slice (z1) or of four 16-column slices (z2).
   auto finish_row = [&](int row, int col0, f4 lo, f4 hi, const Resid &r, int slice) {
     add_bias(col0, lo, hi);
     lo += r.lo; hi += r.hi;
@@ -931,7 +1128,9 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
     float v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = (float)r8[i];
-    put_stat<8, 8>(j.stat_out, m, slice, v, opaque_thread_id() & 7);
+    const int t8 = opaque_thread_id() & 7;
+    if constexpr (ph == PH_OUT) put_stat<8, 8, kNS1>(j.stat_out, m, slice, v, t8);
+    else put_stat<8, 2, kNS2>(j.stat_out, m, 4 * slice + (t8 >> 1), v, t8 & 1);
   };
   if constexpr (ph == PH_QKV) {
     const int which = j.which, head = j.head;
@@ -941,7 +1140,16 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       st16<true>(j.out, ((((which * a.B + b) * NH + head) * a.S + s) * HD + col0) * 2, pack_h8(lo, hi));
     });
   } else if constexpr (ph == PH_OUT) {
-    reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) { finish_row(row, col0, lo, hi, residual(row, col0, nullptr), d.b); });
+    reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
+      const h8 rv = as_h8(zres);
+      f4 rlo = f4{(float)rv[0], (float)rv[1], (float)rv[2], (float)rv[3]}, rhi = f4{(float)rv[4], (float)rv[5], (float)rv[6], (float)rv[7]};
+      if (j.rstats) {      // the residual is LN2 of the previous layer's sum
+        const RowStat rs = table_stat(lds, row);
+        rlo = (rlo - rs.mean) * rs.rstd; rhi = (rhi - rs.mean) * rs.rstd;
+        residual_affine(col0, rlo, rhi);
+      }
+      finish_row(row, col0, lo, hi, Resid{rlo, rhi}, d.b);
+    });
   } else if constexpr (ph == PH_FC1) {
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
       add_bias(col0, lo, hi);
@@ -952,12 +1160,16 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
 #pragma unroll
         for (int i = 0; i < 4; ++i) { lo[i] = gelu_tanh(lo[i]); hi[i] = gelu_tanh(hi[i]); }
       }
-      st16<true>(j.out, ((j.g.m0 + row) * F + j.g.n0 + col0) * 2, pack_h8(lo, hi));
+      const u4 hv = pack_h8(lo, hi);
+      if (a.packed) {
+        st16<true>(j.out, h_operand_offset(j.g.m0 + row, j.g.n0 + col0) * 2, hv);
+        if (a.fc1_out) st16<true>(a.fc1_out, ((j.g.m0 + row) * F + j.g.n0 + col0) * 2, hv);
+      } else st16<true>(j.out, ((j.g.m0 + row) * F + j.g.n0 + col0) * 2, hv);
     });
   } else {
-    // FC2: the partial sum of this K quarter goes to memory; the four workgroups of a tile draw a ticket each once
-    // their partial sums are acknowledged, and the one that draws the last ticket adds the other three to its own
-    // (in the order of the quarters, whoever is last), finishes the rows (bias, residual LN1(z1), statistics) and
+    // FC2, split-K form: the partial sum of this K quarter goes to memory; the four workgroups of a tile draw a ticket
+    // each once their partial sums are acknowledged, and the one that draws the last ticket adds the other three to its
+    // own (in the order of the quarters, whoever is last), finishes the rows (bias, residual LN1(z1), statistics) and
     // marks the tile complete for the workgroups of the next layer.
     const int ks = j.which, ns = d.b >> 2;
     reduce_tile(lds, acc, [&](int row, int col0, f4 lo, f4 hi) {
@@ -967,12 +1179,12 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       st16<true>(j.aux, off + 16, __builtin_bit_cast(u4, hi));
       wait_all_memory();
       __syncthreads();
-      unsigned *ticket_lds = reinterpret_cast<unsigned *>(lds + kBiasOff + 256);
+      unsigned *ticket_lds = reinterpret_cast<unsigned *>(lds + kTicketOff);
       unsigned ticket = 0;
       if (tid == 0) ticket = __hip_atomic_fetch_add(a.flags + kTileCntWord + (l * kTileWords + d.a * 12 + ns), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       // (while the ticket travels: what the workgroup that turns out to be last adds to the sum.  ln1_out, asked for by
       // single-layer callers only, is written by whoever runs this, with the same values.)
-      const Resid res = residual(row, col0, a.ln1_out);
+      const Resid res = residual_z1(row, col0, a.ln1_out);
       if (tid == 0) *ticket_lds = ticket;
       __syncthreads();
       const bool last = (*ticket_lds & 3u) == 3u;
@@ -1066,7 +1278,7 @@ template <int NKT, bool MULTI>
 __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int b = blockIdx.x, tid = threadIdx.x;
-  const Shape sh{args.B, args.S, args.M, args.M / 32, (int)gridDim.x};
+  const Shape sh{args.B, args.S, args.M, args.M / 32, (int)gridDim.x, args.packed};
   Sync sy;
   sync_begin(sy, args.flags, args.ctl + kCtlErrWord, args.trace, args.trace_cap);
   const int L = args.num_layers;
@@ -1150,8 +1362,10 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
     const bool ready = pf == l * 8 + ph;
     pf = -1;
     if constexpr (ph == PH_QKV) {
-      if (l > 0) await_tiles(sy, f0.d.a, phase_seq(sy, l - 1, PH_RED), l * PH_SLOTS + ph);
-      else if (ready) {                                       // (no wait in front of the very first phase)
+      if (l > 0) {
+        if (sh.packed) await(sy, wm(PH_QKV), phase_seq(sy, l - 1, PH_FC2), l * PH_SLOTS + ph);
+        else await_tiles(sy, f0.d.a, phase_seq(sy, l - 1, PH_RED), l * PH_SLOTS + ph);
+      } else if (ready) {                                       // (no wait in front of the very first phase)
         if (tid >= 64) wait_vmcnt<0>();
         __syncthreads();
       }
@@ -1160,7 +1374,7 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
     if constexpr (MULTI) for (int i = 1; i < f0.count; ++i) {      // further m-tiles of the same weight slice, which stays where it is
       const It d{f0.d.a + i * f0.step, f0.d.b};
       __syncthreads();                                        // the partial tiles of the previous item have been read
-      if (ph == PH_QKV && l > 0) await_tiles(sy, d.a, phase_seq(sy, l - 1, PH_RED), sy.trace_cap);      // (its own m-tile)
+      if (ph == PH_QKV && l > 0 && !sh.packed) await_tiles(sy, d.a, phase_seq(sy, l - 1, PH_RED), sy.trace_cap);      // (its own m-tile)
       run_gemm_item_t<ph>(lds, args, l, d, make_job_t<ph>(args, l, d), true, &sy);
     }
     stamp_mark(sy, l * PH_SLOTS + ph, 2);
@@ -1175,11 +1389,12 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
   if (mine_bits != 0) {
     unsigned needs = 0;
     for (int ph = PH_ATT; ph <= PH_FC2; ++ph) needs |= (wait_needs(sh, ph, b, tid) ? 1u : 0u) << ph;
+    if (sh.packed) needs |= (wait_needs(sh, PH_QKV, b, tid) ? 1u : 0u) << PH_QKV | (wait_needs(sh, PH_FIN, b, tid) ? 1u : 0u) << PH_FIN;
     lds[tid] = (unsigned char)needs;
     __syncthreads();
     if (tid < 64) {
       const unsigned four = *reinterpret_cast<const unsigned *>(lds + 4 * tid);
-      for (int ph = PH_ATT; ph <= PH_FC2; ++ph)
+      for (int ph = PH_QKV; ph <= PH_FIN; ++ph)
         for (int t = 0; t < 4; ++t) wm_all |= ((four >> (8 * t + ph)) & 1u) << (4 * ph + t);
     }
     __syncthreads();
@@ -1202,11 +1417,13 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
     gemm_phase(l, std::integral_constant<int, PH_FC1>{});
     gemm_phase(l, std::integral_constant<int, PH_FC2>{});
   }
-  if (mine(PH_FIN))
+  if (mine(PH_FIN)) {
+    if (sh.packed) await(sy, wm(PH_FIN), phase_seq(sy, L - 1, PH_FC2), (L - 1) * PH_SLOTS + PH_FIN);
     for_items(sh, PH_FIN, b, [&](const It &d, bool first) {
-      await_tiles(sy, d.a, phase_seq(sy, L - 1, PH_RED), first ? (L - 1) * PH_SLOTS + PH_FIN : sy.trace_cap);
+      if (!sh.packed) await_tiles(sy, d.a, phase_seq(sy, L - 1, PH_RED), first ? (L - 1) * PH_SLOTS + PH_FIN : sy.trace_cap);
       run_fin_item(args, d);
     });
+  }
   sync_end(sy, L);
 }
 
@@ -1216,7 +1433,7 @@ template <int NKT>
 __global__ void __launch_bounds__(256) k_small_phase(Args args, int l, int ph) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int b = blockIdx.x;
-  const Shape sh{args.B, args.S, args.M, args.M / 32, (int)gridDim.x};
+  const Shape sh{args.B, args.S, args.M, args.M / 32, (int)gridDim.x, args.packed};
   if (ph == PH_ATT) {
     const AttnArgs aa = attn_args(args, l);
     for_items(sh, ph, b, [&](const It &d, bool) { attn_item_split<NKT>(lds, aa, d.b, d.a); });

@@ -23,7 +23,7 @@ class BertCfg(C.Structure):
 
 
 BERT_W_FIELDS = ["w_qkv", "b_qkv", "w_o", "b_o", "ln1_g", "ln1_b", "w_fc1", "b_fc1", "w_fc2", "b_fc2",
-                 "ln2_g", "ln2_b"]
+                 "ln2_g", "ln2_b", "w_fc2_packed"]
 
 
 class BertLayerW(C.Structure):
@@ -95,7 +95,9 @@ SIGNATURES = {
     "souffle_bert_encoder_fused_static": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
                                                     C.c_void_p, C.c_void_p]),
     "souffle_bert_polled_copies": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p]),
-    "souffle_bert_handover_plan": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "souffle_bert_handover_plan": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "souffle_bert_fc2_packed_bytes": (C.c_size_t, []),
+    "souffle_bert_pack_fc2": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "souffle_bert_embed": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
                                      C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                      C.c_void_p]),

@@ -68,7 +68,13 @@ int main() {
   std::vector<_Float16> got((size_t)M * H);
   double worst_max = 0, worst_mean = 0;
   int bad = 0;
-  for (int fused = 1; fused >= 0; --fused) {
+  // four runs: fused and per-op, first with the [K][N] FC2 matrix alone, then with its packed copy as well
+  void *d2p = nullptr;
+  HIP_OK(hipMalloc(&d2p, souffle_bert_fc2_packed_bytes()));
+  if (souffle_bert_pack_fc2(d2, d2p, st)) { fprintf(stderr, "pack: %s\n", souffle_last_error()); return 2; }
+  for (int run = 0; run < 4; ++run) {
+    const int fused = (run & 1) == 0;
+    w.w_fc2_packed = run >= 2 ? d2p : nullptr;
     HIP_OK(hipMemsetAsync(dy, 0xff, (size_t)M * H * 2, st));
     const int rc = fused ? souffle_bert_layer_fused(&cfg, &w, dx, nullptr, dy, nullptr, ws, ws_bytes, st)
                          : souffle_bert_layer_unfused(&cfg, &w, dx, nullptr, dy, nullptr, ws, ws_bytes, st);
@@ -90,7 +96,7 @@ int main() {
   }
   printf("{\"caller\": \"plain C++ over the C ABI\", \"version\": \"%s\", \"max_abs\": %.6f, \"mean_abs\": %.6f, \"ok\": %s}\n",
          souffle_version(), worst_max, worst_mean, bad ? "false" : "true");
-  for (void *p : {dx, dqkv, d_o, d1, d2, db1, dy, ws}) (void)hipFree(p);
+  for (void *p : {dx, dqkv, d_o, d1, d2, d2p, db1, dy, ws}) (void)hipFree(p);
   (void)hipStreamDestroy(st);
   return bad;
 }

@@ -24,28 +24,31 @@ def run_layer(w, x, B, S, opt_level, **kw):
     return outs
 
 
+@pytest.mark.parametrize("pack", [True, False])
 @pytest.mark.parametrize("opt_level", [4, 1])
 @pytest.mark.parametrize("B,S", [(1, 128), (1, 384), (1, 64), (2, 256)])
-def test_layer_config0_all_stages(B, S, opt_level):
-    """Benchmark config 0 (zero biases, gamma 1, beta 0, tanh-GELU, scale 1/8, eps 1e-12, no mask)."""
-    announce("bert layer cfg0 B=%d S=%d opt=%d" % (B, S, opt_level))
+def test_layer_config0_all_stages(B, S, opt_level, pack):
+    """Benchmark config 0 (zero biases, gamma 1, beta 0, tanh-GELU, scale 1/8, eps 1e-12, no mask), with the packed
+    copy of the FC2 weights (whole-K FC2 items) and with the [K][N] matrix alone (split-K FC2)."""
+    announce("bert layer cfg0 B=%d S=%d opt=%d pack=%d" % (B, S, opt_level, pack))
     w, x = synth.bert_layer_weights(0, 0), synth.bert_input(0, B, S)
     ref = oracle.bert_layer(x, w, B, S, dump=True)
-    got = run_layer(w, x, B, S, opt_level)
+    got = run_layer(w, x, B, S, opt_level, pack=pack)
     for n, g, r in zip(NAMES, got, ref):
         assert_close(n, g, r)
 
 
+@pytest.mark.parametrize("pack", [True, False])
 @pytest.mark.parametrize("opt_level", [3, 2])
-def test_layer_bias_affine_mask(opt_level):
-    announce("bert layer bias+affine+mask opt=%d" % opt_level)
+def test_layer_bias_affine_mask(opt_level, pack):
+    announce("bert layer bias+affine+mask opt=%d pack=%d" % (opt_level, pack))
     B, S = 2, 128
     w, x = synth.bert_layer_weights(0, 1, with_bias=True), synth.bert_input(7, B, S)
     keep = synth.uniform01(synth.seed_of(0, 99), B * S * S).reshape(B, S, S) < 0.85
     keep[:, :, 0] = True
     mask = np.where(keep, 0.0, -10000.0).astype(np.float16)
     ref = oracle.bert_layer(x, w, B, S, mask=mask, dump=True)
-    got = run_layer(w, x, B, S, opt_level, mask=dev(mask))
+    got = run_layer(w, x, B, S, opt_level, mask=dev(mask), pack=pack)
     for n, g, r in zip(NAMES, got, ref):
         assert_close(n, g, r)
 
@@ -77,32 +80,38 @@ def test_fast_path_equals_dump_path_and_is_deterministic():
     announce("bert layer dump=False determinism")
     B, S = 1, 128
     w, x = synth.bert_layer_weights(0, 0), synth.bert_input(0, B, S)
-    full = run_layer(w, x, B, S, 4)[-1]
-    a = run_layer(w, x, B, S, 4, dump=False)
-    b = run_layer(w, x, B, S, 4, dump=False)
-    c = run_layer(w, x, B, S, 1, dump=False)
-    assert torch.equal(a, b) and torch.equal(a, full)
-    assert torch.equal(a, c), "fused and per-op paths run the same arithmetic"
+    for pack in (True, False):
+        full = run_layer(w, x, B, S, 4, pack=pack)[-1]
+        a = run_layer(w, x, B, S, 4, dump=False, pack=pack)
+        b = run_layer(w, x, B, S, 4, dump=False, pack=pack)
+        c = run_layer(w, x, B, S, 1, dump=False, pack=pack)
+        assert torch.equal(a, b) and torch.equal(a, full)
+        assert torch.equal(a, c), "fused and per-op paths run the same arithmetic"
 
 
-@pytest.mark.parametrize("B,S,layers", [(1, 128, 12), (1, 384, 12), (32, 128, 12), (9, 128, 2), (8, 128, 2), (3, 384, 2)])
-def test_encoder_matches_oracle(B, S, layers):
-    announce("bert encoder B=%d S=%d L=%d" % (B, S, layers))
+# (13 x 128 and 5 x 384: 1664 and 1920 rows, no multiple of 256: the many-rows kernel on its 128 x 128 tiles)
+@pytest.mark.parametrize("B,S,layers,pack", [(1, 128, 12, True), (1, 384, 12, True), (32, 128, 12, True), (9, 128, 2, True), (8, 128, 2, True),
+                                             (3, 384, 2, True), (1, 128, 12, False), (1, 384, 3, False), (9, 128, 2, False), (2, 512, 2, True),
+                                             (13, 128, 2, True), (5, 384, 2, True)])
+def test_encoder_matches_oracle(B, S, layers, pack):
+    announce("bert encoder B=%d S=%d L=%d pack=%d" % (B, S, layers, pack))
     import bert_binding
     ws = [synth.bert_layer_weights(2, l) for l in range(layers)]
     x = synth.bert_input(2, B, S)
     ref = oracle.bert_encoder(x, ws, B, S)
-    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S)
+    enc = bert_binding.Encoder([dev_weights(w) for w in ws], B, S, pack=pack)
     y_f = enc(dev(x), fused=True)
     y_u = enc(dev(x), fused=False)
     torch.cuda.synchronize()
+    assert enc.ws.status() == 0
     # errors of successive layers do not compound past the tolerance because each layer ends in a LayerNorm
     assert_close("encoder fused", y_f, ref)
     assert_close("encoder unfused", y_u, ref)
     assert torch.equal(y_f, y_u)
 
 
-@pytest.mark.parametrize("B,S,layers", [(32, 128, 5), (16, 128, 4), (64, 128, 3), (8, 384, 3), (8, 256, 3), (32, 64, 3), (4, 512, 2), (6, 384, 2)])
+@pytest.mark.parametrize("B,S,layers", [(32, 128, 5), (16, 128, 4), (64, 128, 3), (8, 384, 3), (8, 256, 3), (32, 64, 3), (4, 512, 2), (6, 384, 2),
+                                        (13, 128, 2), (5, 384, 2)])
 def test_many_rows_encoder_reuses_its_buffers(B, S, layers):
     """At many rows all layers of the fused launch share one set of inter-stage buffers (kept coherent
     by a cache invalidation at the barrier that ends a layer) and the LayerNorms are handed over per
@@ -191,6 +200,18 @@ def test_few_rows_handovers_on_repeated_launches(B, S, layers):
     assert_close("encoder x1", z_1, oracle.bert_encoder(x1, ws, B, S))
 
 
+def test_pack_fc2_layout():
+    """souffle_bert_pack_fc2: 48 slices of 16 columns, 96 k-steps of 64 lanes x 8 halves each; lane L of k-step t holds
+    W[32 t + 8 (L / 16) + 0..7][16 s + L % 16]."""
+    announce("bert pack_fc2 layout")
+    import bert_binding
+    w = synth.bert_layer_weights(1, 0)["fc2_weight"]
+    got = bert_binding.pack_fc2(dev(w)).cpu().numpy().reshape(48, 96, 64, 8)
+    s_, t_, L_, j_ = np.meshgrid(np.arange(48), np.arange(96), np.arange(64), np.arange(8), indexing="ij")
+    want = w[32 * t_ + 8 * (L_ // 16) + j_, 16 * s_ + L_ % 16]
+    assert np.array_equal(got, want)
+
+
 def test_few_rows_polled_copy_is_voted_in_the_first_launches():
     """Each XCD polls one of two copies of the hand-over words; which one is decided by votes that workgroup x of
     XCD x casts at the end of the first eight launches on a workspace.  A fresh workspace has no votes and polls the
@@ -232,10 +253,11 @@ def test_few_rows_shapes_take_turns_in_one_workspace():
     import bert_binding
     ws = [synth.bert_layer_weights(6, l, with_bias=True) for l in range(4)]
     dws = [dev_weights(w) for w in ws]
-    cases = [(1, 128, 4), (2, 64, 2), (1, 256, 3), (3, 128, 1), (1, 384, 2), (1, 128, 4)]
+    # (with and without the packed copy of the FC2 weights: the two forms of FC2 use different words of the workspace)
+    cases = [(1, 128, 4, True), (2, 64, 2, False), (1, 256, 3, True), (3, 128, 1, True), (1, 384, 2, False), (1, 128, 4, False)]
     encs, xs, want = [], [], []
-    for B, S, layers in cases:
-        enc = bert_binding.Encoder(dws[:layers], B, S)
+    for B, S, layers, pack in cases:
+        enc = bert_binding.Encoder(dws[:layers], B, S, pack=pack)
         x = dev(synth.bert_input(7, B, S))
         want.append(enc(x).clone())
         encs.append(enc)
@@ -341,7 +363,7 @@ def test_sequence_lengths_that_are_not_built(B, S, layers, masked):
     assert_close("encoder fused", y_f, ref)
     assert torch.equal(y_f, y_u)
     if layers == 1:
-        outs = run_layer(ws[0], x, B, S, 4, mask=md)
+        outs = run_layer(ws[0], x, B, S, 4, mask=md, pack=True)      # (the encoder object packs its FC2 weights: same form of FC2)
         full = oracle.bert_layer(x, ws[0], B, S, mask=mask, dump=True)
         for n, g, r in zip(NAMES, outs, full):
             assert_close(n, g, r)

@@ -14,18 +14,21 @@ QKV, ATT, OUT, FC1, FC2, FIN = 0, 1, 2, 3, 4, 6
 H, HD = 768, 64
 
 
-def plan(B, S, G, phase, b):
+def plan(B, S, G, packed, phase, b):
     items = (C.c_int * 64)()
     n = C.c_int(0)
     needs = (C.c_ubyte * G)()
-    sh.check(sh.lib().souffle_bert_handover_plan(B, S, G, phase, b, items, 32, C.byref(n), needs))
+    sh.check(sh.lib().souffle_bert_handover_plan(B, S, G, packed, phase, b, items, 32, C.byref(n), needs))
     assert n.value <= 32, n.value
     return [(items[2 * i], items[2 * i + 1]) for i in range(n.value)], np.frombuffer(needs, dtype=np.uint8).copy()
 
 
-def writes(phase, item, B, S):
+def writes(phase, item, B, S, packed):
     """(tensor, row range, column range) written by an item."""
     a, b = item
+    if phase == FC2:                       # whole-K form only: (m-tile, 16 columns) of the sum z2 (and their statistics)
+        assert packed
+        return ("z2", range(32 * a, 32 * a + 32), range(16 * b, 16 * b + 16))
     if phase == QKV:                       # (m-tile, which * 12 + head) -> rows of q, k or v of one head
         return ("qkv%d" % (b // 12), range(32 * a, 32 * a + 32), range((b % 12) * HD, (b % 12 + 1) * HD))
     if phase == ATT:                       # (query block, batch * 12 + head) -> 16 rows of ctx, the head's columns
@@ -38,9 +41,14 @@ def writes(phase, item, B, S):
     raise AssertionError(phase)
 
 
-def reads(phase, item, B, S):
+def reads(phase, item, B, S, packed):
     """What an item reads of the phase before it: a list of (tensor, rows, columns)."""
     a, b = item
+    if phase in (QKV, FIN):                # whole-K form: whole rows of z2 (QKV of a later layer: LayerNorm over the row; FIN: the
+        assert packed                      # row statistics)
+        return [("z2", range(32 * a, 32 * a + 32), range(0, H))]
+    if phase == FC2 and packed:            # the whole K of h
+        return [("h", range(32 * a, 32 * a + 32), range(0, 4 * H))]
     if phase == ATT:
         batch, head = b // 12, b % 12
         cols = range(head * HD, (head + 1) * HD)
@@ -65,11 +73,13 @@ def overlap(r, w):
 SHAPES = [(1, 64), (1, 128), (2, 128), (1, 256), (3, 256), (1, 384), (2, 384), (1, 512), (7, 128), (15, 64), (8, 128), (2, 512), (11, 128)]
 
 
+# (the kernel runs grids that are multiples of 8 up to 256; the plan functions are also defined, and checked, for other grids)
 @pytest.mark.parametrize("B,S", SHAPES)
 @pytest.mark.parametrize("G", [256, 304, 100])
-def test_every_dependence_is_waited_for_and_every_item_has_one_owner(B, S, G):
+@pytest.mark.parametrize("packed", [1, 0])
+def test_every_dependence_is_waited_for_and_every_item_has_one_owner(B, S, G, packed):
     M = B * S
-    owned = {ph: [plan(B, S, G, ph, b) for b in range(G)] for ph in (QKV, ATT, OUT, FC1, FC2, FIN)}
+    owned = {ph: [plan(B, S, G, packed, ph, b) for b in range(G)] for ph in (QKV, ATT, OUT, FC1, FC2, FIN)}
     # partition: every item of a phase exactly once
     expect = {QKV: {(mt, ws) for mt in range(M // 32) for ws in range(36)},
               ATT: {(qb, bh) for qb in range(S // 16) for bh in range(B * 12)},
@@ -82,13 +92,14 @@ def test_every_dependence_is_waited_for_and_every_item_has_one_owner(B, S, G):
         assert len(flat) == len(set(flat)), "phase %d: an item has two owners" % ph
         assert set(flat) == expect[ph], "phase %d: items missing or surplus" % ph
     # coverage: consumer workgroup b must wait for every producer workgroup pb whose items write what b's items read
-    for cph, pph in ((ATT, QKV), (OUT, ATT), (FC1, OUT), (FC2, FC1)):
-        prod = [[writes(pph, it, B, S) for it in items] for items, _ in owned[pph]]
+    pairs = ((ATT, QKV), (OUT, ATT), (FC1, OUT), (FC2, FC1)) + (((QKV, FC2), (FIN, FC2)) if packed else ())
+    for cph, pph in pairs:
+        prod = [[writes(pph, it, B, S, packed) for it in items] for items, _ in owned[pph]]
         for b in range(G):
             items, needs = owned[cph][b]
             if not items:
                 continue
-            rd = [r for it in items for r in reads(cph, it, B, S)]
+            rd = [r for it in items for r in reads(cph, it, B, S, packed)]
             for pb in range(G):
                 if prod[pb] and any(overlap(r, w) for r in rd for w in prod[pb]):
                     assert needs[pb], "B=%d S=%d G=%d: workgroup %d phase %d reads what workgroup %d writes and does not wait for it" % (B, S, G, b, cph, pb)
@@ -99,9 +110,9 @@ def test_every_dependence_is_waited_for_and_every_item_has_one_owner(B, S, G):
 def test_plan_rejects_what_the_few_rows_path_does_not_run():
     n = C.c_int(0)
     lib = sh.lib()
-    assert lib.souffle_bert_handover_plan(12, 128, 256, 0, 0, None, 0, C.byref(n), None) == -2     # 1536 rows: the many-rows path
-    assert lib.souffle_bert_handover_plan(10, 128, 256, 0, 0, None, 0, C.byref(n), None) == -2     # 1280 rows, a multiple of 256: likewise
-    assert lib.souffle_bert_handover_plan(1, 100, 256, 0, 0, None, 0, C.byref(n), None) == -2
-    assert lib.souffle_bert_handover_plan(1, 128, 256, 5, 0, None, 0, C.byref(n), None) == -2
-    assert lib.souffle_bert_handover_plan(1, 128, 256, 0, 256, None, 0, C.byref(n), None) == -2
-    assert lib.souffle_bert_handover_plan(1, 128, 256, 0, 0, None, 0, None, None) == -1
+    assert lib.souffle_bert_handover_plan(12, 128, 256, 1, 0, 0, None, 0, C.byref(n), None) == -2     # 1536 rows: the many-rows path
+    assert lib.souffle_bert_handover_plan(10, 128, 256, 0, 0, 0, None, 0, C.byref(n), None) == -2     # 1280 rows, a multiple of 256: likewise
+    assert lib.souffle_bert_handover_plan(1, 100, 256, 1, 0, 0, None, 0, C.byref(n), None) == -2
+    assert lib.souffle_bert_handover_plan(1, 128, 256, 1, 5, 0, None, 0, C.byref(n), None) == -2
+    assert lib.souffle_bert_handover_plan(1, 128, 256, 0, 0, 256, None, 0, C.byref(n), None) == -2
+    assert lib.souffle_bert_handover_plan(1, 128, 256, 1, 0, 0, None, 0, None, None) == -1
