@@ -1140,7 +1140,15 @@ static int launch_small_t(sk::Args &a, int grid, hipStream_t st) {
   const sk::Shape sh{a.B, a.S, a.M, a.M / 32, grid, a.packed};
   return sk::single_pass(sh) ? launch_small_tt<NKT, false>(a, grid, st) : launch_small_tt<NKT, true>(a, grid, st);
 }
+// The few-rows kernels deal weight slices to XCDs by workgroup number modulo 8 and keep one flag word and one row of
+// wait masks per workgroup.
+static int check_small_grid(int grid) {
+  if (grid <= 0 || grid % 8 != 0 || grid > sk::kMaxGrid)
+    return fail(SOUFFLE_ERR_DEVICE, "the few-rows encoder needs a grid that is a multiple of 8 in 8..%d workgroups (this device gives %d)", sk::kMaxGrid, grid);
+  return SOUFFLE_OK;
+}
 static int launch_small(sk::Args &a, int grid, hipStream_t st) {
+  if (int rc = check_small_grid(grid)) return rc;
   switch (a.S) {
 #ifdef SOUFFLE_DEV_ONLY_S128      // development builds: one sequence length, a fifth of the compile time
     case 128: return launch_small_t<8>(a, grid, st);
@@ -1174,6 +1182,7 @@ static int run_small_unfused_t(sk::Args &a, int grid, hipStream_t st) {
   return SOUFFLE_OK;
 }
 static int run_small_unfused(sk::Args &a, int grid, hipStream_t st) {
+  if (int rc = check_small_grid(grid)) return rc;
   switch (a.S) {
 #ifdef SOUFFLE_DEV_ONLY_S128      // development builds: one sequence length, a fifth of the compile time
     case 128: return run_small_unfused_t<8>(a, grid, st);

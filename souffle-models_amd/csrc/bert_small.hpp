@@ -81,7 +81,18 @@ constexpr int kSideVotes = 8;
 constexpr int kFlagWords = kFlagBaseWord + 64;
 __host__ __device__ constexpr int pair_base_of(int x) { return (x >> 1) * 4 + (x & 1); }      // XCD x: blocks pair_base, pair_base + 2
 constexpr int kTileCntWord = kFlagWords;                         // kMaxLayers x kTileWords
-constexpr int kFlagRegionWords = kTileCntWord + kMaxLayers * kTileWords;
+// The wait masks of a launch (which workgroups' flag words a workgroup polls in front of each phase) depend on the shape
+// and the grid alone.  The first launch of a shape on a workspace works them out (some 5 us) and leaves them here, two
+// words per workgroup and lane of a wave; the workgroup that ends last then stores the key of the shape, and every
+// later launch that finds its own key reads its masks back with one load per thread.
+constexpr int kMaskKeyWord = kTileCntWord + kMaxLayers * kTileWords;
+constexpr int kMaskTabWord = kMaskKeyWord + 4;                   // kMaxGrid x 64 lanes x 2 words
+constexpr int kMaxGrid = 256;                                    // one flag word per workgroup in a copy's block, one mask row per workgroup
+static_assert(kMaxGrid <= kBlockTileWord, "the flag words of a copy lie in front of its tile words");
+constexpr int kFlagRegionWords = kMaskTabWord + kMaxGrid * 128;
+__host__ __device__ __forceinline__ unsigned mask_key(int B, int S, int G, int packed) {
+  return 0x80000000u | ((unsigned)(packed != 0) << 30) | ((unsigned)G << 16) | ((unsigned)(S / 64) << 12) | (unsigned)B;
+}
 static_assert(kFlagWords % 4 == 0 && kTileWords % 4 == 0, "16-byte polls");
 constexpr int kMaxFlagSpin = 1 << 21;                          // about a second of polling
 
@@ -96,6 +107,7 @@ struct Sync {
   unsigned base;         // flag value of (layer l, phase p) = base + 1 + l * PH_SLOTS + p
   int block;             // the copy this workgroup polls
   unsigned votes;        // the vote word of this workgroup's XCD as the launch found it
+  unsigned key;          // key of this launch's wait masks, 0 when the workspace already holds them
   bool failed;
   // optional stamps of the 100 MHz clock, slot i = layer * PH_SLOTS + phase: trace[(2 i + {0,1}) * G + block] = entry to /
   // exit from the wait in front of the phase, trace[(2 cap + 8 i + id) * G + block] = marks inside it (0 operands of the
@@ -240,6 +252,7 @@ __device__ __forceinline__ void sync_begin(Sync &sy, unsigned *flags, unsigned *
   const int x = blockIdx.x & 7;
   sy.votes = __hip_atomic_load(flags + kSideWord + x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   sy.block = pair_base_of(x) + (((int)sy.votes >> 16) < 0 ? 2 : 0);
+  sy.key = 0;      // (set by the kernel once it knows whether the workspace holds this shape's wait masks)
 }
 // One vote on which of the XCD's two copies is nearer: loads of two unused lines of each (the last 768 bytes of a
 // block are never written, and the weights that stream through the L2 in a launch have long evicted them), in the
@@ -271,6 +284,8 @@ __device__ __forceinline__ void sync_end(Sync &sy, int num_layers) {
   if (threadIdx.x == 0) {
     const unsigned old = __hip_atomic_fetch_add(sy.flags + kFlagDoneWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (old + 1 == gridDim.x) {
+      // (every workgroup stored its wait masks long before it ended, and waited for the acknowledgement at its first publication)
+      if (sy.key) __hip_atomic_store(sy.flags + kMaskKeyWord, sy.key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(sy.flags + kFlagDoneWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(sy.flags + kFlagBaseWord, sy.base + (unsigned)((num_layers + 1) * PH_SLOTS), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -311,6 +326,29 @@ __device__ __forceinline__ void await_words(Sync &sy, const unsigned *words, uns
 #endif
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+}
+// The calling WAVE alone waits for the workgroups named by its `mask` (4 per lane): for what only this wave reads.  No
+// workgroup barrier; the caller's loads of those workgroups' results follow in program order.
+__device__ __forceinline__ void await_wave(Sync &sy, unsigned mask, unsigned seq, int slot) {
+  stamp_wait(sy, slot, 0);
+  if (!sy.failed) {
+    const unsigned *words = sy.flags + sy.block * kBlockWords;
+    const int lane = (int)threadIdx.x & 63;
+    for (int spin = 0;; ++spin) {
+      const u4 f = ld16<true>(words, lane * 16);
+      bool ok = true;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) ok &= !((mask >> t) & 1u) || (int)(f[t] - seq) >= 0;
+      if (__all(ok)) break;
+      if (spin >= kMaxFlagSpin) {
+        sy.failed = true;
+        if (lane == 0) (void)__hip_atomic_fetch_or(sy.err, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+    }
+  }
+  stamp_wait(sy, slot, 1);
+  compiler_fence();
 }
 // ... the workgroups named by `mask` (4 per lane) have published `seq`
 __device__ __forceinline__ void await(Sync &sy, unsigned mask, unsigned seq, int slot) {
@@ -965,11 +1003,17 @@ __device__ __forceinline__ int h_operand_offset(int m, int n) {
 // MFMAs run behind the data as it arrives.  The four partial tiles are summed through LDS, and the
 // workgroup that multiplied a tile finishes its rows: + bias + LN1(z1), rounded, with the statistics of the 16
 // columns.  No partial sum leaves the CU.
-__device__ __forceinline__ void run_fc2_whole_k(unsigned char *lds, const Args &a, int l, const It &d, const Job &j, bool w_ready, const Sync *sy) {
+// wsy / wmask / wseq: this WAVE waits here, for the FC1 workgroups that wrote its K quarter of the rows (the twelve
+// slices 12 w .. 12 w + 11 of h).  A wave whose producers are early takes its quarter in while another still waits
+// for a late one.
+__device__ __forceinline__ void run_fc2_whole_k(unsigned char *lds, const Args &a, int l, const It &d, const Job &j, bool w_ready, const Sync *sy,
+                                                Sync *wsy = nullptr, unsigned wmask = 0, unsigned wseq = 0) {
   const int tid = opaque_thread_id(), lane = tid & 63, w = tid >> 6, l16 = lane & 15, gq = lane >> 4;
   if (!w_ready) issue_weights(lds, j, false);
   // the residual: this thread's four columns of z1 (threads 0..127: row tid / 4), and the rows' statistics
   const int row = (tid >> 2) & 31, c4 = (tid & 3) * 4;
+  // (behind the wait: an FC1 workgroup of this m-tile has published only after the out-projection finished the m-tile's z1)
+  if (wsy) await_wave(*wsy, wmask, wseq, l * PH_SLOTS + PH_FC2);
   const u2 zres = ld8<true>(j.res, ((j.g.m0 + row) * H + j.g.n0 + c4) * 2);
   issue_stats_rows<kNS1>(lds, j.rstats, j.g.m0);
   // this wave's K quarter of the 32 rows: segment (8 k-steps = 512 bytes of a row) after segment, in the order rot, rot + 1, ...
@@ -987,7 +1031,7 @@ __device__ __forceinline__ void run_fc2_whole_k(unsigned char *lds, const Args &
       });
     });
   }
-  wait_vmcnt<48>();                                   // everything older than the 48 activation loads: residual, statistics, a weight slice requested here
+  wait_vmcnt<48>();                                   // everything older than the 48 activation loads: residual, statistics, this wave's quarter of the weight slice
   if (sy && sy->trace) stamp_mark(*sy, l * PH_SLOTS + PH_FC2, 0);
   combine_stats_rows<kNS1>(lds, a.eps);               // (read behind the barrier in front of the epilogue)
   f4 acc[2][2];
@@ -1041,10 +1085,11 @@ __device__ __forceinline__ void run_fc2_whole_k(unsigned char *lds, const Args &
 
 // One GEMM item from operand fetch to the stores of its epilogue.
 template <int PH>
-__device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &a, int l, const It &d, const Job &j, bool w_ready, const Sync *sy = nullptr) {
+__device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &a, int l, const It &d, const Job &j, bool w_ready, const Sync *sy = nullptr,
+                                                Sync *wsy = nullptr, unsigned wmask = 0, unsigned wseq = 0) {
   constexpr int ph = PH;
   if constexpr (ph == PH_FC2) {
-    if (a.packed) { run_fc2_whole_k(lds, a, l, d, j, w_ready, sy); return; }
+    if (a.packed) { run_fc2_whole_k(lds, a, l, d, j, w_ready, sy, wsy, wmask, wseq); return; }
   }
   if (!w_ready) issue_weights(lds, j, false);
   // what the item reads of other workgroups' results, statistics first (they are needed first)
@@ -1281,10 +1326,13 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
   const Shape sh{args.B, args.S, args.M, args.M / 32, (int)gridDim.x, args.packed};
   Sync sy;
   sync_begin(sy, args.flags, args.ctl + kCtlErrWord, args.trace, args.trace_cap);
+  const unsigned masks_key = mask_key(sh.B, sh.S, sh.G, sh.packed);
+  const bool masks_kept = __hip_atomic_load(args.flags + kMaskKeyWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == masks_key;
+  if (!masks_kept) sy.key = masks_key;      // (every workgroup: the one that ends last stores the key, and it may be one without items)
   const int L = args.num_layers;
   stamp_wait(sy, PH_SLOTS - 1, 0);          // (slot 7 of layer 0 is no phase: start of the kernel, end of its set-up)
   // In which phases this workgroup has items (one bit per phase; packed so that the phase code indexes no register array).
-  unsigned wm_all = 0, mine_bits = 0;
+  unsigned wm_all = 0, wm_fc2 = 0, mine_bits = 0;      // wm_fc2: whole-K FC2, this wave's producers (those of its K quarter of h)
   for (int ph = 0; ph <= PH_FIN; ++ph)
     if (ph != PH_RED) mine_bits |= (has_items(sh, ph, b) ? 1u : 0u) << ph;       // (the split-K sum is finished inside FC2)
   auto mine = [&](int ph) { return ((mine_bits >> ph) & 1u) != 0; };
@@ -1309,7 +1357,8 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
         if (mine(PH_ATT)) done = true;                  // the attention tiles overlap the W region
       } else if constexpr (pp != PH_RED) {
         if (mine(pp)) {
-          issue_weights(lds, make_job_t<pp>(args, l + dl, first_of(std::integral_constant<int, pp>{}).d), true);
+          // (whole-K FC2: every wave requests its own quarter, since every wave waits for itself)
+          issue_weights(lds, make_job_t<pp>(args, l + dl, first_of(std::integral_constant<int, pp>{}).d), !(pp == PH_FC2 && sh.packed));
           pf = (l + dl) * 8 + pp;
           done = true;
         }
@@ -1369,8 +1418,11 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
         if (tid >= 64) wait_vmcnt<0>();
         __syncthreads();
       }
+    } else if (ph == PH_FC2 && sh.packed) {
+      // (every wave waits for its own producers inside the item; the weight slice requested ahead is this wave's own quarter)
     } else await(sy, wm(ph), phase_seq(sy, l, ph - 1), l * PH_SLOTS + ph);
-    run_gemm_item_t<ph>(lds, args, l, f0.d, j0, ready, &sy);
+    if (ph == PH_FC2 && sh.packed) run_gemm_item_t<ph>(lds, args, l, f0.d, j0, ready, &sy, &sy, wm_fc2, phase_seq(sy, l, PH_FC1));
+    else run_gemm_item_t<ph>(lds, args, l, f0.d, j0, ready, &sy);
     if constexpr (MULTI) for (int i = 1; i < f0.count; ++i) {      // further m-tiles of the same weight slice, which stays where it is
       const It d{f0.d.a + i * f0.step, f0.d.b};
       __syncthreads();                                        // the partial tiles of the previous item have been read
@@ -1386,18 +1438,38 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
   // Who feeds whom (wave 0: 4 workgroups per lane, one nibble per phase), worked out while the first weight slice
   // travels.  Thread t answers for producer workgroup t; the answers reach the lanes of wave 0 through LDS (the start
   // of the X region, which nothing has been requested into yet).  QKV and FIN wait for tiles, not for workgroups.
+  // Lane i of a wave keeps two words: one nibble per phase (the four workgroups 4 i .. 4 i + 3), and for whole-K FC2 one
+  // nibble per K quarter (which of the four wrote that quarter of h).  Found in the workspace when a launch of this
+  // shape has left them there, worked out otherwise.
   if (mine_bits != 0) {
-    unsigned needs = 0;
-    for (int ph = PH_ATT; ph <= PH_FC2; ++ph) needs |= (wait_needs(sh, ph, b, tid) ? 1u : 0u) << ph;
-    if (sh.packed) needs |= (wait_needs(sh, PH_QKV, b, tid) ? 1u : 0u) << PH_QKV | (wait_needs(sh, PH_FIN, b, tid) ? 1u : 0u) << PH_FIN;
-    lds[tid] = (unsigned char)needs;
-    __syncthreads();
-    if (tid < 64) {
-      const unsigned four = *reinterpret_cast<const unsigned *>(lds + 4 * tid);
+    unsigned *tab = args.flags + kMaskTabWord + b * 128;      // this workgroup's row: two words per lane
+    unsigned quarters = 0;
+    if (masks_kept) {
+      const u2 v = ld8<true>(tab, (tid & 63) * 8);
+      wm_all = v[0]; quarters = v[1];
+    } else {
+      unsigned needs = 0, quarter = 0;
+      for (int ph = PH_ATT; ph <= PH_FC2; ++ph) needs |= (wait_needs(sh, ph, b, tid) ? 1u : 0u) << ph;
+      if (sh.packed) {
+        needs |= (wait_needs(sh, PH_QKV, b, tid) ? 1u : 0u) << PH_QKV | (wait_needs(sh, PH_FIN, b, tid) ? 1u : 0u) << PH_FIN;
+        It pd;
+        if (tid < sh.G && wg_item(sh, PH_FC1, tid, 0, pd)) quarter = (unsigned)pd.b / 12u;      // (a workgroup has ONE weight slice per phase)
+      }
+      lds[tid] = (unsigned char)(needs | (quarter << 7));
+      lds[256 + tid] = (unsigned char)(quarter >> 1);
+      __syncthreads();
+      const int i = tid & 63;
+      const unsigned four = *reinterpret_cast<const unsigned *>(lds + 4 * i), hi = *reinterpret_cast<const unsigned *>(lds + 256 + 4 * i);
       for (int ph = PH_QKV; ph <= PH_FIN; ++ph)
         for (int t = 0; t < 4; ++t) wm_all |= ((four >> (8 * t + ph)) & 1u) << (4 * ph + t);
+      for (int t = 0; t < 4; ++t) {
+        const unsigned q = ((four >> (8 * t + 7)) & 1u) | (((hi >> (8 * t)) & 1u) << 1);
+        quarters |= ((four >> (8 * t + PH_FC2)) & 1u) << (4 * q + t);
+      }
+      __syncthreads();
+      if (tid < 64) st8<true>(tab, tid * 8, u2{wm_all, quarters});
     }
-    __syncthreads();
+    wm_fc2 = (quarters >> (4 * (tid >> 6))) & 15u;
   }
   stamp_wait(sy, PH_SLOTS - 1, 1);
 #pragma unroll 1
