@@ -41,6 +41,7 @@ def parse():
     p.add_argument("--no-sub", action="store_true", help="skip the S=384 and B=32 sub-results of the default workload")
     p.add_argument("--no-coop", action="store_true", help="skip the cooperative-launch timing of the encoder workloads")
     p.add_argument("--weight-sets", type=int, default=4)
+    p.add_argument("--no-pack", action="store_true", help="encoders keep the [K][N] FC2 matrices only (split-K FC2) instead of packing them once")
     return p.parse_args()
 
 
@@ -95,7 +96,7 @@ def encoder_sub_result(args, B, S, L=12):
     dev = torch.device("cuda:0")
     layers_np = [synth.bert_layer_weights(2, l) for l in range(L)]
     x_np = synth.bert_input(2, B, S)
-    enc = bert_binding.Encoder([{k: torch.from_numpy(v).to(dev) for k, v in w.items()} for w in layers_np], B, S)
+    enc = bert_binding.Encoder([{k: torch.from_numpy(v).to(dev) for k, v in w.items()} for w in layers_np], B, S, pack=not args.no_pack)
     x = torch.from_numpy(x_np).to(dev)
     out = torch.empty((B * S, 768), dtype=torch.float16, device=dev)
     y = enc(x, out=out).float().cpu().numpy()
@@ -153,7 +154,7 @@ def bench_encoder(args, B, S, L, name):
     sets = [[to_dev(w) for w in layers_np]]
     for s in range(1, max(1, args.weight_sets)):
         sets.append([{k: v.clone() for k, v in sets[0][(l + s) % L].items()} for l in range(L)])
-    encs = [bert_binding.Encoder(ls, B, S) for ls in sets]
+    encs = [bert_binding.Encoder(ls, B, S, pack=not args.no_pack) for ls in sets]
     out = torch.empty((M, 768), dtype=torch.float16, device=dev)
 
     # parity gate
