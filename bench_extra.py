@@ -250,6 +250,100 @@ def bench_swin_merge(args):
     return res
 
 
+def _parity(name, got, ref, max_abs=2e-2, mean_abs=2e-3):
+    import numpy as np
+    d = np.abs(np.asarray(got, np.float32).reshape(-1) - np.asarray(ref, np.float32).reshape(-1))
+    if not (np.isfinite(got).all() and d.max() <= max_abs and d.mean() <= mean_abs):
+        print("PARITY FAILURE (%s): max-abs %.4g mean-abs %.4g" % (name, d.max(), d.mean()), file=sys.stderr)
+        sys.exit(1)
+    return {"max_abs": float(d.max()), "mean_abs": float(d.mean())}
+
+
+def sub_results(args):
+    """The other BASELINE configurations as short sub-results of the default line: each checked against the CPU oracle
+    first (unless --no-cpu) and then timed as bare C-ABI launches on preallocated outputs (HIP events on the launch
+    stream, min over rounds of the mean: the reference's timing rule)."""
+    import numpy as np
+    import torch
+    import souffle_hip as sh
+    import synth
+    out = {}
+    oracle = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle
+    thr = _threads()
+    timed = lambda launch: sh.bench_us(launch, warmup=10, rounds=3, repeat=max(10, min(50, args.steps)))
+
+    # configs[1]: stacked LSTM
+    import lstm_binding
+    w_ih, w_hh, x = synth.lstm_tensors(1)
+    d = lambda a, t: torch.from_numpy(a).to("cuda:0", dtype=t).contiguous()
+    dx, dwi, dwh = d(x, torch.float32).view(1, 100, 256), d(w_ih, torch.float16), d(w_hh, torch.float16)
+    y = lstm_binding.fused_lstm(dx, dwi, dwh)[0].cpu().numpy()
+    par = _parity("lstm", y, oracle.lstm(x, w_ih, w_hh)) if oracle else None
+    mn, med = timed(lambda: lstm_binding.fused_lstm(dx, dwi, dwh))
+    out["lstm"] = {"workload": "stacked LSTM 10x256, T=100, batch 1 (BASELINE configs[1])", "us": mn, "median_us": med, "parity": par,
+                   "us_per_wavefront_step": mn / 109, "note": "109 dependent steps; timed through the binding (it allocates the output)"}
+
+    # configs[3]: Swin block pair
+    import swin_transformer_binding as sb
+    ws = [synth.swin_block_weights(3, b) for b in range(2)]
+    xs = synth.swin_input(3)
+    dw = [{k: torch.from_numpy(v).cuda() for k, v in w.items()} for w in ws]
+    dxs = torch.from_numpy(xs).cuda()
+    ys = torch.empty_like(dxs)
+    launch = sb.block_pair_launcher(dxs, dw[0], dw[1], ys)
+    launch()
+    par = _parity("swin", ys.float().cpu().numpy(), oracle.swin_block_pair(xs, ws, threads=thr)) if oracle else None
+    mn, med = timed(launch)
+    flops = 2 * (2.0 * 3136 * 196608 + 4.0 * 64 * 4 * 49 * 49 * 32)
+    out["swin_pair"] = {"workload": "Swin-Base stage-1 block pair 56x56, C=128, window 7, shift 3 (BASELINE configs[3])", "us": mn, "median_us": med,
+                        "parity": par, "mfma_frac": flops / (mn * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS}
+
+    # the reference's SE module, its ten shapes (fp32; tolerance 1e-4 relative to the largest value)
+    import efficientnet_se_module_binding as eb
+    shapes = [(32, 112, 8), (96, 56, 4), (144, 56, 6), (144, 28, 6), (240, 28, 10), (240, 14, 10), (480, 14, 20),
+              (672, 14, 28), (672, 7, 28), (1152, 7, 48)]
+    a100 = [23.33, 14.14, 15.65, 12.48, 12.86, 12.03, 12.86, 13.86, 13.28, 15.36]   # cpp/efficientnet/scripts/efficientnet-se_module_v2-max-block.xlsx, "Duration [usecond]", A100
+    rows, worst = [], 0.0
+    g = torch.Generator(device="cpu").manual_seed(5)
+    for (Cc, Hh, R), ref_us in zip(shapes, a100):
+        xn = torch.rand((1, Cc, Hh, Hh), generator=g).numpy()
+        wr, we = (torch.randn((R, Cc), generator=g) * 0.3).numpy(), (torch.randn((Cc, R), generator=g) * 0.3).numpy()
+        xd, wrd, wed = torch.from_numpy(xn).cuda(), torch.from_numpy(wr).cuda(), torch.from_numpy(we).cuda()
+        yd, pd = torch.empty_like(xd), torch.empty((1, Cc), device="cuda:0")
+        launch = eb.se_launcher(xd, wrd, wed, yd, pd, combine="add")
+        launch()
+        if oracle:
+            ref = oracle.se_module(xn.reshape(Cc, Hh * Hh), wr, we, combine="add")
+            ref_y = ref[0] if isinstance(ref, (tuple, list)) else ref
+            err = float(np.abs(yd.cpu().numpy().reshape(-1) - np.asarray(ref_y, np.float32).reshape(-1)).max() / max(1.0, float(np.abs(ref_y).max())))
+            if not err <= 1e-4:
+                print("PARITY FAILURE (se C=%d H=%d): relative error %.3g" % (Cc, Hh, err), file=sys.stderr)
+                sys.exit(1)
+            worst = max(worst, err)
+        mn, _ = timed(launch)
+        rows.append({"C": Cc, "H": Hh, "R": R, "us": mn, "reference_a100_us": ref_us, "vs_reference_a100": ref_us / mn})
+    out["se"] = {"workload": "EfficientNet-B0 SE module, the reference's 10 shapes, fp32, combine = add as in the reference", "us": sum(r["us"] for r in rows),
+                 "parity": {"max_rel": worst} if oracle else None, "reference_a100_sum_us": sum(a100), "per_shape": rows}
+
+    # configs[4]: MBConv stack
+    import efficientnet_binding as efb
+    blocks = synth.mbconv_stack_weights()
+    xm = synth.mbconv_input()
+    up = lambda v: torch.from_numpy(v).cuda() if isinstance(v, np.ndarray) else v
+    stack = efb.MBConvStack([{k: up(v) for k, v in b.items()} for b in blocks])
+    dxm = torch.from_numpy(xm).cuda()
+    ym = stack(dxm).float().cpu().numpy()
+    par = _parity("mbconv", ym, oracle.mbconv_stack(xm, blocks, threads=thr)) if oracle else None
+    mn, med = timed(lambda: stack(dxm))
+    stages = sum(3 if b["expand_w"] is not None else 2 for b in blocks)
+    out["mbconv"] = {"workload": "EfficientNet-B0 MBConv stack (16 blocks), 112x112x32 -> 7x7x320, fp16 (BASELINE configs[4], behind the stem)", "us": mn,
+                     "median_us": med, "parity": par, "stages": stages, "us_per_stage": mn / stages}
+    return out
+
+
 def run(args):
     if args.workload == "swin_merge":
         return bench_swin_merge(args)
