@@ -265,6 +265,16 @@ def bench_encoder(args, B, S, L, name):
         res["extra"]["cooperative_launch_error"] = str(e)
     finally:
         sh.set_cooperative_launch(0)
+    # the same launch with the memory model's release / acquire fences around every hand-over (souffle_set_strict_fences):
+    # the by-the-book form, same bits (tests/test_strict_fences.py), kept as a fallback
+    try:
+        sh.set_strict_fences(True)
+        _, strict_ev = time_steps(lambda i: encs[i % len(encs)](x, out=out), max(10, args.steps // 4), 3)
+        res["extra"]["strict_fences_us"] = strict_ev * 1e3
+    except sh.SouffleError as e:
+        res["extra"]["strict_fences_error"] = str(e)
+    finally:
+        sh.set_strict_fences(False)
     if cpu:
         res["cpu_baseline"] = cpu
         res["extra"]["gpu_speedup_vs_cpu"] = cpu["value"] / (cold_ev * 1e3)

@@ -94,6 +94,17 @@ int souffle_set_stage_trace(void *device_buf, size_t bytes);
  * guarantee.  The environment variable SOUFFLE_COOPERATIVE_LAUNCH=1 sets the initial value. */
 int souffle_set_cooperative_launch(int on);
 
+/* The hand-overs between the workgroups of the persistent kernels (flag words of the encoder, grid barriers,
+ * row-block and window hand-overs) rest on write-through stores that are acknowledged before the flag is stored and
+ * on cache-coherent (sc1) loads behind the poll; on MI355X that is sufficient and costs about 2 us per hand-over.
+ * on != 0 adds what the memory model prescribes by the book to every one of them: an agent-scope release fence in
+ * front of the flag store and an agent-scope acquire fence behind the poll (an L2 write-back and an L1/L2
+ * invalidation each time; about 14 us per hand-over).  Same results, bit for bit.  For a driver, firmware or part
+ * whose caches are not known to behave as measured here, and for checking a suspected coherence problem.
+ * The environment variable SOUFFLE_STRICT_FENCES=1 sets the initial value.  The reference separates its stages
+ * with cooperative-groups grid.sync() (cpp/bert/kernels/fused_sqq_bert.cu), which carries these fences always. */
+int souffle_set_strict_fences(int on);
+
 /* Reads (and optionally clears) the sticky failure flags of a workspace after waiting for
  * `stream`: 0 = every launch that used it ran to completion; bit 0 = an LSTM wait, bit 1 = a
  * grid barrier or a hand-over of the encoder gave up (bounded spins; the output of

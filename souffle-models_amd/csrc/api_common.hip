@@ -61,6 +61,16 @@ int swin_split_mode() {
   }
   return v;
 }
+static std::atomic<int> g_strict{-1};
+int strict_fences_mode() {
+  int v = g_strict.load();
+  if (v < 0) {
+    const char *e = getenv("SOUFFLE_STRICT_FENCES");
+    v = (e && e[0] == '1') ? 1 : 0;
+    g_strict.store(v);
+  }
+  return v;
+}
 static std::atomic<int> g_cooperative{-1};
 static bool cooperative_mode() {
   int v = g_cooperative.load();
@@ -245,9 +255,9 @@ extern "C" int souffle_l2_stream_probe(const void *src, size_t src_bytes, int it
 // goes into what it writes next, so each stage costs a store acknowledgement, a barrier and one
 // memory round trip, like a real stage with no arithmetic.
 namespace souffle {
-__global__ void __launch_bounds__(256) k_stage_floor(unsigned *ctl, u4 *buf, int n, int mode, unsigned *out) {
+__global__ void __launch_bounds__(256) k_stage_floor(unsigned *ctl, u4 *buf, int n, int mode, unsigned *out, int strict) {
   GridBarrier bar;
-  grid_barrier_begin(bar, ctl);
+  grid_barrier_begin(bar, ctl, strict != 0);
   const int grid = gridDim.x, peer = (blockIdx.x + 37) % grid;
   u4 v = {blockIdx.x, 1u, 2u, 3u};
   for (int i = 0; i < n; ++i) {
@@ -275,7 +285,8 @@ extern "C" int souffle_stage_floor_probe(void *ws, size_t ws_bytes, int stages, 
   unsigned *ctl = static_cast<unsigned *>(ws);
   u4 *buf = reinterpret_cast<u4 *>(static_cast<char *>(ws) + ctl_bytes);
   unsigned *out = reinterpret_cast<unsigned *>(static_cast<char *>(ws) + ctl_bytes + (size_t)df.num_cus * 32);
-  void *args[] = {&ctl, &buf, &stages, &mode, &out};
+  int strict = strict_fences_mode();
+  void *args[] = {&ctl, &buf, &stages, &mode, &out, &strict};
   return launch_persistent((const void *)souffle::k_stage_floor, df.num_cus, 256, args, 0, static_cast<hipStream_t>(stream));
 }
 
@@ -284,6 +295,10 @@ extern "C" int souffle_set_cooperative_launch(int on) {
   return SOUFFLE_OK;
 }
 
+extern "C" int souffle_set_strict_fences(int on) {
+  souffle::g_strict.store(on ? 1 : 0);
+  return SOUFFLE_OK;
+}
 extern "C" int souffle_set_swin_split(int on) {
   souffle::g_swin_split.store(on ? 1 : 0);
   return SOUFFLE_OK;

@@ -57,6 +57,7 @@ struct Params {
   int trace_cap;
   size_t layer_stride;
   int layer_sets;      // layer l uses buffer set l % layer_sets
+  int strict;          // souffle_set_strict_fences
 };
 struct Args : Params {
   LayerW layers[kMaxLayers];
@@ -449,6 +450,7 @@ __device__ __forceinline__ void rowblock_sync(const Params &a, GridBarrier &bar,
   const bool tr = bar.trace && bar.trace_idx < bar.trace_cap && threadIdx.x == 0;
   if (tr) bar.trace[(size_t)(2 * bar.trace_idx) * bar.nblk + blockIdx.x] = wall_clock64();
   wait_all_memory();                             // this wave's write-through stores are acknowledged
+  strict_release(bar.strict);
   __syncthreads();
   if (threadIdx.x == 0)
     for (int it = first; it < m_tiles * 16; it += stride) {
@@ -478,6 +480,7 @@ __device__ __forceinline__ void rowblock_sync(const Params &a, GridBarrier &bar,
   if (tr) bar.trace[(size_t)(2 * bar.trace_idx + 1) * bar.nblk + blockIdx.x] = wall_clock64();
   bar.trace_idx++;
   __syncthreads();
+  strict_acquire(bar.strict);
   compiler_fence();                              // no load of the other tiles' results is scheduled above the poll
 }
 template <bool COH, int NZ>
@@ -766,7 +769,7 @@ __global__ void __launch_bounds__(256) k_encoder_mega(Args args) {
   half_t *lds = reinterpret_cast<half_t *>(lds_raw);
   using Tile = TileLarge;
   GridBarrier bar;
-  grid_barrier_begin(bar, args.ctl);
+  grid_barrier_begin(bar, args.ctl, args.strict != 0);
   bar.trace = args.trace;
   bar.trace_cap = args.trace_cap;
   const int first = blockIdx.x, stride = gridDim.x;
@@ -1026,6 +1029,7 @@ static int fill_args(Args &a, const souffle_bert_cfg *c, const souffle_bert_laye
   char *base = static_cast<char *>(ws);
   a.B = c->batch; a.S = c->seq_len; a.M = c->batch * c->seq_len; a.act = c->act; a.num_layers = nl;
   a.splitk_o = 1; a.splitk_f = 1; a.scale = c->scale; a.eps = c->ln_eps;
+  a.strict = strict_fences_mode();
   a.big = p.big ? 1 : 0;
   a.x = static_cast<const half_t *>(x); a.mask = static_cast<const half_t *>(mask); a.y = static_cast<half_t *>(y);
   a.ctl = reinterpret_cast<unsigned *>(base + p.off_ctl);
@@ -1061,6 +1065,7 @@ static int fill_small(sk::Args &a, const souffle_bert_cfg *c, const souffle_bert
   char *base = static_cast<char *>(ws);
   a.B = c->batch; a.S = c->seq_len; a.M = c->batch * c->seq_len; a.act = c->act; a.num_layers = nl;
   a.scale = c->scale; a.eps = c->ln_eps;
+  a.strict = strict_fences_mode();
   a.x = static_cast<const half_t *>(x); a.mask = static_cast<const half_t *>(mask); a.y = static_cast<half_t *>(y);
   a.ctl = reinterpret_cast<unsigned *>(base + p.off_ctl);
   a.flags = reinterpret_cast<unsigned *>(base + p.off_flags);

@@ -109,6 +109,7 @@ struct Sync {
   unsigned votes;        // the vote word of this workgroup's XCD as the launch found it
   unsigned key;          // key of this launch's wait masks, 0 when the workspace already holds them
   bool failed;
+  bool strict;           // release / acquire fences of the memory model around every hand-over (strict_release)
   // optional stamps of the 100 MHz clock, slot i = layer * PH_SLOTS + phase: trace[(2 i + {0,1}) * G + block] = entry to /
   // exit from the wait in front of the phase, trace[(2 cap + 8 i + id) * G + block] = marks inside it (0 operands of the
   // first k-step there, 1 MFMAs done, 2 stores issued, 3 published)
@@ -245,6 +246,7 @@ __device__ __forceinline__ void sync_begin(Sync &sy, unsigned *flags, unsigned *
   sy.flags = flags;
   sy.err = err;
   sy.failed = false;
+  sy.strict = false;
   sy.trace = trace;
   sy.trace_cap = trace_cap;
   sy.base = __hip_atomic_load(flags + kFlagBaseWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -295,6 +297,7 @@ __device__ __forceinline__ void sync_end(Sync &sy, int num_layers) {
 // This workgroup's items of a phase are written: publish.
 __device__ __forceinline__ void publish(const Sync &sy, unsigned seq) {
   wait_vmcnt<0>();                               // this wave's write-through stores are acknowledged
+  strict_release(sy.strict);
   __builtin_amdgcn_s_barrier();                  // ... and every wave's
   compiler_fence();
   if (threadIdx.x < kCopyBlocks)
@@ -325,6 +328,7 @@ __device__ __forceinline__ void await_words(Sync &sy, const unsigned *words, uns
   if (sy.trace && slot < sy.trace_cap && threadIdx.x == 64) sy.trace[(size_t)(2 * sy.trace_cap + 8 * slot + 5) * gridDim.x + blockIdx.x] = wall_clock64();
 #endif
   __builtin_amdgcn_s_barrier();
+  strict_acquire(sy.strict);
   asm volatile("" ::: "memory");
 }
 // The calling WAVE alone waits for the workgroups named by its `mask` (4 per lane): for what only this wave reads.  No
@@ -348,6 +352,7 @@ __device__ __forceinline__ void await_wave(Sync &sy, unsigned mask, unsigned seq
     }
   }
   stamp_wait(sy, slot, 1);
+  strict_acquire(sy.strict);
   compiler_fence();
 }
 // ... the workgroups named by `mask` (4 per lane) have published `seq`
@@ -862,6 +867,7 @@ __device__ __forceinline__ void attn_item_split(unsigned char *lds, const AttnAr
 struct Args {
   int B, S, M, act, num_layers;
   int packed;                          // every layer has w_fc2p: FC2 runs in its whole-K form
+  int strict;                          // souffle_set_strict_fences
   float scale, eps;
   const half_t *x, *mask;
   half_t *y;
@@ -1223,6 +1229,7 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       st16<true>(j.aux, off, __builtin_bit_cast(u4, lo));
       st16<true>(j.aux, off + 16, __builtin_bit_cast(u4, hi));
       wait_all_memory();
+      strict_release(a.strict != 0);
       __syncthreads();
       unsigned *ticket_lds = reinterpret_cast<unsigned *>(lds + kTicketOff);
       unsigned ticket = 0;
@@ -1235,6 +1242,7 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       const bool last = (*ticket_lds & 3u) == 3u;
       compiler_fence();
       if (!last) return;
+      strict_acquire(a.strict != 0);
       f4 slo = {0.f, 0.f, 0.f, 0.f}, shi = {0.f, 0.f, 0.f, 0.f};
       u4 plo[4], phi[4];
 #pragma unroll
@@ -1252,6 +1260,7 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       finish_row(row, col0, slo, shi, res, ns);
       if (sy) {
         wait_all_memory();
+        strict_release(a.strict != 0);
         __syncthreads();
         if (tid < kCopyBlocks)
           __hip_atomic_store(a.flags + tid * kBlockWords + kBlockTileWord + d.a * 12 + ns, phase_seq(*sy, l, PH_RED), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1326,6 +1335,7 @@ __global__ void __launch_bounds__(256) k_encoder_small(Args args) {
   const Shape sh{args.B, args.S, args.M, args.M / 32, (int)gridDim.x, args.packed};
   Sync sy;
   sync_begin(sy, args.flags, args.ctl + kCtlErrWord, args.trace, args.trace_cap);
+  sy.strict = args.strict != 0;
   const unsigned masks_key = mask_key(sh.B, sh.S, sh.G, sh.packed);
   const bool masks_kept = __hip_atomic_load(args.flags + kMaskKeyWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == masks_key;
   if (!masks_kept) sy.key = masks_key;      // (every workgroup: the one that ends last stores the key, and it may be one without items)

@@ -245,8 +245,22 @@ constexpr bool ctl_words_distinct() {
 static_assert(ctl_words_distinct(), "two words of the control block share a place");
 constexpr int kMaxBarrierSpin = 1 << 20;       // about a second of polling; a barrier normally completes in microseconds
 
+// The hand-overs of this library rest on write-through (sc1) stores that are acknowledged before a flag is stored, and
+// on sc1 loads behind the poll (served by the L2, never by a stale L1 line).  The memory model's own form is an
+// agent-scope release fence in front of the flag store and an agent-scope acquire fence behind the poll (an L2
+// write-back and an L1/L2 invalidation per hand-over: measured at 14 us each, against 2).  `strict` switches them on
+// in every hand-over (souffle_set_strict_fences): for a driver or part whose caches might behave differently, and
+// for the test that requires both forms to give the same bits.
+__device__ __forceinline__ void strict_release(bool strict) {
+  if (strict) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+}
+__device__ __forceinline__ void strict_acquire(bool strict) {
+  if (strict) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+
 struct GridBarrier {
   unsigned *ctl;
+  bool strict;       // release / acquire fences of the memory model around every hand-over (see strict_release)
   unsigned target;   // value this workgroup's arrival counter holds once its XCD is complete
   unsigned gsz;      // workgroups that share this workgroup's counter
   unsigned epoch;    // number of the last barrier passed
@@ -273,8 +287,9 @@ __device__ __forceinline__ void trace_mark(const GridBarrier &b, int id) {
 #define STAGE_MARK(tb, id) do { (void)(tb); } while (0)
 #endif
 
-__device__ __forceinline__ void grid_barrier_begin(GridBarrier &b, unsigned *ctl) {
+__device__ __forceinline__ void grid_barrier_begin(GridBarrier &b, unsigned *ctl, bool strict = false) {
   b.ctl = ctl;
+  b.strict = strict;
   b.nblk = gridDim.x;
   b.count = 0;
   b.failed = false;
@@ -316,6 +331,7 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b, Mid mid) {
   const bool tr = b.trace && b.trace_idx < b.trace_cap && threadIdx.x == 0;
   if (tr) b.trace[(size_t)(2 * b.trace_idx) * b.nblk + blockIdx.x] = wall_clock64();
   wait_all_memory();                       // write-through stores are acknowledged
+  strict_release(b.strict);
   __builtin_amdgcn_s_barrier();
   compiler_fence();
 #ifdef SOUFFLE_STAGE_MARKS
@@ -347,6 +363,7 @@ __device__ __forceinline__ void grid_sync(GridBarrier &b, Mid mid) {
   if (tr) b.trace[(size_t)(2 * b.trace_idx + 1) * b.nblk + blockIdx.x] = wall_clock64();
   b.trace_idx++;
   __builtin_amdgcn_s_barrier();            // no memory wait here: loads queued by mid() may still be in flight
+  strict_acquire(b.strict);
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   compiler_fence();                        // no load of what the other workgroups wrote is scheduled above the poll
 }

@@ -26,6 +26,10 @@ int device_facts(DeviceFacts *out);
 // 1: the Swin block pair runs four workgroups per window (souffle_set_swin_split / SOUFFLE_SWIN_SPLIT).
 int swin_split_mode();
 
+// 1: every hand-over between workgroups also runs the release / acquire fences of the memory model
+// (souffle_set_strict_fences / SOUFFLE_STRICT_FENCES).
+int strict_fences_mode();
+
 // Process-wide stage-trace buffer set by souffle_set_stage_trace (NULL = tracing off).
 void stage_trace(unsigned long long **buf, int *max_barriers, int nblk);
 

@@ -32,6 +32,7 @@ struct Args {
   float *y;
   u2 *hbuf;          // [layers][timesteps][256] of (value bits, step tag)
   unsigned *ctl;     // grid-barrier control block; word kCtlErrWord = sticky error flag
+  int strict;        // souffle_set_strict_fences (the grid barrier at the end; the step tags travel with their values)
 };
 
 __device__ __forceinline__ float sigmoidf_(float v) { return 1.0f / (1.0f + __expf(-v)); }
@@ -47,7 +48,7 @@ __global__ void __launch_bounds__(256) k_lstm(Args a) {
   const int slot = a.gate_order == SOUFFLE_GATES_IFGO ? k : (k == 1 ? 2 : (k == 2 ? 1 : k));
 
   GridBarrier bar;
-  grid_barrier_begin(bar, a.ctl);
+  grid_barrier_begin(bar, a.ctl, a.strict != 0);
 
   // weights of this lane: row (l, slot, unit), columns 32j + 8c .. +7 of [W_ih | W_hh]
   u4 w[16];
@@ -172,6 +173,7 @@ extern "C" int souffle_lstm_fused(const souffle_lstm_cfg *cfg, const void *w_ih,
   a.w_ih = static_cast<const half_t *>(w_ih); a.w_hh = static_cast<const half_t *>(w_hh);
   a.bias = bias; a.x = x; a.y = y;
   a.ctl = static_cast<unsigned *>(ws);
+  a.strict = strict_fences_mode();
   a.hbuf = reinterpret_cast<u2 *>(static_cast<char *>(ws) + round_up(kCtlWords * 4, 256));
   void *args[] = {&a};
   return launch_persistent((const void *)lstm::k_lstm, grid, 256, args, 0, static_cast<hipStream_t>(stream));

@@ -57,6 +57,7 @@ struct Block {
 
 struct Args {
   int nblk, stage_begin, stage_end, trace_cap;
+  int strict;                    // souffle_set_strict_fences
   unsigned *ctl;
   unsigned long long *trace;     // optional stage stamps (souffle_set_stage_trace)
   Block blk[MAX_BLOCKS];
@@ -520,7 +521,7 @@ __global__ void __launch_bounds__(256) k_mbconv(const Args a) {
   __shared__ u4 slab[1024];
   __shared__ float r_s[MAX_R];
   GridBarrier bar;
-  grid_barrier_begin(bar, a.ctl);
+  grid_barrier_begin(bar, a.ctl, a.strict != 0);
   bar.trace = a.trace;
   bar.trace_cap = a.trace_cap;
   for (int st = a.stage_begin; st < a.stage_end; ++st) {
@@ -666,6 +667,7 @@ extern "C" int souffle_mbconv_stack(const souffle_mbconv_block *blocks, int num_
     mbconv::Args a;
     a.nblk = n;
     a.ctl = static_cast<unsigned *>(ws);
+    a.strict = strict_fences_mode();
     a.trace = nullptr; a.trace_cap = 0;
     if (fused) stage_trace(&a.trace, &a.trace_cap, grid);
     for (int i = 0; i < n; ++i) {

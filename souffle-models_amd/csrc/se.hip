@@ -23,6 +23,7 @@ struct Args {
   const float *x, *w_reduce, *b_reduce, *w_expand, *b_expand;
   float *y, *pooled, *part;
   unsigned *ctl;
+  int strict;        // souffle_set_strict_fences
 };
 
 __global__ void __launch_bounds__(256) k_se(Args a) {
@@ -33,7 +34,7 @@ __global__ void __launch_bounds__(256) k_se(Args a) {
   const int gw = blockIdx.x * 4 + wave, nw = gridDim.x * 4;
   const int units = a.C * a.chunks, slice = (a.HW + a.chunks - 1) / a.chunks;
   GridBarrier bar;
-  grid_barrier_begin(bar, a.ctl);
+  grid_barrier_begin(bar, a.ctl, a.strict != 0);
 
   float v[UPW][EPT];
 #pragma unroll
@@ -176,7 +177,7 @@ extern "C" int souffle_se_module_fused(const float *x, const float *w_reduce, co
   if (int rc = se::plan(C, HW, R, df.num_cus, &chunks)) return rc;
   if ((long long)C * chunks > 4096) return fail(SOUFFLE_ERR_SHAPE, "too many (channel, chunk) units");
   se::Args a{C, HW, R, chunks, combine, x, w_reduce, b_reduce, w_expand, b_expand, y, pooled,
-             reinterpret_cast<float *>(static_cast<char *>(ws) + round_up(kCtlWords * 4, 256)), static_cast<unsigned *>(ws)};
+             reinterpret_cast<float *>(static_cast<char *>(ws) + round_up(kCtlWords * 4, 256)), static_cast<unsigned *>(ws), strict_fences_mode()};
   void *args[] = {&a};
   return launch_persistent((const void *)se::k_se, df.num_cus, 256, args, 0, static_cast<hipStream_t>(stream));
 }

@@ -36,6 +36,7 @@ struct Args {
   half_t *xctx;                // quad kernel: [window][64][C] attention output, a head's columns written by its workgroup
   float *xpart;                // quad kernel: [window][head][64][C] fp32 FC2 partial sums
   unsigned *xflags;            // quad kernel: [window][16] hand-over words (4 used)
+  int strict;                  // souffle_set_strict_fences
   BlockW w[2];
 };
 
@@ -390,7 +391,7 @@ __device__ void block_for_window(unsigned char *lds, WeightRing &ring, const Arg
 __global__ void __launch_bounds__(256) k_block_pair(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   GridBarrier bar;
-  grid_barrier_begin(bar, a.ctl);
+  grid_barrier_begin(bar, a.ctl, a.strict != 0);
   WeightRing ring{lds + OFF_RING, lds_address(lds + OFF_RING), 0, 0};
   const int nwin = (a.Hh / WS) * (a.Ww / WS), step = gridDim.x;
   if ((int)blockIdx.x >= nwin) {
@@ -494,8 +495,9 @@ __device__ __forceinline__ void qchunk_mma(const unsigned char *buf, const half_
 }
 // This workgroup's data of a hand-over are written: publish `val` in its flag word, then wait until
 // the window's four words have reached it.  Every thread calls it; the wait is bounded.
-__device__ __forceinline__ void quad_handover(unsigned *flags, unsigned *ctl, int win, int h, unsigned val) {
+__device__ __forceinline__ void quad_handover(unsigned *flags, unsigned *ctl, int win, int h, unsigned val, bool strict) {
   wait_all_memory();                             // the write-through stores are acknowledged
+  strict_release(strict);
   __syncthreads();
   if (threadIdx.x == 0) __hip_atomic_store(flags + win * 16 + h, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (threadIdx.x < 64) {
@@ -510,6 +512,7 @@ __device__ __forceinline__ void quad_handover(unsigned *flags, unsigned *ctl, in
     }
   }
   __syncthreads();
+  strict_acquire(strict);
   compiler_fence();                              // no load of the other three workgroups' rows is scheduled above the poll
 }
 
@@ -645,7 +648,7 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
     }
   }
   mark();
-  quad_handover(a.xflags, a.ctl, win, h, fv);
+  quad_handover(a.xflags, a.ctl, win, h, fv, a.strict != 0);
   mark();
   for (int idx = tid; idx < NP * (C / 8); idx += 256) {
     const int r = idx / (C / 8), c8 = idx % (C / 8);
@@ -700,7 +703,7 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
       st16<true>(a.xpart, (((win * NH + h) * NP + row) * C + nt * QN + j * 16 + g * 4) * 4, __builtin_bit_cast(u4, acc[j]));
   }
   mark();
-  quad_handover(a.xflags, a.ctl, win, h, fv + 1);
+  quad_handover(a.xflags, a.ctl, win, h, fv + 1, a.strict != 0);
   mark();
   // out[:, 32h .. 32h+32) = x1 + b2 + P_0 + P_1 + P_2 + P_3, scattered back to the token rows
   for (int idx = tid; idx < N * (HD / 4); idx += 256) {
@@ -717,7 +720,7 @@ __device__ void block_for_window_quad(unsigned char *lds, WeightRing &ring, cons
 __global__ void __launch_bounds__(256) k_block_pair_quad(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   GridBarrier bar;
-  grid_barrier_begin(bar, a.ctl);
+  grid_barrier_begin(bar, a.ctl, a.strict != 0);
   WeightRing ring{lds + OFF_RING, lds_address(lds + OFF_RING), 0, 0};
   const int nwin = (a.Hh / WS) * (a.Ww / WS), quads = gridDim.x / NH;
   // The hand-over words grow from launch to launch: a launch uses four values above those of the one
@@ -744,13 +747,14 @@ struct FfnArgs {
   half_t *y1, *y2;
   float *part;
   unsigned *ctl;
+  int strict;
 };
 
 __global__ void __launch_bounds__(256) k_ffn(FfnArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   half_t *gl = reinterpret_cast<half_t *>(lds);
   GridBarrier bar;
-  grid_barrier_begin(bar, a.ctl);
+  grid_barrier_begin(bar, a.ctl, a.strict != 0);
   {
     const int tn = a.F / 64, items = (a.M / 64) * tn;
     for (int it = blockIdx.x; it < items; it += gridDim.x)
@@ -822,6 +826,7 @@ extern "C" int souffle_swin_block_pair_fused(const souffle_swin_cfg *cfg, const 
   a.Hh = cfg->height; a.Ww = cfg->width; a.shift = cfg->shift; a.use_mask = cfg->use_shift_mask && cfg->shift > 0; a.eps = cfg->ln_eps;
   a.x = static_cast<const half_t *>(x); a.y = static_cast<half_t *>(y);
   a.ctl = static_cast<unsigned *>(ws);
+  a.strict = strict_fences_mode();
   const swin::PairWs pw = swin::pair_ws(cfg);
   a.mid = reinterpret_cast<half_t *>(static_cast<char *>(ws) + pw.mid);
   a.xctx = reinterpret_cast<half_t *>(static_cast<char *>(ws) + pw.xctx);
@@ -898,7 +903,7 @@ extern "C" int souffle_swin_ffn_fused(const void *x, const void *w1, const void 
   const size_t need = round_up(kCtlWords * 4, 256) + (size_t)splitk * M * K * 4;
   if (!ws || ws_bytes < need) return fail(SOUFFLE_ERR_WORKSPACE, "workspace missing or too small: need %zu bytes", need);
   swin::FfnArgs a{M, K, F, splitk, (const half_t *)x, (const half_t *)w1, (const half_t *)w2, (half_t *)y1, (half_t *)y2,
-                  reinterpret_cast<float *>(static_cast<char *>(ws) + round_up(kCtlWords * 4, 256)), static_cast<unsigned *>(ws)};
+                  reinterpret_cast<float *>(static_cast<char *>(ws) + round_up(kCtlWords * 4, 256)), static_cast<unsigned *>(ws), strict_fences_mode()};
   static bool attr_done = false;
   if (!attr_done) {
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)swin::k_ffn, hipFuncAttributeMaxDynamicSharedMemorySize, swin::Tile::LDS_BYTES));

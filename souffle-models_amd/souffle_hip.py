@@ -81,6 +81,7 @@ SIGNATURES = {
     "souffle_l2_stream_probe": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double), C.c_void_p]),
     "souffle_set_stage_trace": (C.c_int, [C.c_void_p, C.c_size_t]),
     "souffle_set_cooperative_launch": (C.c_int, [C.c_int]),
+    "souffle_set_strict_fences": (C.c_int, [C.c_int]),
     "souffle_workspace_init": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "souffle_workspace_status": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_uint), C.c_int]),
     "souffle_bert_workspace_bytes": (C.c_size_t, [C.POINTER(BertCfg)]),
@@ -210,6 +211,12 @@ def set_swin_split(on):
 def set_cooperative_launch(on):
     """Launch the persistent kernels cooperatively (True) or plainly (False, the default)."""
     check(lib().souffle_set_cooperative_launch(1 if on else 0))
+
+
+def set_strict_fences(on):
+    """Every hand-over between workgroups also runs the memory model's release / acquire fences (True) or rests on
+    acknowledged write-through stores and coherent loads alone (False, the default).  Same results either way."""
+    check(lib().souffle_set_strict_fences(1 if on else 0))
 
 
 def device_info():

@@ -48,7 +48,7 @@ def test_bert_validation_without_gpu():
     assert bytes_for(1, 128, 12) > 11 * (bytes_for(1, 128, 1) - 4096)
     assert bytes_for(32, 128, 12) == bytes_for(32, 128, 1) == n32
     per_row = 2 * (3 * 768 + 768 + 768 + 768 + 3072 + 768) + 4 * 768 * 2     # qkv, ctx, z1, y1, h, layer output; four fp16 partial sums
-    assert 4096 * per_row <= n32 <= 4096 * per_row + (1 << 17)       # (+ control block, flag and completion words)
+    assert 4096 * per_row <= n32 <= 4096 * per_row + (1 << 19)       # (+ control block, flag and completion words, the kept wait masks)
     assert bytes_for(32, 100, 2) > bytes_for(32, 128, 2)                       # padded to 128 inside the call: room for the padded copies
     w = sh.BertLayerW()
     rc = lib.souffle_bert_layer_fused(C.byref(bad), C.byref(w), None, None, None, None, None, 0, None)
