@@ -114,7 +114,10 @@ int souffle_set_strict_fences(int on);
 int souffle_workspace_status(void *workspace, souffle_stream_t stream, unsigned *flags, int clear);
 
 /* ------------------------------------------------------------------ BERT ---- */
-enum { SOUFFLE_ACT_GELU_TANH = 0, SOUFFLE_ACT_RELU = 1 };
+/* GELU_ERF: 0.5 x (1 + erf(x / sqrt 2)), the form that HuggingFace BERT checkpoints (config "gelu") were trained with,
+ * which cpp/bert/test_souffle_bert_layer.py:131-143,161 loads; the reference's own kernels compute the tanh form
+ * (cpp/bert/bert_base_impl.cu:722-734) or ReLU (cpp/bert/kernels/fused_sqq_feedforward.cu:327-341). */
+enum { SOUFFLE_ACT_GELU_TANH = 0, SOUFFLE_ACT_RELU = 1, SOUFFLE_ACT_GELU_ERF = 2 };
 
 typedef struct {
   int batch, seq_len;          /* runtime; seq_len <= 512.  Lengths other than 64/128/256/384/512 run as the next of

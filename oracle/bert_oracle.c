@@ -73,8 +73,15 @@ float oracle_gelu_tanh(float x) {
   return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
 }
 
+/* 0.5 x (1 + erf(x / sqrt 2)): the activation of the HuggingFace BERT checkpoints that
+   cpp/bert/test_souffle_bert_layer.py:131-143,161 loads ("gelu" = torch.nn.functional.gelu's default form) */
+float oracle_gelu_erf(float x) {
+  return (float)(0.5 * (double)x * (1.0 + erf((double)x * 0.70710678118654752440)));
+}
+
 static void apply_act(float *h, size_t n, int act) {
   if (act == ORACLE_ACT_GELU_TANH) { for (size_t i = 0; i < n; ++i) h[i] = oracle_gelu_tanh(h[i]); }
+  else if (act == ORACLE_ACT_GELU_ERF) { for (size_t i = 0; i < n; ++i) h[i] = oracle_gelu_erf(h[i]); }
   else if (act == ORACLE_ACT_RELU) { for (size_t i = 0; i < n; ++i) h[i] = h[i] > 0.f ? h[i] : 0.f; }
 }
 

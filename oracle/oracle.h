@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-enum { ORACLE_ACT_GELU_TANH = 0, ORACLE_ACT_RELU = 1, ORACLE_ACT_NONE = 2 };
+enum { ORACLE_ACT_GELU_TANH = 0, ORACLE_ACT_RELU = 1, ORACLE_ACT_NONE = 2, ORACLE_ACT_GELU_ERF = 3 };
 
 typedef struct {
   int batch, seq_len, hidden, heads, ffn;
@@ -93,6 +93,7 @@ void oracle_gemm_f32(const float *x, const float *w, const float *bias, float *y
 void oracle_layernorm_f32(const float *z, const float *g, const float *b, float *y,
                           int rows, int dim, float eps);
 float oracle_gelu_tanh(float x);
+float oracle_gelu_erf(float x);
 
 /* ---- stacked LSTM ---- */
 enum { ORACLE_GATES_IFGO = 0, ORACLE_GATES_IGFO = 1 };

@@ -12,7 +12,7 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liboracle.so")
-ACT = {"gelu_tanh": 0, "relu": 1, "none": 2}
+ACT = {"gelu_tanh": 0, "relu": 1, "none": 2, "gelu": 3}      # "gelu": the erf form, as in HuggingFace configs
 _lib = None
 
 
@@ -64,6 +64,8 @@ def lib():
         _lib = C.CDLL(LIB_PATH)
         _lib.oracle_gelu_tanh.restype = C.c_float
         _lib.oracle_gelu_tanh.argtypes = [C.c_float]
+        _lib.oracle_gelu_erf.restype = C.c_float
+        _lib.oracle_gelu_erf.argtypes = [C.c_float]
     return _lib
 
 
@@ -108,6 +110,10 @@ def layernorm(z, g=None, b=None, eps=1e-12):
 
 def gelu_tanh(x):
     return np.array([lib().oracle_gelu_tanh(float(v)) for v in np.asarray(x).ravel()], np.float32).reshape(np.shape(x))
+
+
+def gelu_erf(x):
+    return np.array([lib().oracle_gelu_erf(float(v)) for v in np.asarray(x).ravel()], np.float32).reshape(np.shape(x))
 
 
 def bert_layer(x, weights, batch, seq_len, hidden=768, heads=12, ffn=3072, act="gelu_tanh", scale=0.125,

@@ -42,11 +42,10 @@ def _check_f16_cuda(name, t, shape=None):
 
 
 def make_cfg(batch, seq_len, act="gelu_tanh", scale=0.125, ln_eps=1e-12, num_layers=1):
-    acts = {"gelu_tanh": sh.ACT_GELU_TANH, "relu": sh.ACT_RELU}
-    if act == "gelu":
-        # HuggingFace's "gelu" is the erf form; the reference kernel (and this one) computes the tanh form.  The two
-        # differ by up to 5e-4 per activation, so the name is not taken as an alias.
-        raise ValueError("act='gelu' (the erf form) is not built: the reference computes the tanh form, pass act='gelu_tanh'")
+    # "gelu" is HuggingFace's name for the erf form, which its BERT checkpoints were trained with; the reference's
+    # kernels compute the tanh form ("gelu_tanh", the default here) or ReLU.  The two GELUs differ by up to 5e-4 per
+    # activation, so neither name is an alias of the other.
+    acts = {"gelu_tanh": sh.ACT_GELU_TANH, "relu": sh.ACT_RELU, "gelu": sh.ACT_GELU_ERF}
     if act not in acts:
         raise ValueError("act must be one of %s" % sorted(acts))
     return sh.BertCfg(batch, seq_len, HIDDEN, HEADS, FFN, acts[act], float(scale), float(ln_eps), num_layers, 0)

@@ -123,6 +123,9 @@ __device__ __forceinline__ void stage_fc1(half_t *lds, const Params &a, const La
       if (a.act == SOUFFLE_ACT_RELU) {            // (one test per group of results, not one per result)
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = fmaxf(v[i], 0.f);
+      } else if (a.act == SOUFFLE_ACT_GELU_ERF) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = gelu_erf(v[i]);
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = gelu_tanh(v[i]);
@@ -310,10 +313,17 @@ __device__ __forceinline__ void big_fc1(unsigned char *lds, const Params &a, con
       for (int i = 0; i < 4; ++i) v[i] = gelu_tanh(v[i]);
       return pack_h4(v);
     };
+    auto cvt_erf = [&](int, int, f4 v, h4 bb) {
+      v += f4{(float)bb[0], (float)bb[1], (float)bb[2], (float)bb[3]};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = gelu_erf(v[i]);
+      return pack_h4(v);
+    };
     auto store16 = [&](int m, int nr, u4 v) { st16<COH>(a.h, (m * F + n0 + nr) * 2, v); };
     f4 acc[BigFc1::MI][BigFc1::NT];
     BigFc1::mainloop<H / 32>(lds, a.y1, H, tm * 256, 0, wptr, acc, tb);
     if (a.act == SOUFFLE_ACT_RELU) BigFc1::epilogue_rowvec(lds, tm * 256, acc, bias_at, cvt_relu, store16, tb);
+    else if (a.act == SOUFFLE_ACT_GELU_ERF) BigFc1::epilogue_rowvec(lds, tm * 256, acc, bias_at, cvt_erf, store16, tb);
     else BigFc1::epilogue_rowvec(lds, tm * 256, acc, bias_at, cvt_gelu, store16, tb);
   }
 }
@@ -934,7 +944,7 @@ static int validate(const souffle_bert_cfg *c) {
   const long long m = (long long)c->batch * s;
   if (m >= 1536 && m % 128 != 0) return fail(SOUFFLE_ERR_SHAPE, "batch*seq_len >= 1536 must be a multiple of 128 (got %lld)", m);
   if (m > 65536) return fail(SOUFFLE_ERR_SHAPE, "batch*seq_len must be <= 65536 (got %lld)", m);
-  if (c->act != SOUFFLE_ACT_GELU_TANH && c->act != SOUFFLE_ACT_RELU) return fail(SOUFFLE_ERR_SHAPE, "unknown activation %d", c->act);
+  if (c->act != SOUFFLE_ACT_GELU_TANH && c->act != SOUFFLE_ACT_RELU && c->act != SOUFFLE_ACT_GELU_ERF) return fail(SOUFFLE_ERR_SHAPE, "unknown activation %d", c->act);
   if (!(c->ln_eps >= 0.f)) return fail(SOUFFLE_ERR_SHAPE, "ln_eps must be >= 0");
   return SOUFFLE_OK;
 }

@@ -1207,6 +1207,9 @@ __device__ __forceinline__ void run_gemm_item_t(unsigned char *lds, const Args &
       if (a.act == SOUFFLE_ACT_RELU) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) { lo[i] = fmaxf(lo[i], 0.f); hi[i] = fmaxf(hi[i], 0.f); }
+      } else if (a.act == SOUFFLE_ACT_GELU_ERF) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { lo[i] = gelu_erf(lo[i]); hi[i] = gelu_erf(hi[i]); }
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i) { lo[i] = gelu_tanh(lo[i]); hi[i] = gelu_tanh(hi[i]); }

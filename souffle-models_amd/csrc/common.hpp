@@ -202,6 +202,9 @@ __device__ __forceinline__ float gelu_tanh(float x) {
   return x - x * __builtin_amdgcn_rcpf(e + 1.0f);
 }
 
+// 0.5 x (1 + erf(x / sqrt 2)): the exact form (library erff; some 30 instructions per value).
+__device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f)); }
+
 // -------------------------------------------------------- grid barrier ----
 // Two kinds of words, never mixed on one cache line:
 //  * arrival counter x (x = workgroup % 8, the XCD the workgroup runs on): incremented with an

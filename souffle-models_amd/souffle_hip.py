@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("SOUFFLE_HIP_LIB") or os.path.join(_HERE, "libsouffle_hip.so")
 
-ACT_GELU_TANH, ACT_RELU = 0, 1
+ACT_GELU_TANH, ACT_RELU, ACT_GELU_ERF = 0, 1, 2
 GATES_IFGO, GATES_IGFO = 0, 1
 SE_MUL, SE_ADD = 0, 1
 

@@ -53,6 +53,20 @@ def test_layer_bias_affine_mask(opt_level, pack):
         assert_close(n, g, r)
 
 
+@pytest.mark.parametrize("B,S,opt_level,pack", [(1, 128, 4, True), (1, 128, 1, False), (2, 256, 4, False), (16, 128, 4, False), (9, 128, 4, True), (13, 128, 4, False)])
+def test_layer_erf_gelu(B, S, opt_level, pack):
+    """The exact (erf) GELU of HuggingFace checkpoints, on the few-rows kernel and on both tile sizes of the many-rows one."""
+    announce("bert layer erf-GELU B=%d S=%d opt=%d pack=%d" % (B, S, opt_level, pack))
+    w, x = synth.bert_layer_weights(0, 3, with_bias=True), synth.bert_input(1, B, S)
+    ref = oracle.bert_layer(x, w, B, S, act="gelu", dump=True)
+    got = run_layer(w, x, B, S, opt_level, act="gelu", pack=pack)
+    for n, g, r in zip(NAMES, got, ref):
+        assert_close(n, g, r)
+    # ... and it is not the tanh form: the FC1 outputs of the two differ where the oracle's do
+    tanh_form = run_layer(w, x, B, S, opt_level, pack=pack)[4]
+    assert not torch.equal(tanh_form, got[4])
+
+
 def test_layer_reference_compat_mode():
     """What the reference's fused CUDA path computes: ReLU, scale 1/sqrt(768), eps 1e-5."""
     announce("bert layer reference-compat")

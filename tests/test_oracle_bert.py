@@ -61,7 +61,23 @@ def test_gelu_tanh_closed_form():
     assert abs(oracle.gelu_tanh([10.0])[0] - 10.0) < 1e-5 and abs(oracle.gelu_tanh([-10.0])[0]) < 1e-5
 
 
-@pytest.mark.parametrize("act,scale,eps", [("gelu_tanh", 0.25, 1e-12), ("relu", 1 / 64 ** 0.5, 1e-5)])
+def test_gelu_erf_closed_form():
+    """The exact GELU against torch's library routine in float64, against math.erf at points whose erf is known to many
+    digits, and apart from the tanh form where the two differ most."""
+    import math
+    xs = np.array([-6.0, -2.0, -1.0, -0.5, 0.0, 0.5, 1.0, 2.0, 3.0, 8.0])
+    ref = torch.nn.functional.gelu(torch.from_numpy(xs)).numpy()
+    np.testing.assert_allclose(oracle.gelu_erf(xs), ref, rtol=1e-6, atol=1e-7)
+    for x in (0.3, 1.0, 1.7, -0.9):
+        assert abs(oracle.gelu_erf([x])[0] - 0.5 * x * (1.0 + math.erf(x / math.sqrt(2.0)))) < 1e-6
+    assert abs(oracle.gelu_erf([math.sqrt(2.0)])[0] - 0.5 * math.sqrt(2.0) * (1.0 + 0.8427007929497149)) < 1e-6      # erf(1)
+    assert oracle.gelu_erf([0.0])[0] == 0.0
+    assert abs(oracle.gelu_erf([10.0])[0] - 10.0) < 1e-6 and abs(oracle.gelu_erf([-10.0])[0]) < 1e-6
+    d = np.abs(oracle.gelu_erf(np.linspace(-4, 4, 801)) - oracle.gelu_tanh(np.linspace(-4, 4, 801)))
+    assert 1e-4 < d.max() < 1e-3                      # two different functions, up to about 5e-4 apart
+
+
+@pytest.mark.parametrize("act,scale,eps", [("gelu_tanh", 0.25, 1e-12), ("relu", 1 / 64 ** 0.5, 1e-5), ("gelu", 0.125, 1e-12)])
 def test_small_layer_matches_torch_all_stages(act, scale, eps):
     B, S, H, nh, F = 2, 16, 64, 4, 128
     rng = np.random.default_rng(3)

@@ -41,7 +41,7 @@ def bert_layer(x, w, batch, seq_len, heads, act="gelu_tanh", scale=0.125, ln_eps
     h = y1 @ g("fc1_weight")
     if g("fc1_bias") is not None:
         h = h + g("fc1_bias")
-    h = Fn.gelu(h, approximate="tanh") if act == "gelu_tanh" else torch.relu(h)
+    h = Fn.gelu(h, approximate="tanh") if act == "gelu_tanh" else (Fn.gelu(h) if act == "gelu" else torch.relu(h))
     z2 = h @ g("fc2_weight")
     if g("fc2_bias") is not None:
         z2 = z2 + g("fc2_bias")
