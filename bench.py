@@ -12,6 +12,7 @@ Infinity Cache.  Prints ONE JSON line.
 """
 import argparse
 import json
+import re
 import os
 import sys
 import time
@@ -41,6 +42,7 @@ def parse():
     p.add_argument("--no-cpu", action="store_true")
     p.add_argument("--no-sub", action="store_true", help="skip the sub-results of the default workload (S=384, B=32, LSTM, Swin, SE, MBConv)")
     p.add_argument("--no-coop", action="store_true", help="skip the cooperative-launch timing of the encoder workloads")
+    p.add_argument("--no-strict", action="store_true", help="skip the strict-fence timing of the encoder workloads")
     p.add_argument("--weight-sets", type=int, default=4)
     p.add_argument("--no-pack", action="store_true", help="encoders keep the [K][N] FC2 matrices only (split-K FC2) instead of packing them once")
     return p.parse_args()
@@ -268,6 +270,8 @@ def bench_encoder(args, B, S, L, name):
     # the same launch with the memory model's release / acquire fences around every hand-over (souffle_set_strict_fences):
     # the by-the-book form, same bits (tests/test_strict_fences.py), kept as a fallback
     try:
+        if args.no_strict:
+            raise sh.SouffleError(0, "skipped (--no-strict)")
         sh.set_strict_fences(True)
         _, strict_ev = time_steps(lambda i: encs[i % len(encs)](x, out=out), max(10, args.steps // 4), 3)
         res["extra"]["strict_fences_us"] = strict_ev * 1e3
@@ -305,6 +309,10 @@ def main():
     elif args.workload == "encoder_b32":
         args.weight_sets = 1
         res = bench_encoder(args, 32, 128, 12, "BERT-base 12-layer encoder, B=32, S=128, fp16 (MFMA-bound shape)")
+    elif re.fullmatch(r"encoder_b(\d+)_s(\d+)", args.workload):
+        # any other shape of the 12-layer encoder (development aid: the bench lines of record are the named workloads)
+        B, S = (int(v) for v in re.fullmatch(r"encoder_b(\d+)_s(\d+)", args.workload).groups())
+        res = bench_encoder(args, B, S, 12, "BERT-base 12-layer encoder, B=%d, S=%d, fp16" % (B, S))
     elif args.workload == "copy":
         # A plain device copy of known size: the calibration run for the FETCH_SIZE / WRITE_SIZE
         # counters (counter reading per byte actually read / written).
