@@ -83,15 +83,18 @@ int souffle_workspace_init(void *workspace, size_t workspace_bytes, souffle_stre
  * buf[(2*cap + 8*i + id) * grid + block].  Pass NULL to switch tracing off (the default). */
 int souffle_set_stage_trace(void *device_buf, size_t bytes);
 
-/* How the persistent (grid-barrier) kernels are launched.  The reference launches its fused
- * kernels with cudaLaunchCooperativeKernel (cpp/swin_transformer/swin_transformer_binding.cu:95,
- * cpp/efficientnet/efficientnet_se_module_main.cu:62).  On MI355X a cooperative launch costs
- * ~20 us against ~4 us for a plain one, which is most of a 30 us encoder layer, so the default
- * (on = 0) is a plain launch of a grid that the occupancy query has shown to be co-resident on
- * an otherwise idle device.  Fused calls must then not overlap in time with other fused calls
- * on another stream (two half-resident grids would wait for each other until the bounded
- * barrier spin gives up and the call's output is invalid).  on = 1 restores the runtime's
- * guarantee.  The environment variable SOUFFLE_COOPERATIVE_LAUNCH=1 sets the initial value. */
+/* How the persistent kernels (those whose workgroups wait for one another: grid barriers, flag hand-overs) are
+ * launched.  The reference launches its fused kernels with cudaLaunchCooperativeKernel
+ * (cpp/swin_transformer/swin_transformer_binding.cu:95, cpp/efficientnet/efficientnet_se_module_main.cu:62).
+ * On MI355X a cooperative launch costs about 13 us more than a plain one (282 against 269 us for the 12-layer
+ * encoder at B=1, S=128), so the default (on = 0) is a plain hipLaunchKernel of a grid that the occupancy query has
+ * shown to fit the device at once.  Precondition of that default: the device runs nothing else while a fused call
+ * runs.  Fused calls must not overlap in time with other kernels on another stream or of another process (two
+ * half-resident grids would wait for each other); every wait in the kernels is bounded, so such a call ends, sets
+ * the sticky failure flag of its workspace and leaves an invalid output: check souffle_workspace_status (or
+ * souffle_bert_static_status) where that cannot be excluded.  on = 1 restores the runtime's guarantee and needs a
+ * device that supports cooperative launches.  The environment variable SOUFFLE_COOPERATIVE_LAUNCH=1 sets the
+ * initial value. */
 int souffle_set_cooperative_launch(int on);
 
 /* The hand-overs between the workgroups of the persistent kernels (flag words of the encoder, grid barriers,
@@ -172,7 +175,8 @@ typedef struct {
 
 size_t souffle_bert_workspace_bytes(const souffle_bert_cfg *cfg);
 
-/* One encoder layer as ONE persistent cooperative launch.
+/* One encoder layer as ONE persistent launch (plain by default, see souffle_set_cooperative_launch for the
+ * launch mode and its precondition; failed waits are reported by souffle_workspace_status).
  * Replaces souffle_bert_layer<1,12,384,64,3072>(..., opt_level=3|4)
  * (cpp/bert/bert_binding.cu:23-535, fused path :395-528).
  * x,y: [B*S][768] fp16; mask: additive fp16 [B][S][S] or NULL. */
@@ -187,8 +191,8 @@ int souffle_bert_layer_unfused(const souffle_bert_cfg *cfg, const souffle_bert_l
                                const void *x, const void *mask, void *y,
                                const souffle_bert_dump *dump,
                                void *workspace, size_t workspace_bytes, souffle_stream_t stream);
-/* cfg->num_layers layers with distinct weights in one cooperative launch /
- * as per-op launches.  Replaces souffle_bert_base() (cpp/bert/bert_base_impl.cu:277-308,590-678). */
+/* cfg->num_layers layers with distinct weights in one persistent launch (launch mode and precondition as for
+ * souffle_bert_layer_fused) / as per-op launches.  Replaces souffle_bert_base() (cpp/bert/bert_base_impl.cu:277-308,590-678). */
 int souffle_bert_encoder_fused(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
                                const void *x, const void *mask, void *y,
                                void *workspace, size_t workspace_bytes, souffle_stream_t stream);
@@ -203,10 +207,18 @@ int souffle_bert_encoder_unfused(const souffle_bert_cfg *cfg, const souffle_bert
  * harnesses that forbid hipMalloc.  Same results as souffle_bert_encoder_fused.  A configuration whose
  * workspace (souffle_bert_workspace_bytes) exceeds the array is refused with SOUFFLE_ERR_WORKSPACE
  * (12 layers fit at up to 128 rows, fewer layers at more).  Every call on a GPU uses that GPU's one
- * array: calls that overlap on one GPU (two streams, two threads) race, and the sticky failure word of
- * the bounded waits cannot be read back through this entry point. */
+ * array: calls that overlap on one GPU (two streams, two threads) race.  Nothing is cleared between calls (the
+ * array starts as zeros when the library is loaded; flag values only grow from call to call), so the same work
+ * is enqueued whatever was called before.  Under graph capture: make one eager call of the same configuration
+ * first (the first call on a device looks the array's address up, and the first call of a kernel variant sets
+ * its LDS size and asks the occupancy query, which are not stream work), and replay the graph only while
+ * nothing else uses the array.  The sticky failure word of the bounded waits is read with
+ * souffle_bert_static_status. */
 int souffle_bert_encoder_fused_static(const souffle_bert_cfg *cfg, const souffle_bert_layer_w *layers,
                                       const void *x, const void *mask, void *y, souffle_stream_t stream);
+/* souffle_workspace_status for the array of souffle_bert_encoder_fused_static on the current device (waits for
+ * `stream`; allocates nothing).  No counterpart in the reference; for the same callers. */
+int souffle_bert_static_status(souffle_stream_t stream, unsigned *flags, int clear);
 
 /* The work split and the hand-over plan of the encoder at few rows (up to 1024, and below 1536 where the count is
  * no multiple of 256), evaluated on the host by the functions the

@@ -1262,8 +1262,7 @@ static int run_fused(const souffle_bert_cfg *c, const souffle_bert_layer_w *laye
   if (int rc = validate(c)) return rc;
   DeviceFacts df;
   if (int rc = device_facts(&df)) return rc;
-  if (!df.cooperative) return fail(SOUFFLE_ERR_DEVICE, "device does not support cooperative launch");
-  const Plan p = make_plan(c, nl);
+  const Plan p = make_plan(c, nl);      // (cooperative-launch support is asked for by the launch itself, and only in that mode)
   Padded pd;
   if (int rc = pad_before(pd, c, x_in, mask_in, y_out, dump, ws, ws_bytes, p, df.num_cus, static_cast<hipStream_t>(stream))) return rc;
   if (pd.on) {
@@ -1387,28 +1386,23 @@ constexpr size_t kStaticScratchBytes = (size_t)48 << 20;      // 12 layers at 12
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 // Device memory of `scratch` on the current device, looked up once per device (each device has its own copy of the
-// array at its own address; the array's name in host code is a stand-in, not an address), and the configuration of
-// the last call that used it there.
-struct StaticScratch { unsigned char *ptr; size_t cleared_for; };
-static int static_scratch(StaticScratch **out) {
+// array at its own address; the array's name in host code is a stand-in, not an address).
+static int static_scratch(unsigned char **out) {
   constexpr int kMaxDevices = 64;
-  static StaticScratch per_device[kMaxDevices] = {};
+  static unsigned char *per_device[kMaxDevices] = {};
   static std::mutex mu;
   int dev = -1;
   SOUFFLE_HIP_TRY(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices) return fail(SOUFFLE_ERR_DEVICE, "device index %d is not supported", dev);
   std::lock_guard<std::mutex> lk(mu);
-  if (!per_device[dev].ptr) {
+  if (!per_device[dev]) {
     void *p = nullptr;
     SOUFFLE_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
     if (!p) return fail(SOUFFLE_ERR_DEVICE, "the library's static scratch has no address on device %d", dev);
-    per_device[dev].ptr = static_cast<unsigned char *>(p);
+    per_device[dev] = static_cast<unsigned char *>(p);
   }
-  *out = &per_device[dev];
+  *out = per_device[dev];
   return SOUFFLE_OK;
-}
-__global__ void __launch_bounds__(256) k_clear16(u4 *p, int n16) {
-  for (int i = blockIdx.x * 256 + threadIdx.x; i < n16; i += gridDim.x * 256) p[i] = u4{0u, 0u, 0u, 0u};
 }
 }  // namespace bert
 }  // namespace souffle
@@ -1423,19 +1417,19 @@ extern "C" int souffle_bert_encoder_fused_static(const souffle_bert_cfg *cfg, co
   if (p.total > bert::kStaticScratchBytes)
     return fail(SOUFFLE_ERR_WORKSPACE, "batch %d x seq_len %d x %d layers needs %zu bytes of scratch, the library's static scratch holds %zu: "
                 "use souffle_bert_encoder_fused with a workspace", cfg->batch, cfg->seq_len, nl, p.total, bert::kStaticScratchBytes);
-  bert::StaticScratch *sc = nullptr;
+  unsigned char *sc = nullptr;
   if (int rc = bert::static_scratch(&sc)) return rc;
-  // The control block and the flag words (the first bytes, at the same place for every configuration) must start from
-  // zero when the layout behind them changes: they hold the previous call's barrier counts and flag values.  Between
-  // calls of one configuration they carry over, as in a caller's workspace.  A fill kernel, not a memset node.
-  const size_t key = ((size_t)cfg->batch << 40) ^ ((size_t)cfg->seq_len << 20) ^ (size_t)nl ^ ((size_t)1 << 62);
-  if (sc->cleared_for != key) {
-    const int n16 = (int)(p.off_qkv / 16);
-    hipLaunchKernelGGL(bert::k_clear16, dim3((n16 + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), reinterpret_cast<u4 *>(sc->ptr), n16);
-    SOUFFLE_HIP_TRY(hipGetLastError());
-    sc->cleared_for = key;
-  }
-  return bert::run_fused(cfg, layers, nl, x, mask, y, nullptr, sc->ptr, bert::kStaticScratchBytes, stream);
+  // Nothing is cleared between calls, whatever their configurations: the array starts as zeros when the library is
+  // loaded, like a workspace after souffle_workspace_init; from then on the control block and the flag words (the first
+  // bytes, at the same place for every configuration) carry over from call to call as they do in a caller's workspace
+  // that serves several shapes: sequence numbers only grow, and the kept wait masks are keyed by the shape.  So the same
+  // work is enqueued whether or not earlier calls were made: what a graph capture records does not depend on history.
+  return bert::run_fused(cfg, layers, nl, x, mask, y, nullptr, sc, bert::kStaticScratchBytes, stream);
+}
+extern "C" int souffle_bert_static_status(souffle_stream_t stream, unsigned *flags, int clear) {
+  unsigned char *sc = nullptr;
+  if (int rc = bert::static_scratch(&sc)) return rc;
+  return souffle_workspace_status(sc, stream, flags, clear);
 }
 
 // w_fc2 [3072][768] -> 48 slices of 16 output columns, each 96 k-steps of 1 KB: lane L of a wave finds the eight

@@ -6,18 +6,23 @@
 //   ATT  (head, 16 queries)                       scores, softmax and P.V; keys split over the waves
 //   OUT  (m-tile, 64 of 768 columns)              z1 = ctx.Wo + b + x, fp16, plus row statistics of its 64 columns
 //   FC1  (m-tile, 64 of 3072 columns)             h = act(LN1(z1).W1 + b)
-//   FC2  (m-tile, 64 of 768 columns, K quarter)   fp32 partial sum; the last of a tile's four workgroups to finish adds
-//                                                 the four, the bias and LN1(z1): z2, fp16, plus row statistics
-// and after the last layer FIN (m-tile, 64 columns): y = LN2(z2).  (PH_RED names the completion of that sum: it has a
-// sequence number, which the completion words of the tiles carry, but no items of its own.)
+//   FC2  in one of two forms:
+//        whole-K (every layer has the packed copy of its W2, souffle_bert_pack_fc2): (m-tile, 16 of 768 columns) over all
+//          of K = 3072; the workgroup finishes its rows itself: z2 = sum + bias + LN1(z1), fp16, plus the statistics of
+//          its 16 columns.  h is written by FC1 in the order the MFMA reads it, so that it goes straight to registers.
+//        split-K ([K][N] weights only): (m-tile, 64 of 768 columns, K quarter), fp32 partial sums through memory; the
+//          last of a tile's four workgroups to finish adds the four, the bias and LN1(z1), and sets the tile's
+//          completion word (PH_RED names that completion: it has a sequence number but no items of its own).
+// and after the last layer FIN (m-tile, 64 columns): y = LN2(z2).
 //
 // There is no grid barrier.  A workgroup that has finished its items of a phase waits for the acknowledgement of
 // its write-through stores and publishes the number of that phase in its flag word; a consumer polls the flag
 // words of exactly the workgroups that produce what its items read (9 to 48 of them; which ones follows from the
-// item numbering and is worked out once per launch; the consumers of the FC2 sum poll one completion word per
-// 32 x 64 tile instead, written by whichever workgroup summed the tile).  Flag words exist in eight copies, one per XCD, so that a
-// line is polled by the 32 workgroups of one XCD only: measured 1.65 us per hand-over against 2.25 us for the
-// grid barrier with per-XCD counters, 3.8 us with a single copy.
+// item numbering, is worked out by the first launch of a shape and kept in the workspace for the later ones).  In the
+// whole-K form each WAVE of an FC2 workgroup waits for the FC1 workgroups that wrote its own K quarter of h; in the
+// split-K form the consumers of the FC2 sum poll one completion word per 32 x 64 tile instead.  Flag words exist in
+// 16 copies, two per XCD (see below), so that a line is polled by the 32 workgroups of one XCD only: measured 1.65 us
+// per hand-over against 2.25 us for the grid barrier with per-XCD counters, 3.8 us with a single copy.
 //
 // Memory model of a hand-over (gfx950, one L2 per XCD, one L1 per CU):
 //   producer: data stores with sc1 (write-through to the memory side, which invalidates the copies other L2s hold),
@@ -28,11 +33,12 @@
 // cases where the CU had read the line before, an sc1 load never, and no L2 ever served an old value, neither to
 // plain nor to sc1 loads, within a launch or across launches.  Every load of data that another workgroup of the
 // launch wrote is therefore an sc1 load here.  The release and acquire fences of the compiler's memory model
-// (buffer_wbl2 sc1 / buffer_inv sc1) are not needed on top of that and were measured at 14 us per hand-over.
+// (buffer_wbl2 sc1 / buffer_inv sc1) are not needed on top of that and were measured at 14 us per hand-over; with
+// Args::strict set (souffle_set_strict_fences) every hand-over runs them all the same, as a fallback: same bits.
 //
 // LayerNorm never runs as a pass of its own: producers publish, per row, mean and sum of squared deviations of
-// the 64 columns they wrote; a consumer combines the twelve partials of a row (exact pairwise update, no
-// cancellation) and normalises the operand registers on their way into the MFMA.
+// the columns they wrote (64 for z1: 12 partials per row; 16 for z2: 48); a consumer combines the partials of a row
+// (exact pairwise update, no cancellation) and normalises the operand registers on their way into the MFMA.
 #pragma once
 #include <type_traits>
 #include "bert_defs.hpp"

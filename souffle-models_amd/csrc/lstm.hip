@@ -166,8 +166,8 @@ extern "C" int souffle_lstm_fused(const souffle_lstm_cfg *cfg, const void *w_ih,
   DeviceFacts df;
   if (int rc = device_facts(&df)) return rc;
   const int grid = cfg->layers * lstm::WG_PER_LAYER;
-  if (!df.cooperative || grid > df.num_cus)
-    return fail(SOUFFLE_ERR_DEVICE, "needs a cooperative launch of %d workgroups, device has %d CUs", grid, df.num_cus);
+  if (grid > df.num_cus)
+    return fail(SOUFFLE_ERR_DEVICE, "needs %d workgroups resident at once, device has %d CUs", grid, df.num_cus);
   lstm::Args a;
   a.layers = cfg->layers; a.timesteps = cfg->timesteps; a.gate_order = cfg->gate_order; a.forget_bias = cfg->forget_bias;
   a.w_ih = static_cast<const half_t *>(w_ih); a.w_hh = static_cast<const half_t *>(w_hh);

@@ -172,7 +172,6 @@ extern "C" int souffle_se_module_fused(const float *x, const float *w_reduce, co
   if (!aligned16(ws)) return fail(SOUFFLE_ERR_ALIGN, "workspace must be 16-byte aligned");
   DeviceFacts df;
   if (int rc = device_facts(&df)) return rc;
-  if (!df.cooperative) return fail(SOUFFLE_ERR_DEVICE, "device does not support cooperative launch");
   int chunks = 0;
   if (int rc = se::plan(C, HW, R, df.num_cus, &chunks)) return rc;
   if ((long long)C * chunks > 4096) return fail(SOUFFLE_ERR_SHAPE, "too many (channel, chunk) units");

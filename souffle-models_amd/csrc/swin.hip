@@ -848,7 +848,6 @@ extern "C" int souffle_swin_block_pair_fused(const souffle_swin_cfg *cfg, const 
   }
   DeviceFacts df;
   if (int rc = device_facts(&df)) return rc;
-  if (!df.cooperative) return fail(SOUFFLE_ERR_DEVICE, "device does not support cooperative launch");
   static bool attr_done = false;
   if (!attr_done) {
     SOUFFLE_HIP_TRY(hipFuncSetAttribute((const void *)swin::k_block_pair, hipFuncAttributeMaxDynamicSharedMemorySize, swin::LDS_BYTES));

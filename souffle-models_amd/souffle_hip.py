@@ -95,6 +95,7 @@ SIGNATURES = {
                                                C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "souffle_bert_encoder_fused_static": (C.c_int, [C.POINTER(BertCfg), C.POINTER(BertLayerW), C.c_void_p, C.c_void_p,
                                                     C.c_void_p, C.c_void_p]),
+    "souffle_bert_static_status": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint), C.c_int]),
     "souffle_bert_polled_copies": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p]),
     "souffle_bert_handover_plan": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "souffle_bert_fc2_packed_bytes": (C.c_size_t, []),
